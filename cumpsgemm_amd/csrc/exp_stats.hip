@@ -1,0 +1,406 @@
+// Exponent statistics: per-matrix max exponent, element count above the
+// "ignore" threshold and count of elements that would underflow the fp16 lo
+// term.  HBM-bound streaming reductions for gfx950: 16-byte loads, wave64
+// butterfly reduction, one partial record per workgroup, and the last
+// workgroup to arrive folds the partials and takes the mode decision, so a
+// statistics pass is a single launch with no zero-initialisation step.
+//
+// Results are integer counts and a bit-masked maximum, hence independent of the
+// reduction order and bit-exact with the reference algorithm
+// (src/exp_stats.cu:32-62 counting, :74-184 stage 1 + decision 1, :187-293
+// stage 2 + decision 2, :386-459 max only, :295-379 launch arguments).
+#include "handle.hpp"
+#include "utils.hpp"
+#include <cumpsgemm/cumpsgemm.hpp>
+#include <cumpsgemm/cumpsgemm_ext.h>
+#include <type_traits>
+
+namespace cumpsgemm_amd {
+namespace {
+
+constexpr int kBlock = 256;
+
+struct Acc {
+  float mx;
+  unsigned total;
+  unsigned under;
+};
+
+__device__ inline void count_one(Acc &a, float x, float ignore_thr, float under_thr) {
+  const float ax = fabsf(x);
+  a.mx = fmaxf(a.mx, ax); // NaN operands are ignored
+  if (ax >= ignore_thr) {
+    a.total++;
+    if (ax < under_thr) a.under++;
+  }
+}
+
+// MODE 0: stage 1 (max + counts, absolute thresholds)
+// MODE 1: stage 2 (counts only, thresholds relative to the slot's max exponent;
+//                  runs only if the slot is UNDEFINED)
+// MODE 2: max exponent only
+template <int MODE>
+__global__ __launch_bounds__(kBlock) void exp_stats_kernel(
+    StatsSlot *slot, StatsPartial *partials, unsigned *ticket, const float *ptr,
+    unsigned long long count_f, // flat path: number of floats; 0 = strided path
+    unsigned m_f, unsigned n, unsigned long long ld_f, unsigned nbatch,
+    unsigned long long stride_f, float ignore_thr, float under_thr, float tolerance) {
+  if (MODE == 1) {
+    if (slot->mode != CUMPSGEMM_UNDEFINED) return; // uniform across the grid
+    const float max_exp = __uint_as_float(slot->max_exp_bits);
+    ignore_thr *= max_exp;
+    under_thr *= max_exp;
+  }
+  Acc acc{0.0f, 0u, 0u};
+  const unsigned tid = threadIdx.x;
+  if (count_f != 0) {
+    // contiguous data: head up to 16-byte alignment, float4 body, tail
+    const unsigned long long mis = ((16 - ((uintptr_t)ptr & 15)) & 15) / 4;
+    const unsigned long long head = mis < count_f ? mis : count_f;
+    const float4 *body = reinterpret_cast<const float4 *>(ptr + head);
+    const unsigned long long nvec = (count_f - head) / 4;
+    const unsigned long long gsz = (unsigned long long)gridDim.x * kBlock;
+    unsigned long long i = (unsigned long long)blockIdx.x * kBlock + tid;
+    for (; i + 3 * gsz < nvec; i += 4 * gsz) {
+      const float4 v0 = body[i], v1 = body[i + gsz], v2 = body[i + 2 * gsz], v3 = body[i + 3 * gsz];
+      count_one(acc, v0.x, ignore_thr, under_thr); count_one(acc, v0.y, ignore_thr, under_thr);
+      count_one(acc, v0.z, ignore_thr, under_thr); count_one(acc, v0.w, ignore_thr, under_thr);
+      count_one(acc, v1.x, ignore_thr, under_thr); count_one(acc, v1.y, ignore_thr, under_thr);
+      count_one(acc, v1.z, ignore_thr, under_thr); count_one(acc, v1.w, ignore_thr, under_thr);
+      count_one(acc, v2.x, ignore_thr, under_thr); count_one(acc, v2.y, ignore_thr, under_thr);
+      count_one(acc, v2.z, ignore_thr, under_thr); count_one(acc, v2.w, ignore_thr, under_thr);
+      count_one(acc, v3.x, ignore_thr, under_thr); count_one(acc, v3.y, ignore_thr, under_thr);
+      count_one(acc, v3.z, ignore_thr, under_thr); count_one(acc, v3.w, ignore_thr, under_thr);
+    }
+    for (; i < nvec; i += gsz) {
+      const float4 v = body[i];
+      count_one(acc, v.x, ignore_thr, under_thr); count_one(acc, v.y, ignore_thr, under_thr);
+      count_one(acc, v.z, ignore_thr, under_thr); count_one(acc, v.w, ignore_thr, under_thr);
+    }
+    if (blockIdx.x == 0) {
+      if (tid < head) count_one(acc, ptr[tid], ignore_thr, under_thr);
+      const unsigned long long tail0 = head + nvec * 4;
+      if (tail0 + tid < count_f) count_one(acc, ptr[tail0 + tid], ignore_thr, under_thr);
+    }
+  } else {
+    // strided view: one column (of m_f floats) per workgroup iteration
+    const unsigned long long ncols = (unsigned long long)n * nbatch;
+    for (unsigned long long col = blockIdx.x; col < ncols; col += gridDim.x) {
+      const float *cp = ptr + (col / n) * stride_f + (col % n) * ld_f;
+      for (unsigned i = tid; i < m_f; i += kBlock) count_one(acc, cp[i], ignore_thr, under_thr);
+    }
+  }
+
+  // wave64 butterfly
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) {
+    acc.mx = fmaxf(acc.mx, __shfl_xor(acc.mx, off, 64));
+    acc.total += __shfl_xor(acc.total, off, 64);
+    acc.under += __shfl_xor(acc.under, off, 64);
+  }
+  __shared__ float s_mx[kBlock / 64];
+  __shared__ unsigned s_total[kBlock / 64], s_under[kBlock / 64];
+  __shared__ bool s_last;
+  if ((tid & 63) == 0) {
+    s_mx[tid >> 6] = acc.mx;
+    s_total[tid >> 6] = acc.total;
+    s_under[tid >> 6] = acc.under;
+  }
+  __syncthreads();
+  if (tid == 0) {
+    float mx = 0.0f;
+    unsigned long long t = 0, u = 0;
+    for (int w = 0; w < kBlock / 64; w++) {
+      mx = fmaxf(mx, s_mx[w]);
+      t += s_total[w];
+      u += s_under[w];
+    }
+    StatsPartial p;
+    p.max_bits = __float_as_uint(mx) & 0x7f800000u;
+    p.pad = 0;
+    p.total = t;
+    p.underflow = u;
+    partials[blockIdx.x] = p;
+    __threadfence();
+    const unsigned arrived = atomicAdd(ticket, 1u);
+    s_last = (arrived == gridDim.x - 1);
+  }
+  __syncthreads();
+  if (!s_last) return;
+
+  // last workgroup: fold all partials
+  __threadfence();
+  unsigned mxb = 0;
+  unsigned long long t = 0, u = 0;
+  for (unsigned i = tid; i < gridDim.x; i += kBlock) {
+    const volatile StatsPartial *p = partials + i;
+    const unsigned b = p->max_bits;
+    mxb = b > mxb ? b : mxb;
+    t += p->total;
+    u += p->underflow;
+  }
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) {
+    const unsigned ob = __shfl_xor(mxb, off, 64);
+    mxb = ob > mxb ? ob : mxb;
+    t += __shfl_xor(t, off, 64);
+    u += __shfl_xor(u, off, 64);
+  }
+  __shared__ unsigned r_mx[kBlock / 64];
+  __shared__ unsigned long long r_t[kBlock / 64], r_u[kBlock / 64];
+  if ((tid & 63) == 0) {
+    r_mx[tid >> 6] = mxb;
+    r_t[tid >> 6] = t;
+    r_u[tid >> 6] = u;
+  }
+  __syncthreads();
+  if (tid == 0) {
+    mxb = 0; t = 0; u = 0;
+    for (int w = 0; w < kBlock / 64; w++) {
+      mxb = r_mx[w] > mxb ? r_mx[w] : mxb;
+      t += r_t[w];
+      u += r_u[w];
+    }
+    if (MODE == 0) {
+      slot->max_exp_bits = mxb;
+      const float max_exp = __uint_as_float(mxb);
+      // decision 1: counters compared as floats, like the reference's mixed
+      // u64 * float expression
+      if (((float)u > (float)t * tolerance) || (max_exp > 0.0f && t == 0)) {
+        slot->mode = CUMPSGEMM_UNDEFINED;
+        slot->total = 0;
+        slot->underflow = 0;
+      } else {
+        slot->mode = CUMPSGEMM_FP16TCEC;
+        slot->total = t;
+        slot->underflow = u;
+      }
+    } else if (MODE == 1) {
+      slot->total = t;
+      slot->underflow = u;
+      slot->mode = ((float)u <= (float)t * tolerance) ? CUMPSGEMM_FP16TCEC_SCALING
+                                                      : CUMPSGEMM_TF32TCEC;
+    } else {
+      slot->max_exp_bits = mxb;
+    }
+    *ticket = 0; // ready for the next pass on this stream
+    __threadfence();
+  }
+}
+
+struct View {
+  unsigned long long count_f; // != 0 -> contiguous
+  unsigned m_f, n, nbatch;
+  unsigned long long ld_f, stride_f;
+  unsigned grid;
+};
+
+template <class T>
+View make_view(const cuMpSGEMM_handle *h, unsigned m, unsigned n, unsigned ld, unsigned batch,
+               unsigned stride) {
+  constexpr unsigned ES = std::is_same<T, hipComplex>::value ? 2 : 1;
+  View v{};
+  // stride == 0 -> only the first matrix is looked at (reference src/exp_stats.cu:306)
+  v.nbatch = (stride == 0) ? 1 : batch;
+  v.m_f = m * ES;
+  v.n = n;
+  v.ld_f = (unsigned long long)ld * ES;
+  v.stride_f = (unsigned long long)stride * ES;
+  const bool dense_cols = (ld == m) || n == 1;
+  const bool dense_batch = v.nbatch == 1 || (unsigned long long)stride == (unsigned long long)m * n;
+  const unsigned long long total_f = (unsigned long long)m * n * v.nbatch * ES;
+  unsigned long long blocks;
+  if (dense_cols && dense_batch) {
+    v.count_f = total_f;
+    blocks = (total_f / 4 + kBlock * 4 - 1) / (kBlock * 4);
+  } else {
+    v.count_f = 0;
+    blocks = (unsigned long long)n * v.nbatch;
+  }
+  const unsigned long long cap = std::min<unsigned long long>((unsigned long long)h->num_cus * 8, kMaxStatsBlocks);
+  v.grid = (unsigned)std::max<unsigned long long>(1, std::min(blocks, cap));
+  return v;
+}
+
+unsigned next_slot(cuMpSGEMM_handle *h) {
+  // ring of result slots: 0 and 1 are presets, 2..length-1 cycle
+  // (reference src/exp_stats.cu:15-24)
+  h->stats_current_id++;
+  if (h->stats_current_id >= h->stats_ring_length) h->stats_current_id = 2;
+  return h->stats_current_id;
+}
+
+template <class T>
+void run_exp_stats(cuMpSGEMM_handle *h, unsigned m, unsigned n, const T *ptr, unsigned ld,
+                   unsigned batch, unsigned stride, unsigned slot_id) {
+  const View v = make_view<T>(h, m, n, ld, batch, stride);
+  StatsSlot *slot = h->stats_slots + slot_id;
+  const float *p = reinterpret_cast<const float *>(ptr);
+  {
+    ProfileScope prof(h, "exp_stats_1");
+    hipLaunchKernelGGL(exp_stats_kernel<0>, dim3(v.grid), dim3(kBlock), 0, h->stream, slot,
+                       h->stats_partials, h->stats_ticket, p, v.count_f, v.m_f, v.n, v.ld_f,
+                       v.nbatch, v.stride_f, h->ignore_threshold, h->underflow_threshold,
+                       h->underflow_tolerance_rate);
+  }
+  {
+    ProfileScope prof(h, "exp_stats_2");
+    // stage-2 thresholds are half the stage-1 ones, times the max exponent
+    // (reference src/exp_stats.cu:360-361, :205-206)
+    hipLaunchKernelGGL(exp_stats_kernel<1>, dim3(v.grid), dim3(kBlock), 0, h->stream, slot,
+                       h->stats_partials, h->stats_ticket, p, v.count_f, v.m_f, v.n, v.ld_f,
+                       v.nbatch, v.stride_f, h->ignore_threshold / 2, h->underflow_threshold / 2,
+                       h->underflow_tolerance_rate);
+  }
+}
+
+template <class T>
+void run_exp_max(cuMpSGEMM_handle *h, unsigned m, unsigned n, const T *ptr, unsigned ld,
+                 unsigned batch, unsigned stride, unsigned slot_id) {
+  const View v = make_view<T>(h, m, n, ld, batch, stride);
+  ProfileScope prof(h, "exp_max");
+  hipLaunchKernelGGL(exp_stats_kernel<2>, dim3(v.grid), dim3(kBlock), 0, h->stream,
+                     h->stats_slots + slot_id, h->stats_partials, h->stats_ticket,
+                     reinterpret_cast<const float *>(ptr), v.count_f, v.m_f, v.n, v.ld_f,
+                     v.nbatch, v.stride_f, 0.0f, 0.0f, 0.0f);
+}
+
+void read_slot(cuMpSGEMM_handle *h, unsigned id, StatsSlot &out) {
+  check_hip(hipMemcpyAsync(&out, h->stats_slots + id, sizeof(StatsSlot), hipMemcpyDeviceToHost,
+                           h->stream),
+            "read stats slot");
+  check_hip(hipStreamSynchronize(h->stream), "sync after stats read");
+}
+} // namespace
+} // namespace cumpsgemm_amd
+
+using namespace cumpsgemm_amd;
+
+template <class T>
+unsigned cumpsgemm::exp_stats_ext(handle_t handle, unsigned m, unsigned n, const T *ptr,
+                                  unsigned ld, unsigned batch_size, unsigned stride) {
+  const unsigned id = next_slot(handle);
+  run_exp_stats<T>(handle, m, n, ptr, ld, batch_size, stride, id);
+  return id;
+}
+template <class T>
+unsigned cumpsgemm::exp_max_ext(handle_t handle, unsigned m, unsigned n, const T *ptr,
+                                unsigned ld, unsigned batch_size, unsigned stride) {
+  const unsigned id = next_slot(handle);
+  run_exp_max<T>(handle, m, n, ptr, ld, batch_size, stride, id);
+  return id;
+}
+template unsigned cumpsgemm::exp_stats_ext<float>(handle_t, unsigned, unsigned, const float *,
+                                                  unsigned, unsigned, unsigned);
+template unsigned cumpsgemm::exp_stats_ext<hipComplex>(handle_t, unsigned, unsigned,
+                                                       const hipComplex *, unsigned, unsigned,
+                                                       unsigned);
+template unsigned cumpsgemm::exp_max_ext<float>(handle_t, unsigned, unsigned, const float *,
+                                                unsigned, unsigned, unsigned);
+template unsigned cumpsgemm::exp_max_ext<hipComplex>(handle_t, unsigned, unsigned,
+                                                     const hipComplex *, unsigned, unsigned,
+                                                     unsigned);
+
+std::pair<std::size_t, std::size_t> cumpsgemm::get_exp_stats(handle_t handle, unsigned buffer_id) {
+  StatsSlot s;
+  read_slot(handle, buffer_id, s);
+  return {(std::size_t)s.underflow, (std::size_t)s.total}; // reference src/exp_stats.cu:628
+}
+unsigned cumpsgemm::get_current_exp_stats_buffer_id(handle_t handle) {
+  return handle->stats_current_id;
+}
+void cumpsgemm::reset_exp_stats_buffer_id(handle_t handle) { handle->stats_current_id = 1; }
+void cumpsgemm::set_exp_stats_params(handle_t handle, float ignore_threshold,
+                                     float underflow_threshold, float underflow_ratio_tolerance) {
+  handle->ignore_threshold = ignore_threshold;
+  handle->underflow_threshold = underflow_threshold;
+  handle->underflow_tolerance_rate = underflow_ratio_tolerance;
+}
+void cumpsgemm::enable_exp_stats(handle_t handle) { handle->exp_stats_enabled = true; }
+void cumpsgemm::disable_exp_stats(handle_t handle) { handle->exp_stats_enabled = false; }
+float cumpsgemm::get_max_exp(handle_t handle, unsigned buffer_id) {
+  StatsSlot s;
+  read_slot(handle, buffer_id, s);
+  float f;
+  static_assert(sizeof(f) == sizeof(s.max_exp_bits), "");
+  std::memcpy(&f, &s.max_exp_bits, sizeof(f));
+  return f;
+}
+cuMpSGEMM_compute_mode_t cumpsgemm::get_exp_stats_compute_mode_level(handle_t handle,
+                                                                     unsigned buffer_id) {
+  StatsSlot s;
+  read_slot(handle, buffer_id, s);
+  return (cuMpSGEMM_compute_mode_t)s.mode;
+}
+
+void cumpsgemm::enable_exp_stats_profiling(handle_t handle) { handle->profiler.enabled = true; }
+void cumpsgemm::disable_exp_stats_profiling(handle_t handle) { handle->profiler.enabled = false; }
+void cumpsgemm::reset_exp_stats_profiling(handle_t handle) { handle->profiler.entries.clear(); }
+void cumpsgemm::print_exp_stats_profiling(handle_t handle, unsigned csv) {
+  double total = 0.0;
+  for (const auto &e : handle->profiler.entries) total += e.second.sum;
+  if (csv) {
+    std::printf("name,sum_s,n,avg_s,ratio\n");
+    for (const auto &e : handle->profiler.entries)
+      std::printf("%s,%e,%llu,%e,%e\n", e.first.c_str(), e.second.sum,
+                  (unsigned long long)e.second.n, e.second.sum / e.second.n,
+                  total > 0 ? e.second.sum / total : 0.0);
+  } else {
+    for (const auto &e : handle->profiler.entries)
+      std::printf("%20s : %e [s] (%6.2f%%), n = %llu, avg = %e [s]\n", e.first.c_str(),
+                  e.second.sum, total > 0 ? 100.0 * e.second.sum / total : 0.0,
+                  (unsigned long long)e.second.n, e.second.sum / e.second.n);
+  }
+  std::fflush(stdout);
+}
+std::unordered_map<std::string, cumpsgemm::debug::stats_t>
+cumpsgemm::debug::get_exp_stats_profiling_result(handle_t handle) {
+  std::unordered_map<std::string, stats_t> r;
+  for (const auto &e : handle->profiler.entries) r[e.first] = stats_t{e.second.sum, e.second.n};
+  return r;
+}
+
+extern "C" {
+unsigned cuMpSGEMM_exp_stats_ext_s(cuMpSGEMM_handle_t h, unsigned m, unsigned n, const float *ptr,
+                                   unsigned ld, unsigned batch, unsigned stride) {
+  return cumpsgemm::exp_stats_ext<float>(h, m, n, ptr, ld, batch, stride);
+}
+unsigned cuMpSGEMM_exp_stats_ext_c(cuMpSGEMM_handle_t h, unsigned m, unsigned n,
+                                   const hipComplex *ptr, unsigned ld, unsigned batch,
+                                   unsigned stride) {
+  return cumpsgemm::exp_stats_ext<hipComplex>(h, m, n, ptr, ld, batch, stride);
+}
+unsigned cuMpSGEMM_exp_max_ext_s(cuMpSGEMM_handle_t h, unsigned m, unsigned n, const float *ptr,
+                                 unsigned ld, unsigned batch, unsigned stride) {
+  return cumpsgemm::exp_max_ext<float>(h, m, n, ptr, ld, batch, stride);
+}
+unsigned cuMpSGEMM_exp_max_ext_c(cuMpSGEMM_handle_t h, unsigned m, unsigned n,
+                                 const hipComplex *ptr, unsigned ld, unsigned batch,
+                                 unsigned stride) {
+  return cumpsgemm::exp_max_ext<hipComplex>(h, m, n, ptr, ld, batch, stride);
+}
+void cuMpSGEMM_get_exp_stats(cuMpSGEMM_handle_t h, unsigned id, uint64_t *underflow,
+                             uint64_t *total) {
+  const auto r = cumpsgemm::get_exp_stats(h, id);
+  *underflow = r.first;
+  *total = r.second;
+}
+float cuMpSGEMM_get_max_exp(cuMpSGEMM_handle_t h, unsigned id) {
+  return cumpsgemm::get_max_exp(h, id);
+}
+int cuMpSGEMM_get_exp_stats_compute_mode_level(cuMpSGEMM_handle_t h, unsigned id) {
+  return (int)cumpsgemm::get_exp_stats_compute_mode_level(h, id);
+}
+void cuMpSGEMM_set_exp_stats_params(cuMpSGEMM_handle_t h, float ignore_threshold,
+                                    float underflow_threshold, float tolerance) {
+  cumpsgemm::set_exp_stats_params(h, ignore_threshold, underflow_threshold, tolerance);
+}
+unsigned cuMpSGEMM_get_current_exp_stats_buffer_id(cuMpSGEMM_handle_t h) {
+  return cumpsgemm::get_current_exp_stats_buffer_id(h);
+}
+void cuMpSGEMM_reset_exp_stats_buffer_id(cuMpSGEMM_handle_t h) {
+  cumpsgemm::reset_exp_stats_buffer_id(h);
+}
+void cuMpSGEMM_enable_exp_stats(cuMpSGEMM_handle_t h) { cumpsgemm::enable_exp_stats(h); }
+void cuMpSGEMM_disable_exp_stats(cuMpSGEMM_handle_t h) { cumpsgemm::disable_exp_stats(h); }
+} // extern "C"

@@ -1,0 +1,457 @@
+// Host side of the GEMM path: handle life cycle, tile selection, launches and
+// the C ABI.  Takes the place of reference src/handle.cu:7-52 and
+// src/cumpsgemm.cu:19-605.
+#include "gemm_table.hpp"
+#include "handle.hpp"
+#include "utils.hpp"
+#include <cumpsgemm/cumpsgemm.hpp>
+#include <cumpsgemm/cumpsgemm_ext.h>
+#include <new>
+#include <stdexcept>
+#include <type_traits>
+
+namespace cumpsgemm_amd {
+
+void check_hip(hipError_t err, const char *what) {
+  if (err != hipSuccess) {
+    const std::string msg = std::string(what) + ": " + hipGetErrorString(err);
+    log_error(msg);
+    throw std::runtime_error(msg);
+  }
+}
+
+ProfileScope::ProfileScope(cuMpSGEMM_handle *handle, const char *label)
+    : h(handle), name(label) {
+  if (h->profiler.enabled) {
+    (void)hipStreamSynchronize(h->stream);
+    h->profiler.t0 = std::chrono::steady_clock::now();
+  }
+}
+ProfileScope::~ProfileScope() {
+  if (h->profiler.enabled) {
+    (void)hipStreamSynchronize(h->stream);
+    const auto t1 = std::chrono::steady_clock::now();
+    auto &e = h->profiler.entries[name];
+    e.sum += std::chrono::duration<double>(t1 - h->profiler.t0).count();
+    e.n++;
+  }
+}
+
+const KernelEntry *lookup_kernel(Prec p, bool cplx, bool a_kc, bool b_kc, int cls) {
+  const int layout = (a_kc ? 1 : 0) + (b_kc ? 2 : 0);
+  switch (p) {
+  case Prec::FP16TCEC:
+    return cplx ? &g_tab_fp16tcec_c[layout][cls] : &g_tab_fp16tcec_s[layout][cls];
+  case Prec::FP16TC:
+    return cplx ? &g_tab_fp16tc_c[layout][cls] : &g_tab_fp16tc_s[layout][cls];
+  case Prec::BF16X3:
+    return cplx ? &g_tab_bf16x3_c[layout][cls] : &g_tab_bf16x3_s[layout][cls];
+  case Prec::BF16X2:
+    return cplx ? &g_tab_bf16x2_c[layout][cls] : &g_tab_bf16x2_s[layout][cls];
+  }
+  return nullptr;
+}
+
+namespace {
+__global__ void init_rings_kernel(StatsSlot *slots, int *flags, unsigned *ticket) {
+  // presets of the reference: stats slot 0 -> TF32TCEC, slot 1 -> FP16TCEC
+  // (src/exp_stats.cu:496-499); flag slot 0 -> TF32TCEC, slot 1 -> FP16TCEC with
+  // both scale bits (src/dynamic_launch.cu:6-9)
+  if (threadIdx.x == 0 && blockIdx.x == 0) {
+    slots[0].mode = CUMPSGEMM_TF32TCEC;
+    slots[1].mode = CUMPSGEMM_FP16TCEC;
+    flags[0] = CUMPSGEMM_TF32TCEC;
+    flags[1] = (3 << 5) | CUMPSGEMM_FP16TCEC;
+    *ticket = 0;
+  }
+}
+
+bool mode_to_prec(cuMpSGEMM_compute_mode_t mode, Prec &p) {
+  switch (mode) {
+  case CUMPSGEMM_FP16TCEC:
+  case CUMPSGEMM_FP16TCEC_SCALING: // scaling is orchestrated outside the kernel
+    p = Prec::FP16TCEC;
+    return true;
+  case CUMPSGEMM_FP16TC:
+    p = Prec::FP16TC;
+    return true;
+  case CUMPSGEMM_TF32TCEC:
+    p = Prec::BF16X3;
+    return true;
+  case CUMPSGEMM_TF32TC:
+    p = Prec::BF16X2;
+    return true;
+  default:
+    return false;
+  }
+}
+
+struct Plan {
+  const KernelEntry *entry;
+  int cls;
+  unsigned tiles_m, tiles_n, ksplit, k_chunk;
+};
+
+// Shape -> tile class and split-K factor.  The reference fills "two waves of
+// SMs" (src/cumpsgemm.cu:252-253, x32 for batches :453-454); here a class is
+// accepted when its tiles give every CU at least one resident workgroup set
+// (occ * 4 / waves-per-group groups per CU), else the next smaller tile is
+// tried; if even the smallest tile leaves CUs idle and K is long, K is split.
+Plan make_plan(const cuMpSGEMM_handle *h, Prec p, bool cplx, bool a_kc, bool b_kc,
+               uint64_t m, uint64_t n, uint64_t k, uint64_t batch, int force_cls) {
+  Plan plan{};
+  int cls = 0;
+  if (force_cls >= 0) {
+    cls = force_cls;
+  } else {
+    for (cls = 0; cls < kNumTileClasses - 1; cls++) {
+      const KernelEntry *e = lookup_kernel(p, cplx, a_kc, b_kc, cls);
+      const uint64_t tiles = ((m + e->bm - 1) / e->bm) * ((n + e->bn - 1) / e->bn) * batch;
+      // skip a class whose tile is mostly padding for this shape
+      const bool wasteful = (m * 2 <= (uint64_t)e->bm) || (n * 2 <= (uint64_t)e->bn);
+      if (!wasteful && tiles >= (uint64_t)h->num_cus * 2) break;
+    }
+  }
+  const KernelEntry *e = lookup_kernel(p, cplx, a_kc, b_kc, cls);
+  plan.entry = e;
+  plan.cls = cls;
+  plan.tiles_m = (unsigned)((m + e->bm - 1) / e->bm);
+  plan.tiles_n = (unsigned)((n + e->bn - 1) / e->bn);
+  const uint64_t tiles = (uint64_t)plan.tiles_m * plan.tiles_n * batch;
+  unsigned ksplit = 1;
+  if (tiles < h->num_cus && k >= 256) {
+    const uint64_t want = ((uint64_t)h->num_cus * 2 + tiles - 1) / tiles;
+    const uint64_t max_by_k = k / 128; // keep at least 4 K-steps per workgroup
+    ksplit = (unsigned)(want < max_by_k ? want : max_by_k);
+    if (ksplit < 1) ksplit = 1;
+    if (ksplit > 64) ksplit = 64;
+  }
+  unsigned k_chunk = (unsigned)((k + ksplit - 1) / ksplit);
+  k_chunk = (k_chunk + 31) / 32 * 32;
+  ksplit = (unsigned)((k + k_chunk - 1) / k_chunk);
+  plan.ksplit = ksplit;
+  plan.k_chunk = k_chunk;
+  return plan;
+}
+
+template <class T> struct scalar_parts;
+template <> struct scalar_parts<float> {
+  static void get(const float *s, float &re, float &im) { re = *s; im = 0.0f; }
+};
+template <> struct scalar_parts<hipComplex> {
+  static void get(const hipComplex *s, float &re, float &im) { re = s->x; im = s->y; }
+};
+
+template <class T>
+hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
+                         hipblasOperation_t op_B, uint64_t m, uint64_t n, uint64_t k,
+                         const T *alpha, const T *a, uint64_t lda, uint64_t stridea,
+                         const T *b, uint64_t ldb, uint64_t strideb, const T *beta, T *c,
+                         uint64_t ldc, uint64_t stridec, uint64_t batch,
+                         cuMpSGEMM_compute_mode_t mode, unsigned *used_id,
+                         const char *label) {
+  constexpr bool CPLX = std::is_same<T, hipComplex>::value;
+  if (h == nullptr || alpha == nullptr || beta == nullptr) return HIPBLAS_STATUS_INVALID_VALUE;
+  if (m == 0 || n == 0 || batch == 0) return HIPBLAS_STATUS_SUCCESS;
+  if (m > 0x7fffffffull || n > 0x7fffffffull || k > 0x7fffffffull || batch > 65535ull)
+    return HIPBLAS_STATUS_INVALID_VALUE;
+  const bool a_kc = (op_A != HIPBLAS_OP_N);
+  const bool b_kc = (op_B == HIPBLAS_OP_N);
+  if (lda < (a_kc ? k : m) || ldb < (b_kc ? k : n) || ldc < m) {
+    if (k != 0) return HIPBLAS_STATUS_INVALID_VALUE;
+  }
+
+  GemmArgs args{};
+  args.m = (uint32_t)m;
+  args.n = (uint32_t)n;
+  args.k = (uint32_t)k;
+  args.a = a;
+  args.b = b;
+  args.c = c;
+  args.lda = lda;
+  args.ldb = ldb;
+  args.ldc = ldc;
+  args.stride_a = stridea;
+  args.stride_b = strideb;
+  args.stride_c = stridec;
+  scalar_parts<T>::get(alpha, args.alpha_re, args.alpha_im);
+  scalar_parts<T>::get(beta, args.beta_re, args.beta_im);
+  args.conj_a = (CPLX && op_A == HIPBLAS_OP_C) ? 1u : 0u;
+  args.conj_b = (CPLX && op_B == HIPBLAS_OP_C) ? 1u : 0u;
+
+  // which kernels to launch: one for a fixed mode; for AUTO both candidates,
+  // each gated on the device flag so that no host synchronisation is needed
+  // (reference src/cumpsgemm.cu:305-368, src/cumpsgemm_kernel.cuh:478-489)
+  struct Launch {
+    Prec p;
+    uint32_t accept;
+  } launches[2];
+  int nlaunch = 0;
+  if (mode == CUMPSGEMM_AUTO) {
+    launches[nlaunch++] = {Prec::BF16X3, 1u << CUMPSGEMM_TF32TCEC};
+    launches[nlaunch++] = {Prec::FP16TCEC,
+                           (1u << CUMPSGEMM_FP16TCEC) | (1u << CUMPSGEMM_FP16TCEC_SCALING)};
+    args.launch_flag = h->flag_buffer + h->flag_enabled_id;
+  } else {
+    Prec p;
+    if (!mode_to_prec(mode, p)) return HIPBLAS_STATUS_INVALID_VALUE;
+    launches[nlaunch++] = {p, 0u};
+    args.launch_flag = nullptr;
+  }
+
+  int force_cls = -1;
+  if (const char *f = std::getenv("CUMPSGEMM_FORCE_TILE_CLASS")) {
+    force_cls = std::atoi(f);
+    if (force_cls < 0 || force_cls >= kNumTileClasses) force_cls = -1;
+  }
+
+  ProfileScope prof(h, label);
+  const bool beta_zero = args.beta_re == 0.0f && args.beta_im == 0.0f;
+
+  if (k == 0) { // C = beta * C
+    const unsigned blocks = (unsigned)std::min<uint64_t>((m * n + 255) / 256, 65535);
+    hipLaunchKernelGGL(prescale_c_kernel<CPLX>, dim3(blocks, (unsigned)batch), dim3(256), 0,
+                       h->stream, reinterpret_cast<float *>(c), args.m, args.n, ldc, stridec,
+                       args.beta_re, args.beta_im);
+    return HIPBLAS_STATUS_SUCCESS;
+  }
+
+  // AUTO launches two gated kernels that must agree on how C is prepared, so
+  // the split-K decision is taken once, from the first candidate.
+  Plan plan0 = make_plan(h, launches[0].p, CPLX, a_kc, b_kc, m, n, k, batch, force_cls);
+  const bool split = plan0.ksplit > 1;
+  if (split) {
+    const unsigned blocks = (unsigned)std::min<uint64_t>((m * n + 255) / 256, 65535);
+    hipLaunchKernelGGL(prescale_c_kernel<CPLX>, dim3(blocks, (unsigned)batch), dim3(256), 0,
+                       h->stream, reinterpret_cast<float *>(c), args.m, args.n, ldc, stridec,
+                       args.beta_re, args.beta_im);
+  }
+  (void)beta_zero;
+
+  for (int i = 0; i < nlaunch; i++) {
+    Plan plan = (i == 0) ? plan0
+                         : make_plan(h, launches[i].p, CPLX, a_kc, b_kc, m, n, k, batch, force_cls);
+    if (split) { // same K partition for every candidate
+      plan.ksplit = plan0.ksplit;
+      plan.k_chunk = plan0.k_chunk;
+    } else {
+      plan.ksplit = 1;
+      plan.k_chunk = (unsigned)k;
+    }
+    args.tiles_m = plan.tiles_m;
+    args.tiles_n = plan.tiles_n;
+    args.k_chunk = plan.k_chunk;
+    args.atomic_out = split ? 1u : 0u;
+    args.flag_accept_mask = launches[i].accept;
+    const dim3 grid(plan.tiles_m * plan.tiles_n, (unsigned)batch, plan.ksplit);
+    plan.entry->launch(args, grid, h->stream);
+    if (used_id != nullptr) {
+      *used_id = (mode == CUMPSGEMM_AUTO) ? ~0u : (unsigned)plan.cls + (split ? 100u : 0u);
+    }
+  }
+  const hipError_t err = hipGetLastError();
+  if (err != hipSuccess) {
+    log_error(std::string("GEMM launch failed: ") + hipGetErrorString(err));
+    return HIPBLAS_STATUS_EXECUTION_FAILED;
+  }
+  return HIPBLAS_STATUS_SUCCESS;
+}
+} // namespace
+} // namespace cumpsgemm_amd
+
+using namespace cumpsgemm_amd;
+
+template <class T>
+hipblasStatus_t cumpsgemm::gemm(cuMpSGEMM_handle_t handle, hipblasOperation_t op_A,
+                                hipblasOperation_t op_B, uint64_t m, uint64_t n, uint64_t k,
+                                const T *alpha, const T *a_dmem_ptr, uint64_t lda,
+                                const T *b_dmem_ptr, uint64_t ldb, const T *beta,
+                                T *c_dmem_ptr, uint64_t ldc,
+                                cuMpSGEMM_compute_mode_t compute_mode,
+                                unsigned *used_kernel_module_id) {
+  return run_gemm<T>(handle, op_A, op_B, m, n, k, alpha, a_dmem_ptr, lda, 0, b_dmem_ptr, ldb, 0,
+                     beta, c_dmem_ptr, ldc, 0, 1, compute_mode, used_kernel_module_id,
+                     "gemm_kernel");
+}
+
+template <class T>
+hipblasStatus_t cumpsgemm::gemm_stridedBatch(
+    cuMpSGEMM_handle_t handle, hipblasOperation_t op_A, hipblasOperation_t op_B, uint64_t m,
+    uint64_t n, uint64_t k, const T *alpha, const T *a_dmem_ptr, uint64_t lda, uint64_t stridea,
+    const T *b_dmem_ptr, uint64_t ldb, uint64_t strideb, const T *beta, T *c_dmem_ptr,
+    uint64_t ldc, uint64_t stridec, uint64_t batch_count, cuMpSGEMM_compute_mode_t compute_mode,
+    unsigned *used_kernel_module_id) {
+  // batches beyond the grid's y limit are issued in slices
+  uint64_t done = 0;
+  hipblasStatus_t st = HIPBLAS_STATUS_SUCCESS;
+  while (done < batch_count && st == HIPBLAS_STATUS_SUCCESS) {
+    const uint64_t nb = std::min<uint64_t>(batch_count - done, 65535);
+    st = run_gemm<T>(handle, op_A, op_B, m, n, k, alpha, a_dmem_ptr + done * stridea, lda,
+                     stridea, b_dmem_ptr + done * strideb, ldb, strideb, beta,
+                     c_dmem_ptr + done * stridec, ldc, stridec, nb, compute_mode,
+                     used_kernel_module_id, "batched_gemm_kernel");
+    done += nb;
+  }
+  return st;
+}
+
+template hipblasStatus_t cumpsgemm::gemm<float>(cuMpSGEMM_handle_t, hipblasOperation_t,
+                                                hipblasOperation_t, uint64_t, uint64_t, uint64_t,
+                                                const float *, const float *, uint64_t,
+                                                const float *, uint64_t, const float *, float *,
+                                                uint64_t, cuMpSGEMM_compute_mode_t, unsigned *);
+template hipblasStatus_t cumpsgemm::gemm<hipComplex>(
+    cuMpSGEMM_handle_t, hipblasOperation_t, hipblasOperation_t, uint64_t, uint64_t, uint64_t,
+    const hipComplex *, const hipComplex *, uint64_t, const hipComplex *, uint64_t,
+    const hipComplex *, hipComplex *, uint64_t, cuMpSGEMM_compute_mode_t, unsigned *);
+template hipblasStatus_t cumpsgemm::gemm_stridedBatch<float>(
+    cuMpSGEMM_handle_t, hipblasOperation_t, hipblasOperation_t, uint64_t, uint64_t, uint64_t,
+    const float *, const float *, uint64_t, uint64_t, const float *, uint64_t, uint64_t,
+    const float *, float *, uint64_t, uint64_t, uint64_t, cuMpSGEMM_compute_mode_t, unsigned *);
+template hipblasStatus_t cumpsgemm::gemm_stridedBatch<hipComplex>(
+    cuMpSGEMM_handle_t, hipblasOperation_t, hipblasOperation_t, uint64_t, uint64_t, uint64_t,
+    const hipComplex *, const hipComplex *, uint64_t, uint64_t, const hipComplex *, uint64_t,
+    uint64_t, const hipComplex *, hipComplex *, uint64_t, uint64_t, uint64_t,
+    cuMpSGEMM_compute_mode_t, unsigned *);
+
+extern "C" {
+
+hipblasStatus_t cuMpSGEMM_create(cuMpSGEMM_handle_t *handle) {
+  if (handle == nullptr) return HIPBLAS_STATUS_INVALID_VALUE;
+  cuMpSGEMM_handle *h = new (std::nothrow) cuMpSGEMM_handle;
+  if (h == nullptr) return HIPBLAS_STATUS_ALLOC_FAILED;
+  *handle = nullptr;
+  int dev = 0, cus = 0;
+  if (hipGetDevice(&dev) != hipSuccess ||
+      hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) {
+    delete h;
+    return HIPBLAS_STATUS_NOT_INITIALIZED;
+  }
+  h->device = dev;
+  h->num_cus = (unsigned)cus;
+  bool ok = true;
+  ok = ok && hipMalloc(&h->stats_slots, sizeof(StatsSlot) * h->stats_ring_length) == hipSuccess;
+  ok = ok && hipMalloc(&h->stats_partials, sizeof(StatsPartial) * kMaxStatsBlocks) == hipSuccess;
+  ok = ok && hipMalloc(&h->stats_ticket, sizeof(unsigned)) == hipSuccess;
+  ok = ok && hipMalloc(&h->flag_buffer, sizeof(int) * h->flag_ring_length) == hipSuccess;
+  ok = ok && hipHostMalloc(&h->host_scratch, sizeof(unsigned long long) * 4, hipHostMallocDefault) ==
+                 hipSuccess;
+  if (!ok) {
+    cuMpSGEMM_destroy(h);
+    return HIPBLAS_STATUS_ALLOC_FAILED;
+  }
+  ok = ok && hipMemsetAsync(h->stats_slots, 0, sizeof(StatsSlot) * h->stats_ring_length, nullptr) == hipSuccess;
+  ok = ok && hipMemsetAsync(h->flag_buffer, 0, sizeof(int) * h->flag_ring_length, nullptr) == hipSuccess;
+  hipLaunchKernelGGL(init_rings_kernel, dim3(1), dim3(1), 0, nullptr, h->stats_slots,
+                     h->flag_buffer, h->stats_ticket);
+  ok = ok && hipStreamSynchronize(nullptr) == hipSuccess;
+  if (!ok) {
+    cuMpSGEMM_destroy(h);
+    return HIPBLAS_STATUS_INTERNAL_ERROR;
+  }
+  *handle = h;
+  return HIPBLAS_STATUS_SUCCESS;
+}
+
+hipblasStatus_t cuMpSGEMM_destroy(cuMpSGEMM_handle_t handle) {
+  if (handle == nullptr) return HIPBLAS_STATUS_SUCCESS;
+  (void)hipFree(handle->stats_slots);
+  (void)hipFree(handle->stats_partials);
+  (void)hipFree(handle->stats_ticket);
+  (void)hipFree(handle->flag_buffer);
+  if (handle->host_scratch) (void)hipHostFree(handle->host_scratch);
+  delete handle;
+  return HIPBLAS_STATUS_SUCCESS;
+}
+
+hipblasStatus_t cuMpSGEMM_set_stream(cuMpSGEMM_handle_t handle, hipStream_t stream) {
+  if (handle == nullptr) return HIPBLAS_STATUS_INVALID_VALUE;
+  handle->stream = stream;
+  return HIPBLAS_STATUS_SUCCESS;
+}
+
+const char *cuMpSGEMM_get_compute_mode_string(cuMpSGEMM_compute_mode_t mode) {
+  static const char *const names[] = {
+      "CUBLAS",        "FP16TCEC",      "TF32TCEC", "FP16TC", "TF32TC",    "CUBLAS_SIMT",
+      "CUBLAS_FP16TC", "CUBLAS_TF32TC", "DRY_RUN",  "AUTO",   "UNDEFINED", "FP16TCEC_SCALING",
+      "FP32_SIMT"};
+  const int i = (int)mode;
+  return (i >= 0 && i <= 12) ? names[i] : "Unknown";
+}
+
+hipblasStatus_t cuMpSGEMM_sgemm(cuMpSGEMM_handle_t handle, hipblasOperation_t op_A,
+                                hipblasOperation_t op_B, uint64_t m, uint64_t n, uint64_t k,
+                                const float *alpha, const float *a_dmem_ptr, uint64_t lda,
+                                const float *b_dmem_ptr, uint64_t ldb, const float *beta,
+                                float *c_dmem_ptr, uint64_t ldc,
+                                cuMpSGEMM_compute_mode_t compute_mode) {
+  return cumpsgemm::gemm<float>(handle, op_A, op_B, m, n, k, alpha, a_dmem_ptr, lda, b_dmem_ptr,
+                                ldb, beta, c_dmem_ptr, ldc, compute_mode);
+}
+
+hipblasStatus_t cuMpSGEMM_cgemm(cuMpSGEMM_handle_t handle, hipblasOperation_t op_A,
+                                hipblasOperation_t op_B, uint64_t m, uint64_t n, uint64_t k,
+                                const hipComplex *alpha, const hipComplex *a_dmem_ptr,
+                                uint64_t lda, const hipComplex *b_dmem_ptr, uint64_t ldb,
+                                const hipComplex *beta, hipComplex *c_dmem_ptr, uint64_t ldc,
+                                cuMpSGEMM_compute_mode_t compute_mode) {
+  return cumpsgemm::gemm<hipComplex>(handle, op_A, op_B, m, n, k, alpha, a_dmem_ptr, lda,
+                                     b_dmem_ptr, ldb, beta, c_dmem_ptr, ldc, compute_mode);
+}
+
+hipblasStatus_t cuMpSGEMM_sgemm_strided_batch(
+    cuMpSGEMM_handle_t handle, hipblasOperation_t op_A, hipblasOperation_t op_B, uint64_t m,
+    uint64_t n, uint64_t k, const float *alpha, const float *a_dmem_ptr, uint64_t lda,
+    uint64_t stridea, const float *b_dmem_ptr, uint64_t ldb, uint64_t strideb, const float *beta,
+    float *c_dmem_ptr, uint64_t ldc, uint64_t stridec, uint64_t batch_count,
+    cuMpSGEMM_compute_mode_t compute_mode) {
+  return cumpsgemm::gemm_stridedBatch<float>(handle, op_A, op_B, m, n, k, alpha, a_dmem_ptr, lda,
+                                             stridea, b_dmem_ptr, ldb, strideb, beta, c_dmem_ptr,
+                                             ldc, stridec, batch_count, compute_mode);
+}
+
+hipblasStatus_t cuMpSGEMM_cgemm_strided_batch(
+    cuMpSGEMM_handle_t handle, hipblasOperation_t op_A, hipblasOperation_t op_B, uint64_t m,
+    uint64_t n, uint64_t k, const hipComplex *alpha, const hipComplex *a_dmem_ptr, uint64_t lda,
+    uint64_t stridea, const hipComplex *b_dmem_ptr, uint64_t ldb, uint64_t strideb,
+    const hipComplex *beta, hipComplex *c_dmem_ptr, uint64_t ldc, uint64_t stridec,
+    uint64_t batch_count, cuMpSGEMM_compute_mode_t compute_mode) {
+  return cumpsgemm::gemm_stridedBatch<hipComplex>(handle, op_A, op_B, m, n, k, alpha, a_dmem_ptr,
+                                                  lda, stridea, b_dmem_ptr, ldb, strideb, beta,
+                                                  c_dmem_ptr, ldc, stridec, batch_count,
+                                                  compute_mode);
+}
+
+// ---- extension entry points (cumpsgemm_ext.h) -------------------------------
+hipblasStatus_t cuMpSGEMM_sgemm_ex(cuMpSGEMM_handle_t handle, hipblasOperation_t op_A,
+                                   hipblasOperation_t op_B, uint64_t m, uint64_t n, uint64_t k,
+                                   const float *alpha, const float *a, uint64_t lda,
+                                   const float *b, uint64_t ldb, const float *beta, float *c,
+                                   uint64_t ldc, cuMpSGEMM_compute_mode_t mode,
+                                   unsigned *used_kernel_module_id) {
+  return cumpsgemm::gemm<float>(handle, op_A, op_B, m, n, k, alpha, a, lda, b, ldb, beta, c, ldc,
+                                mode, used_kernel_module_id);
+}
+hipblasStatus_t cuMpSGEMM_cgemm_ex(cuMpSGEMM_handle_t handle, hipblasOperation_t op_A,
+                                   hipblasOperation_t op_B, uint64_t m, uint64_t n, uint64_t k,
+                                   const hipComplex *alpha, const hipComplex *a, uint64_t lda,
+                                   const hipComplex *b, uint64_t ldb, const hipComplex *beta,
+                                   hipComplex *c, uint64_t ldc, cuMpSGEMM_compute_mode_t mode,
+                                   unsigned *used_kernel_module_id) {
+  return cumpsgemm::gemm<hipComplex>(handle, op_A, op_B, m, n, k, alpha, a, lda, b, ldb, beta, c,
+                                     ldc, mode, used_kernel_module_id);
+}
+
+int cuMpSGEMM_describe_tile_config(int compute_mode, int is_complex, int op_A, int op_B,
+                                   int tile_class, char *buf, size_t buf_len) {
+  Prec p;
+  if (!mode_to_prec((cuMpSGEMM_compute_mode_t)compute_mode, p) || tile_class < 0 ||
+      tile_class >= kNumTileClasses || buf == nullptr || buf_len == 0)
+    return -1;
+  const KernelEntry *e = lookup_kernel(p, is_complex != 0, op_A != HIPBLAS_OP_N,
+                                       op_B == HIPBLAS_OP_N, tile_class);
+  std::snprintf(buf, buf_len, "%s threads=%d lds=%d occ=%d", e->name, e->threads, e->lds_bytes,
+                e->occ);
+  return 0;
+}
+} // extern "C"

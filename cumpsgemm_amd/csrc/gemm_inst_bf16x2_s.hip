@@ -1,0 +1,5 @@
+// Kernel instances of the tile table for one (precision, element type) pair.
+#include "gemm_table.hpp"
+namespace cumpsgemm_amd {
+CUMPSGEMM_DEFINE_TABLE(g_tab_bf16x2_s, CUMPSGEMM_REAL_ROW, Prec::BF16X2)
+} // namespace cumpsgemm_amd

@@ -1,0 +1,5 @@
+// Kernel instances of the tile table for one (precision, element type) pair.
+#include "gemm_table.hpp"
+namespace cumpsgemm_amd {
+CUMPSGEMM_DEFINE_TABLE(g_tab_fp16tc_c, CUMPSGEMM_CPLX_ROW, Prec::FP16TC)
+} // namespace cumpsgemm_amd

@@ -1,0 +1,76 @@
+// gfx950 tile-configuration table: for every (precision, real/complex, layout
+// of A, layout of B) a short list of kernel instances ordered from the largest
+// tile to the smallest.  The host picks by problem shape (see gemm_host.hip).
+// This table is what takes the place of the reference's per-architecture
+// instance tables and kernel_module_code keys (src/instance.hpp:33-63,
+// src/instance_sm80.cu, src/cumpsgemm.cu:19-89).
+#pragma once
+#include "gemm_kernel.hpp"
+
+namespace cumpsgemm_amd {
+
+struct KernelEntry {
+  void (*launch)(const GemmArgs &, dim3 grid, hipStream_t stream);
+  int bm, bn;      // workgroup tile
+  int wm, wn;      // wave tile
+  int threads;     // workgroup size
+  int lds_bytes;   // dynamic LDS per workgroup
+  int occ;         // waves per SIMD the kernel was compiled for
+  const char *name;
+};
+
+constexpr int kNumTileClasses = 3; // 0 = large ... 2 = small
+
+// layout index = (a_kc ? 1 : 0) + (b_kc ? 2 : 0)
+const KernelEntry *lookup_kernel(Prec p, bool cplx, bool a_kc, bool b_kc, int cls);
+
+template <class Cfg>
+void launch_cfg(const GemmArgs &args, dim3 grid, hipStream_t stream) {
+  static bool attr_done = false;
+  if (!attr_done) {
+    if (Cfg::LDS_BYTES > 64 * 1024) {
+      (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_tcec_kernel<Cfg>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES);
+    }
+    attr_done = true;
+  }
+  hipLaunchKernelGGL(gemm_tcec_kernel<Cfg>, grid, dim3(Cfg::NT), Cfg::LDS_BYTES, stream, args);
+}
+
+template <class Cfg> constexpr KernelEntry make_entry(const char *name) {
+  return KernelEntry{&launch_cfg<Cfg>, Cfg::BM,  Cfg::BN,        Cfg::WM,  Cfg::WN,
+                     Cfg::NT,          Cfg::LDS_BYTES, Cfg::OCC, name};
+}
+
+// Per-(precision, type) tables, one translation unit each (gemm_inst_*.hip).
+// Indexed [layout][class].
+#define CUMPSGEMM_DECLARE_TABLE(sym) extern KernelEntry sym[4][kNumTileClasses];
+CUMPSGEMM_DECLARE_TABLE(g_tab_fp16tcec_s)
+CUMPSGEMM_DECLARE_TABLE(g_tab_fp16tcec_c)
+CUMPSGEMM_DECLARE_TABLE(g_tab_fp16tc_s)
+CUMPSGEMM_DECLARE_TABLE(g_tab_fp16tc_c)
+CUMPSGEMM_DECLARE_TABLE(g_tab_bf16x3_s)
+CUMPSGEMM_DECLARE_TABLE(g_tab_bf16x3_c)
+CUMPSGEMM_DECLARE_TABLE(g_tab_bf16x2_s)
+CUMPSGEMM_DECLARE_TABLE(g_tab_bf16x2_c)
+#undef CUMPSGEMM_DECLARE_TABLE
+
+// Real tiles: {BM, BN, WM, WN, OCC} per class; complex likewise.
+// One row of a table = the same three tile classes for one layout pair.
+#define CUMPSGEMM_REAL_ROW(P, AKC, BKC)                                              \
+  {                                                                                  \
+    make_entry<GemmCfg<P, false, AKC, BKC, 128, 128, 64, 64, 2>>("128x128x32_w64x64"), \
+    make_entry<GemmCfg<P, false, AKC, BKC, 64, 64, 32, 32, 2>>("64x64x32_w32x32"),   \
+    make_entry<GemmCfg<P, false, AKC, BKC, 32, 32, 32, 32, 2>>("32x32x32_w32x32")    \
+  }
+#define CUMPSGEMM_CPLX_ROW(P, AKC, BKC)                                              \
+  {                                                                                  \
+    make_entry<GemmCfg<P, true, AKC, BKC, 64, 64, 32, 32, 2>>("c64x64x32_w32x32"),   \
+    make_entry<GemmCfg<P, true, AKC, BKC, 64, 64, 32, 32, 2>>("c64x64x32_w32x32"),   \
+    make_entry<GemmCfg<P, true, AKC, BKC, 32, 32, 32, 32, 2>>("c32x32x32_w32x32")    \
+  }
+#define CUMPSGEMM_DEFINE_TABLE(sym, ROW, P)                                          \
+  KernelEntry sym[4][kNumTileClasses] = {ROW(P, false, false), ROW(P, true, false), \
+                                         ROW(P, false, true), ROW(P, true, true)};
+
+} // namespace cumpsgemm_amd

@@ -1,0 +1,88 @@
+// Library-private state behind the opaque cuMpSGEMM_handle_t.
+// Plays the role of reference src/handle.hpp:7-29, src/exp_stats.hpp:7-29 and
+// src/dynamic_launch.hpp:8-19, laid out for this implementation.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <cumpsgemm/cumpsgemm.h>
+#include <algorithm>
+#include <cstring>
+#include <chrono>
+#include <cstdint>
+#include <string>
+#include <unordered_map>
+
+namespace cumpsgemm_amd {
+
+// One result slot of the exponent-statistics ring (device memory).
+struct StatsSlot {
+  uint32_t max_exp_bits;        // bits(max|x|) & 0x7f800000
+  int32_t mode;                 // cuMpSGEMM_compute_mode_t decided for the matrix
+  unsigned long long total;     // #{|x| >= ignore threshold}
+  unsigned long long underflow; // #{ignore <= |x| < underflow threshold}
+  uint32_t pad[2];
+};
+static_assert(sizeof(StatsSlot) == 32, "slot layout");
+
+// Per-workgroup partial result of a statistics pass (device scratch).
+struct StatsPartial {
+  uint32_t max_bits;
+  uint32_t pad;
+  unsigned long long total;
+  unsigned long long underflow;
+};
+
+struct Profiler {
+  struct Entry {
+    double sum = 0.0;
+    uint64_t n = 0;
+  };
+  bool enabled = false;
+  std::unordered_map<std::string, Entry> entries;
+  std::chrono::steady_clock::time_point t0;
+};
+
+constexpr unsigned kRingLength = 10000;        // reference src/exp_stats.cu:574
+constexpr unsigned kMaxStatsBlocks = 4096;     // partial-result scratch entries
+} // namespace cumpsgemm_amd
+
+struct cuMpSGEMM_handle {
+  int device = 0;
+  unsigned num_cus = 0;
+  hipStream_t stream = nullptr;
+
+  // ---- exponent statistics ----
+  bool exp_stats_enabled = false;
+  cumpsgemm_amd::StatsSlot *stats_slots = nullptr;       // [ring_length]
+  cumpsgemm_amd::StatsPartial *stats_partials = nullptr; // [kMaxStatsBlocks]
+  unsigned *stats_ticket = nullptr;                      // self-resetting arrival counter
+  unsigned stats_ring_length = cumpsgemm_amd::kRingLength;
+  unsigned stats_current_id = 1; // slots 0 / 1 are reserved presets
+  float ignore_threshold = 0.0f;
+  float underflow_threshold = 1.0f / 32768.0f;
+  float underflow_tolerance_rate = 0.0f;
+
+  // ---- launch-flag ring (AUTO mode) ----
+  int *flag_buffer = nullptr; // [flag_ring_length]
+  unsigned flag_ring_length = cumpsgemm_amd::kRingLength;
+  unsigned flag_current_id = 1;
+  bool flag_enabled = false;
+  unsigned flag_enabled_id = 0;
+
+  // pinned host word for small read-backs
+  unsigned long long *host_scratch = nullptr; // [4]
+
+  cumpsgemm_amd::Profiler profiler;
+};
+
+namespace cumpsgemm_amd {
+// Wall-clock bracket around a launch when profiling is on (reference:
+// cutf profiler start_timer_sync / stop_timer_sync, src/cumpsgemm.cu:263-271).
+struct ProfileScope {
+  cuMpSGEMM_handle *h;
+  const char *name;
+  ProfileScope(cuMpSGEMM_handle *handle, const char *label);
+  ~ProfileScope();
+};
+
+void check_hip(hipError_t err, const char *what);
+} // namespace cumpsgemm_amd

@@ -1,0 +1,436 @@
+// hipBLAS interposer.  When libcumpsgemm.so is LD_PRELOADed the six symbols
+// below shadow hipBLAS's; each call asks the mode rule what to do and either
+// forwards to the real hipBLAS function (found with dlsym(RTLD_NEXT)) or runs
+// the TCEC pipeline on the library's global handle, on the caller's stream.
+//
+// Takes the place of reference src/cumpsgemm_cublas.cu: mode query :198-220,
+// per-call flow :222-593 / :595-976, intercepted symbols :979-1187,
+// hijack_control :1189-1271, global handle and env configuration :101-157.
+#include "handle.hpp"
+#include "pipeline.hpp"
+#include "utils.hpp"
+#include <cumpsgemm/cumpsgemm.hpp>
+#include <cumpsgemm/cumpsgemm_ext.h>
+#include <cumpsgemm/hijack_control.hpp>
+#include <dlfcn.h>
+#include <mutex>
+#include <sstream>
+#include <stdexcept>
+#include <type_traits>
+
+namespace {
+using namespace cumpsgemm_amd;
+
+cuMpSGEMM_handle_t g_handle = nullptr;
+std::once_flag g_handle_once;
+std::string g_last_called;
+bool g_mx2x2_enabled = false;
+bool g_restore_AB = true;
+cumpsgemm::hijack_control::control_function_t g_control_func;
+enum { STATIC_MODE, DYNAMIC_MODE } g_hijack_mode = DYNAMIC_MODE;
+cuMpSGEMM_compute_mode_t g_static_mode = CUMPSGEMM_CUBLAS;
+
+std::string sci(double v) {
+  std::stringstream ss;
+  ss << std::scientific << v;
+  return ss.str();
+}
+
+const char *op_str(hipblasOperation_t op) {
+  switch (op) {
+  case HIPBLAS_OP_N: return "N";
+  case HIPBLAS_OP_T: return "T";
+  case HIPBLAS_OP_C: return "C";
+  default: return "?";
+  }
+}
+
+// The next definition of `name` after this library in the lookup order (the
+// real hipBLAS when we are preloaded); falls back to opening libhipblas.so.
+void *real_symbol(const char *name) {
+  void *p = dlsym(RTLD_NEXT, name);
+  if (p == nullptr) {
+    static void *lib = dlopen("libhipblas.so", RTLD_NOW | RTLD_GLOBAL);
+    if (lib == nullptr) lib = dlopen("libhipblas.so.3", RTLD_NOW | RTLD_GLOBAL);
+    if (lib != nullptr) p = dlsym(lib, name);
+  }
+  if (p == nullptr)
+    log_error(std::string("Could not load the hipBLAS function \"") + name + "\"");
+  return p;
+}
+
+hipStream_t caller_stream(hipblasHandle_t hb) {
+  using fn_t = hipblasStatus_t (*)(hipblasHandle_t, hipStream_t *);
+  static fn_t fn = reinterpret_cast<fn_t>(real_symbol("hipblasGetStream"));
+  hipStream_t s = nullptr;
+  if (fn != nullptr && hb != nullptr) (void)fn(hb, &s);
+  return s;
+}
+
+bool mx2x2_enabled() {
+  if (g_mx2x2_enabled) return true;
+  return env_flag("CUMPSGEMM_CUSTOM_GEMM_MX2X2", false);
+}
+
+float env_float(const char *name, float dflt) {
+  const char *v = std::getenv(name);
+  return v ? std::stof(v) : dflt;
+}
+int env_int(const char *name, int dflt) {
+  const char *v = std::getenv(name);
+  return v ? std::stoi(v) : dflt;
+}
+
+cuMpSGEMM_handle_t global_handle() {
+  std::call_once(g_handle_once, []() {
+    log_info("Initialize cuMpSGEMM handle...");
+    if (cuMpSGEMM_create(&g_handle) != HIPBLAS_STATUS_SUCCESS) {
+      log_error("Initialization failed.");
+      g_handle = nullptr;
+      return;
+    }
+    const float ignore_thr = env_float("CUMPSGEMM_AUTO_IGNORE_THRESHOLD", 0.0f);
+    const float under_thr = env_float("CUMPSGEMM_AUTO_UNDERFLOW_THRESHOLD", 1.0f / 32768);
+    const float tol = env_float("CUMPSGEMM_AUTO_UNDERFLOW_TOLERANCE_RATE", 0.0f);
+    const int restore = env_int("CUMPSGEMM_AUTO_RESTORE_AB_SCALING", 1);
+    log_info("AUTO config: ignore_threshold=" + sci(ignore_thr) + " @Init");
+    log_info("AUTO config: underflow_threshold=" + sci(under_thr) + " @Init");
+    log_info("AUTO config: underflow_tolerance_rate=" + sci(tol) + " @Init");
+    log_info("AUTO config: restore_AB_scaling=" + std::to_string(restore) + " @Init");
+    log_info(std::string("CUSTOM_GEMM_MX2X2: ") + (mx2x2_enabled() ? "enabled" : "disabled") +
+             " @Init");
+    cumpsgemm::set_exp_stats_params(g_handle, ignore_thr, under_thr, tol);
+    g_restore_AB = restore != 0;
+  });
+  return g_handle;
+}
+
+using rule_fn_t = cuMpSGEMM_compute_mode_t (*)(const char *, hipblasHandle_t, hipblasOperation_t,
+                                               hipblasOperation_t, unsigned, unsigned, unsigned);
+
+// The user's rule library, looked up once.  The documented contract is that a
+// libcumpsgemm_rule.so on the loader path which defines
+// cuMpSGEMM_get_compute_mode replaces the built-in rule.
+rule_fn_t user_rule() {
+  static rule_fn_t fn = []() -> rule_fn_t {
+    void *lib = dlopen("libcumpsgemm_rule.so", RTLD_NOW | RTLD_LOCAL);
+    if (lib == nullptr) {
+      log_warning("Failed to load libcumpsgemm_rule.so. Default rule will be used.");
+      return nullptr;
+    }
+    void *p = dlsym(lib, "cuMpSGEMM_get_compute_mode");
+    if (p == nullptr) {
+      log_warning("Failed to load a function cuMpSGEMM_get_compute_mode during selecting "
+                  "hijacking function. Default rule will be used.");
+      return nullptr;
+    }
+    return reinterpret_cast<rule_fn_t>(p);
+  }();
+  return fn;
+}
+
+cuMpSGEMM_compute_mode_t query_mode(const char *func_name, hipblasHandle_t hb,
+                                    hipblasOperation_t op_A, hipblasOperation_t op_B, unsigned m,
+                                    unsigned n, unsigned k) {
+  if (g_hijack_mode == STATIC_MODE) return g_static_mode;
+  if (g_control_func) return g_control_func((int)op_A, (int)op_B, m, n, k);
+  if (rule_fn_t fn = user_rule()) return fn(func_name, hb, op_A, op_B, m, n, k);
+  return cuMpSGEMM_get_compute_mode(func_name, hb, op_A, op_B, m, n, k);
+}
+
+bool forwards_to_hipblas(cuMpSGEMM_compute_mode_t mode) {
+  return mode == CUMPSGEMM_CUBLAS || mode == CUMPSGEMM_CUBLAS_FP16TC ||
+         mode == CUMPSGEMM_CUBLAS_TF32TC || mode == CUMPSGEMM_CUBLAS_SIMT;
+}
+
+bool is_pow2(uint64_t v) { return (v & (v - 1)) == 0; }
+
+template <class T> struct ffi;
+template <> struct ffi<float> {
+  static constexpr const char *gemm = "hipblasSgemm";
+  static constexpr const char *gemm_sb = "hipblasSgemmStridedBatched";
+};
+template <> struct ffi<hipComplex> {
+  static constexpr const char *gemm = "hipblasCgemm";
+  static constexpr const char *gemm_sb = "hipblasCgemmStridedBatched";
+};
+
+template <class T>
+hipblasStatus_t forward_gemm(hipblasHandle_t hb, hipblasOperation_t op_A, hipblasOperation_t op_B,
+                             int m, int n, int k, const T *alpha, const T *a, int lda, const T *b,
+                             int ldb, const T *beta, T *c, int ldc) {
+  using fn_t = hipblasStatus_t (*)(hipblasHandle_t, hipblasOperation_t, hipblasOperation_t, int,
+                                   int, int, const T *, const T *, int, const T *, int, const T *,
+                                   T *, int);
+  static fn_t fn = reinterpret_cast<fn_t>(real_symbol(ffi<T>::gemm));
+  if (fn == nullptr) return HIPBLAS_STATUS_NOT_SUPPORTED;
+  return fn(hb, op_A, op_B, m, n, k, alpha, a, lda, b, ldb, beta, c, ldc);
+}
+
+template <class T>
+hipblasStatus_t forward_gemm_sb(hipblasHandle_t hb, hipblasOperation_t op_A,
+                                hipblasOperation_t op_B, int m, int n, int k, const T *alpha,
+                                const T *a, int lda, long long sa, const T *b, int ldb,
+                                long long sb, const T *beta, T *c, int ldc, long long sc,
+                                int batch) {
+  using fn_t = hipblasStatus_t (*)(hipblasHandle_t, hipblasOperation_t, hipblasOperation_t, int,
+                                   int, int, const T *, const T *, int, long long, const T *, int,
+                                   long long, const T *, T *, int, long long, int);
+  static fn_t fn = reinterpret_cast<fn_t>(real_symbol(ffi<T>::gemm_sb));
+  if (fn == nullptr) return HIPBLAS_STATUS_NOT_SUPPORTED;
+  return fn(hb, op_A, op_B, m, n, k, alpha, a, lda, sa, b, ldb, sb, beta, c, ldc, sc, batch);
+}
+
+// One intercepted call.  batched == false: strides are ignored, batch == 1.
+template <class T>
+hipblasStatus_t hijack_core(const char *func_name, hipblasHandle_t hb, hipblasOperation_t op_A,
+                            hipblasOperation_t op_B, int m, int n, int k, const T *alpha,
+                            const T *a, int lda, long long sa, const T *b, int ldb, long long sb,
+                            const T *beta, T *c, int ldc, long long sc, int batch, bool batched) {
+  if (m <= 0 || n <= 0 || k <= 0 || lda <= 0 || ldb <= 0 || ldc <= 0 || (batched && batch <= 0)) {
+    return HIPBLAS_STATUS_INVALID_VALUE;
+  }
+  const cuMpSGEMM_compute_mode_t mode = query_mode(func_name, hb, op_A, op_B, m, n, k);
+  cuMpSGEMM_handle_t h = global_handle();
+
+  log_info(std::string(func_name) + " op=(" + op_str(op_A) + ", " + op_str(op_B) + "), shape=(" +
+           std::to_string(m) + ", " + std::to_string(n) + ", " + std::to_string(k) + ")" +
+           (batched ? ", batch=" + std::to_string(batch) : std::string()) +
+           ", mode=" + cuMpSGEMM_get_compute_mode_string(mode) + "[" +
+           (g_hijack_mode == DYNAMIC_MODE ? "dynamic" : "static") +
+           "][exp_stats:" + ((h && h->exp_stats_enabled) ? "1" : "0") + "]");
+  g_last_called = std::string(func_name) + "," + op_str(op_A) + "," + op_str(op_B) + "," +
+                  std::to_string(m) + "," + std::to_string(n) + "," + std::to_string(k) + "," +
+                  std::to_string(batched ? batch : 1) + "," +
+                  cuMpSGEMM_get_compute_mode_string(mode);
+
+  if (mode == CUMPSGEMM_DRY_RUN) return HIPBLAS_STATUS_SUCCESS;
+  if (h == nullptr) return HIPBLAS_STATUS_NOT_INITIALIZED;
+
+  // kernels of this library run on the caller's stream so that ordering with
+  // the application's other work is preserved
+  cuMpSGEMM_set_stream(h, caller_stream(hb));
+  const uint64_t nb = batched ? (uint64_t)batch : 1;
+  const uint64_t usa = batched ? (uint64_t)sa : 0, usb = batched ? (uint64_t)sb : 0,
+                 usc = batched ? (uint64_t)sc : 0;
+
+  if (mx2x2_enabled() && n == 2 && k == 2 && is_pow2((uint64_t)m)) {
+    log_info(" +---> gemm_Mx2x2");
+    if constexpr (std::is_same<T, float>::value)
+      return cuMpSGEMM_sgemm_Mx2x2(h, op_A, op_B, m, alpha, a, lda, usa, b, ldb, usb, beta, c, ldc,
+                                   usc, nb);
+    else
+      return cuMpSGEMM_cgemm_Mx2x2(h, op_A, op_B, m, alpha, a, lda, usa, b, ldb, usb, beta, c, ldc,
+                                   usc, nb);
+  }
+  if (mx2x2_enabled() && m == 2 && k == 2 && is_pow2((uint64_t)n)) {
+    log_info(" +---> gemm_2xNx2");
+    if constexpr (std::is_same<T, float>::value)
+      return cuMpSGEMM_sgemm_2xNx2(h, op_A, op_B, n, alpha, a, lda, usa, b, ldb, usb, beta, c, ldc,
+                                   usc, nb);
+    else
+      return cuMpSGEMM_cgemm_2xNx2(h, op_A, op_B, n, alpha, a, lda, usa, b, ldb, usb, beta, c, ldc,
+                                   usc, nb);
+  }
+
+  if (forwards_to_hipblas(mode)) {
+    const hipblasStatus_t st =
+        batched ? forward_gemm_sb<T>(hb, op_A, op_B, m, n, k, alpha, a, lda, sa, b, ldb, sb, beta,
+                                     c, ldc, sc, batch)
+                : forward_gemm<T>(hb, op_A, op_B, m, n, k, alpha, a, lda, b, ldb, beta, c, ldc);
+    if (h->exp_stats_enabled) {
+      // statistics of the result, as the reference does for forwarded calls
+      // (src/cumpsgemm_cublas.cu:420-425)
+      cumpsgemm::exp_stats_ext<T>(h, (unsigned)m, (unsigned)n, c, (unsigned)ldc,
+                                  batched ? (unsigned)batch : 1u, batched ? (unsigned)sc : 0u);
+    }
+    return st;
+  }
+  if (mode == CUMPSGEMM_FP32_SIMT || mode == CUMPSGEMM_UNDEFINED) {
+    log_error(std::string("mode ") + cuMpSGEMM_get_compute_mode_string(mode) +
+              " is not executable; forwarding to hipBLAS");
+    return batched ? forward_gemm_sb<T>(hb, op_A, op_B, m, n, k, alpha, a, lda, sa, b, ldb, sb,
+                                        beta, c, ldc, sc, batch)
+                   : forward_gemm<T>(hb, op_A, op_B, m, n, k, alpha, a, lda, b, ldb, beta, c, ldc);
+  }
+  // the scaled modes write A and B in place and restore them afterwards
+  return gemm_pipeline<T>(h, op_A, op_B, m, n, k, alpha, const_cast<T *>(a), lda, usa,
+                          const_cast<T *>(b), ldb, usb, beta, c, ldc, usc, nb, batched, mode,
+                          g_restore_AB, nullptr);
+}
+} // namespace
+
+// ---- intercepted hipBLAS symbols (prototypes of ROCm 7.2 hipblas.h) ----------
+extern "C" {
+hipblasStatus_t hipblasSgemm(hipblasHandle_t handle, hipblasOperation_t transA,
+                             hipblasOperation_t transB, int m, int n, int k, const float *alpha,
+                             const float *AP, int lda, const float *BP, int ldb, const float *beta,
+                             float *CP, int ldc) {
+  return hijack_core<float>(__func__, handle, transA, transB, m, n, k, alpha, AP, lda, 0, BP, ldb,
+                            0, beta, CP, ldc, 0, 1, false);
+}
+
+hipblasStatus_t hipblasCgemm(hipblasHandle_t handle, hipblasOperation_t transA,
+                             hipblasOperation_t transB, int m, int n, int k,
+                             const hipComplex *alpha, const hipComplex *AP, int lda,
+                             const hipComplex *BP, int ldb, const hipComplex *beta, hipComplex *CP,
+                             int ldc) {
+  return hijack_core<hipComplex>(__func__, handle, transA, transB, m, n, k, alpha, AP, lda, 0, BP,
+                                 ldb, 0, beta, CP, ldc, 0, 1, false);
+}
+
+hipblasStatus_t hipblasSgemmStridedBatched(hipblasHandle_t handle, hipblasOperation_t transA,
+                                           hipblasOperation_t transB, int m, int n, int k,
+                                           const float *alpha, const float *AP, int lda,
+                                           long long strideA, const float *BP, int ldb,
+                                           long long strideB, const float *beta, float *CP,
+                                           int ldc, long long strideC, int batchCount) {
+  return hijack_core<float>(__func__, handle, transA, transB, m, n, k, alpha, AP, lda, strideA, BP,
+                            ldb, strideB, beta, CP, ldc, strideC, batchCount, true);
+}
+
+hipblasStatus_t hipblasCgemmStridedBatched(hipblasHandle_t handle, hipblasOperation_t transA,
+                                           hipblasOperation_t transB, int m, int n, int k,
+                                           const hipComplex *alpha, const hipComplex *AP, int lda,
+                                           long long strideA, const hipComplex *BP, int ldb,
+                                           long long strideB, const hipComplex *beta,
+                                           hipComplex *CP, int ldc, long long strideC,
+                                           int batchCount) {
+  return hijack_core<hipComplex>(__func__, handle, transA, transB, m, n, k, alpha, AP, lda,
+                                 strideA, BP, ldb, strideB, beta, CP, ldc, strideC, batchCount,
+                                 true);
+}
+
+// Only all-FP32-real or all-FP32-complex calls are taken over; every other
+// type combination goes to hipBLAS untouched (reference :1050-1108).
+hipblasStatus_t hipblasGemmEx(hipblasHandle_t handle, hipblasOperation_t transA,
+                              hipblasOperation_t transB, int m, int n, int k, const void *alpha,
+                              const void *A, hipDataType aType, int lda, const void *B,
+                              hipDataType bType, int ldb, const void *beta, void *C,
+                              hipDataType cType, int ldc, hipblasComputeType_t computeType,
+                              hipblasGemmAlgo_t algo) {
+  if (aType == HIP_R_32F && bType == HIP_R_32F && cType == HIP_R_32F) {
+    return hijack_core<float>(__func__, handle, transA, transB, m, n, k,
+                              static_cast<const float *>(alpha), static_cast<const float *>(A),
+                              lda, 0, static_cast<const float *>(B), ldb, 0,
+                              static_cast<const float *>(beta), static_cast<float *>(C), ldc, 0, 1,
+                              false);
+  }
+  if (aType == HIP_C_32F && bType == HIP_C_32F && cType == HIP_C_32F) {
+    return hijack_core<hipComplex>(
+        __func__, handle, transA, transB, m, n, k, static_cast<const hipComplex *>(alpha),
+        static_cast<const hipComplex *>(A), lda, 0, static_cast<const hipComplex *>(B), ldb, 0,
+        static_cast<const hipComplex *>(beta), static_cast<hipComplex *>(C), ldc, 0, 1, false);
+  }
+  using fn_t = hipblasStatus_t (*)(hipblasHandle_t, hipblasOperation_t, hipblasOperation_t, int,
+                                   int, int, const void *, const void *, hipDataType, int,
+                                   const void *, hipDataType, int, const void *, void *,
+                                   hipDataType, int, hipblasComputeType_t, hipblasGemmAlgo_t);
+  static fn_t fn = reinterpret_cast<fn_t>(real_symbol("hipblasGemmEx"));
+  if (fn == nullptr) return HIPBLAS_STATUS_NOT_SUPPORTED;
+  return fn(handle, transA, transB, m, n, k, alpha, A, aType, lda, B, bType, ldb, beta, C, cType,
+            ldc, computeType, algo);
+}
+
+hipblasStatus_t hipblasGemmStridedBatchedEx(
+    hipblasHandle_t handle, hipblasOperation_t transA, hipblasOperation_t transB, int m, int n,
+    int k, const void *alpha, const void *A, hipDataType aType, int lda, hipblasStride strideA,
+    const void *B, hipDataType bType, int ldb, hipblasStride strideB, const void *beta, void *C,
+    hipDataType cType, int ldc, hipblasStride strideC, int batchCount,
+    hipblasComputeType_t computeType, hipblasGemmAlgo_t algo) {
+  if (aType == HIP_R_32F && bType == HIP_R_32F && cType == HIP_R_32F) {
+    return hijack_core<float>(__func__, handle, transA, transB, m, n, k,
+                              static_cast<const float *>(alpha), static_cast<const float *>(A),
+                              lda, strideA, static_cast<const float *>(B), ldb, strideB,
+                              static_cast<const float *>(beta), static_cast<float *>(C), ldc,
+                              strideC, batchCount, true);
+  }
+  if (aType == HIP_C_32F && bType == HIP_C_32F && cType == HIP_C_32F) {
+    return hijack_core<hipComplex>(
+        __func__, handle, transA, transB, m, n, k, static_cast<const hipComplex *>(alpha),
+        static_cast<const hipComplex *>(A), lda, strideA, static_cast<const hipComplex *>(B), ldb,
+        strideB, static_cast<const hipComplex *>(beta), static_cast<hipComplex *>(C), ldc, strideC,
+        batchCount, true);
+  }
+  using fn_t = hipblasStatus_t (*)(hipblasHandle_t, hipblasOperation_t, hipblasOperation_t, int,
+                                   int, int, const void *, const void *, hipDataType, int,
+                                   hipblasStride, const void *, hipDataType, int, hipblasStride,
+                                   const void *, void *, hipDataType, int, hipblasStride, int,
+                                   hipblasComputeType_t, hipblasGemmAlgo_t);
+  static fn_t fn = reinterpret_cast<fn_t>(real_symbol("hipblasGemmStridedBatchedEx"));
+  if (fn == nullptr) return HIPBLAS_STATUS_NOT_SUPPORTED;
+  return fn(handle, transA, transB, m, n, k, alpha, A, aType, lda, strideA, B, bType, ldb, strideB,
+            beta, C, cType, ldc, strideC, batchCount, computeType, algo);
+}
+} // extern "C"
+
+// ---- hijack_control -----------------------------------------------------------
+namespace cumpsgemm {
+namespace hijack_control {
+cuMpSGEMM_handle_t get_internal_global_handle() { return global_handle(); }
+void set_compute_mode(cuMpSGEMM_compute_mode_t mode) {
+  if (mode == CUMPSGEMM_FP32_SIMT)
+    throw std::runtime_error("CUMPSGEMM_FP32_SIMT mode is currently not supported.");
+  g_static_mode = mode;
+  g_hijack_mode = STATIC_MODE;
+}
+void unset_compute_mode() { g_hijack_mode = DYNAMIC_MODE; }
+void enable_custom_gemm_Mx2x2() { g_mx2x2_enabled = true; }
+void disable_custom_gemm_Mx2x2() { g_mx2x2_enabled = false; }
+void reset_exp_stats_buffer_id() { cumpsgemm::reset_exp_stats_buffer_id(global_handle()); }
+void set_exp_stats_params(float ignore_threshold, float underflow_threshold,
+                          float underflow_tolerance_rate) {
+  log_info("AUTO config: ignore_threshold=" + sci(ignore_threshold) + " @" + __func__);
+  log_info("AUTO config: underflow_threshold=" + sci(underflow_threshold) + " @" + __func__);
+  log_info("AUTO config: underflow_tolerance_rate=" + sci(underflow_tolerance_rate) + " @" +
+           __func__);
+  cumpsgemm::set_exp_stats_params(global_handle(), ignore_threshold, underflow_threshold,
+                                  underflow_tolerance_rate);
+}
+void enable_restoring_AB_after_scaling() {
+  g_restore_AB = true;
+  log_info(std::string("AUTO config: restore_AB_scaling=True @") + __func__);
+}
+void disable_restoring_AB_after_scaling() {
+  g_restore_AB = false;
+  log_info(std::string("AUTO config: restore_AB_scaling=False @") + __func__);
+}
+std::string get_last_called_function_str() { return g_last_called; }
+void set_last_called_function_str(const std::string func_str) { g_last_called = func_str; }
+void clear_last_called_function_str() { g_last_called.clear(); }
+bool is_library_loaded() { return true; }
+void set_control_function(const control_function_t control_function) {
+  g_control_func = control_function;
+}
+void unset_control_function() { g_control_func = nullptr; }
+} // namespace hijack_control
+} // namespace cumpsgemm
+
+extern "C" {
+cuMpSGEMM_handle_t cuMpSGEMM_hijack_get_internal_global_handle(void) { return global_handle(); }
+int cuMpSGEMM_hijack_set_compute_mode(int mode) {
+  try {
+    cumpsgemm::hijack_control::set_compute_mode((cuMpSGEMM_compute_mode_t)mode);
+  } catch (const std::exception &) {
+    return -1;
+  }
+  return 0;
+}
+void cuMpSGEMM_hijack_unset_compute_mode(void) { cumpsgemm::hijack_control::unset_compute_mode(); }
+void cuMpSGEMM_hijack_enable_custom_gemm_Mx2x2(void) { g_mx2x2_enabled = true; }
+void cuMpSGEMM_hijack_disable_custom_gemm_Mx2x2(void) { g_mx2x2_enabled = false; }
+void cuMpSGEMM_hijack_set_restore_AB(int enable) { g_restore_AB = enable != 0; }
+size_t cuMpSGEMM_hijack_get_last_called_function_str(char *buf, size_t buf_len) {
+  if (buf != nullptr && buf_len > 0) {
+    std::snprintf(buf, buf_len, "%s", g_last_called.c_str());
+  }
+  return g_last_called.size();
+}
+void cuMpSGEMM_hijack_clear_last_called_function_str(void) { g_last_called.clear(); }
+int cuMpSGEMM_hijack_is_library_loaded(void) { return 1; }
+int cuMpSGEMM_hijack_query_compute_mode(const char *func_name, int op_A, int op_B, unsigned m,
+                                        unsigned n, unsigned k) {
+  return (int)query_mode(func_name, nullptr, (hipblasOperation_t)op_A, (hipblasOperation_t)op_B, m,
+                         n, k);
+}
+}

@@ -1,0 +1,132 @@
+// Mode pipeline of one GEMM call: statistics -> decision -> scaling -> GEMM ->
+// inverse scaling -> restore.  Everything is enqueued on the handle's stream;
+// the decision lives in device memory (launch flag), so there is no host
+// synchronisation.  Follows the orchestration of the reference's interposer,
+// src/cumpsgemm_cublas.cu:446-577 (single) and :836-960 (strided batch).
+#include "pipeline.hpp"
+#include "handle.hpp"
+#include <cumpsgemm/cumpsgemm_ext.h>
+
+namespace cumpsgemm_amd {
+template <class T>
+hipblasStatus_t gemm_pipeline(cuMpSGEMM_handle_t h, hipblasOperation_t op_A,
+                              hipblasOperation_t op_B, uint64_t m, uint64_t n, uint64_t k,
+                              const T *alpha, T *a, uint64_t lda, uint64_t stridea, T *b,
+                              uint64_t ldb, uint64_t strideb, const T *beta, T *c, uint64_t ldc,
+                              uint64_t stridec, uint64_t batch, bool batched,
+                              cuMpSGEMM_compute_mode_t mode, bool restore_AB, PipelineIds *ids) {
+  // stored shapes of A and B (rows x cols as laid out in memory)
+  const unsigned a_rows = (unsigned)(op_A == HIPBLAS_OP_N ? m : k);
+  const unsigned a_cols = (unsigned)(op_A == HIPBLAS_OP_N ? k : m);
+  const unsigned b_rows = (unsigned)(op_B == HIPBLAS_OP_N ? k : n);
+  const unsigned b_cols = (unsigned)(op_B == HIPBLAS_OP_N ? n : k);
+  // the non-batched form scans one matrix: batch 1, stride 0
+  const unsigned sb = batched ? (unsigned)batch : 1u;
+  const unsigned sa_stride = batched ? (unsigned)stridea : 0u;
+  const unsigned sb_stride = batched ? (unsigned)strideb : 0u;
+  const unsigned sc_stride = batched ? (unsigned)stridec : 0u;
+
+  unsigned a_id = 0, b_id = 0, flag_id = 0;
+  const bool scaled = (mode == CUMPSGEMM_AUTO || mode == CUMPSGEMM_FP16TCEC_SCALING);
+  if (mode == CUMPSGEMM_AUTO) {
+    a_id = cumpsgemm::exp_stats_ext<T>(h, a_rows, a_cols, a, (unsigned)lda, sb, sa_stride);
+    b_id = cumpsgemm::exp_stats_ext<T>(h, b_rows, b_cols, b, (unsigned)ldb, sb, sb_stride);
+    flag_id = cumpsgemm::get_next_dynamic_launch_buffer_id(h);
+    cumpsgemm::set_dynamic_launch_buffer_by_exp_stats(h, flag_id, a_id, b_id);
+    cumpsgemm::scale_A<T>(h, a_id, flag_id, a_rows, a_cols, a, (unsigned)lda, sb, sa_stride);
+    cumpsgemm::scale_B<T>(h, b_id, flag_id, b_rows, b_cols, b, (unsigned)ldb, sb, sb_stride);
+    cumpsgemm::set_dynamic_launch_flag_buffer_id(h, flag_id);
+  } else if (mode == CUMPSGEMM_FP16TCEC_SCALING) {
+    flag_id = 1; // preset: FP16TCEC with both scale bits
+    a_id = cumpsgemm::exp_max_ext<T>(h, a_rows, a_cols, a, (unsigned)lda, sb, sa_stride);
+    b_id = cumpsgemm::exp_max_ext<T>(h, b_rows, b_cols, b, (unsigned)ldb, sb, sb_stride);
+    cumpsgemm::scale_A<T>(h, a_id, flag_id, a_rows, a_cols, a, (unsigned)lda, sb, sa_stride);
+    cumpsgemm::scale_B<T>(h, b_id, flag_id, b_rows, b_cols, b, (unsigned)ldb, sb, sb_stride);
+  }
+  const cuMpSGEMM_compute_mode_t gemm_mode =
+      (mode == CUMPSGEMM_FP16TCEC_SCALING) ? CUMPSGEMM_FP16TCEC : mode;
+  hipblasStatus_t st;
+  if (batched) {
+    st = cumpsgemm::gemm_stridedBatch<T>(h, op_A, op_B, m, n, k, alpha, a, lda, stridea, b, ldb,
+                                         strideb, beta, c, ldc, stridec, batch, gemm_mode);
+  } else {
+    st = cumpsgemm::gemm<T>(h, op_A, op_B, m, n, k, alpha, a, lda, b, ldb, beta, c, ldc,
+                            gemm_mode);
+  }
+  if (scaled) {
+    cumpsgemm::scale_C<T>(h, a_id, b_id, flag_id, (unsigned)m, (unsigned)n, c, (unsigned)ldc, sb,
+                          sc_stride);
+    if (restore_AB) {
+      cumpsgemm::reset_scale_A<T>(h, a_id, flag_id, a_rows, a_cols, a, (unsigned)lda, sb,
+                                  sa_stride);
+      cumpsgemm::reset_scale_B<T>(h, b_id, flag_id, b_rows, b_cols, b, (unsigned)ldb, sb,
+                                  sb_stride);
+    }
+    if (mode == CUMPSGEMM_AUTO) cumpsgemm::unset_dynamic_launch_flag_buffer_id(h);
+  }
+  if (ids != nullptr) {
+    ids->a_slot = a_id;
+    ids->b_slot = b_id;
+    ids->flag_slot = flag_id;
+  }
+  return st;
+}
+
+template hipblasStatus_t gemm_pipeline<float>(cuMpSGEMM_handle_t, hipblasOperation_t,
+                                              hipblasOperation_t, uint64_t, uint64_t, uint64_t,
+                                              const float *, float *, uint64_t, uint64_t, float *,
+                                              uint64_t, uint64_t, const float *, float *, uint64_t,
+                                              uint64_t, uint64_t, bool, cuMpSGEMM_compute_mode_t,
+                                              bool, PipelineIds *);
+template hipblasStatus_t gemm_pipeline<hipComplex>(
+    cuMpSGEMM_handle_t, hipblasOperation_t, hipblasOperation_t, uint64_t, uint64_t, uint64_t,
+    const hipComplex *, hipComplex *, uint64_t, uint64_t, hipComplex *, uint64_t, uint64_t,
+    const hipComplex *, hipComplex *, uint64_t, uint64_t, uint64_t, bool,
+    cuMpSGEMM_compute_mode_t, bool, PipelineIds *);
+} // namespace cumpsgemm_amd
+
+using cumpsgemm_amd::PipelineIds;
+
+extern "C" {
+hipblasStatus_t cuMpSGEMM_sgemm_pipeline(cuMpSGEMM_handle_t handle, hipblasOperation_t op_A,
+                                         hipblasOperation_t op_B, uint64_t m, uint64_t n,
+                                         uint64_t k, const float *alpha, float *a, uint64_t lda,
+                                         uint64_t stridea, float *b, uint64_t ldb,
+                                         uint64_t strideb, const float *beta, float *c,
+                                         uint64_t ldc, uint64_t stridec, uint64_t batch_count,
+                                         cuMpSGEMM_compute_mode_t mode, int restore_AB,
+                                         unsigned *ids_out) {
+  PipelineIds ids;
+  const bool batched = !(batch_count == 1 && stridea == 0 && strideb == 0 && stridec == 0);
+  const auto st = cumpsgemm_amd::gemm_pipeline<float>(handle, op_A, op_B, m, n, k, alpha, a, lda,
+                                                      stridea, b, ldb, strideb, beta, c, ldc,
+                                                      stridec, batch_count, batched, mode,
+                                                      restore_AB != 0, &ids);
+  if (ids_out) {
+    ids_out[0] = ids.a_slot;
+    ids_out[1] = ids.b_slot;
+    ids_out[2] = ids.flag_slot;
+  }
+  return st;
+}
+hipblasStatus_t cuMpSGEMM_cgemm_pipeline(cuMpSGEMM_handle_t handle, hipblasOperation_t op_A,
+                                         hipblasOperation_t op_B, uint64_t m, uint64_t n,
+                                         uint64_t k, const hipComplex *alpha, hipComplex *a,
+                                         uint64_t lda, uint64_t stridea, hipComplex *b,
+                                         uint64_t ldb, uint64_t strideb, const hipComplex *beta,
+                                         hipComplex *c, uint64_t ldc, uint64_t stridec,
+                                         uint64_t batch_count, cuMpSGEMM_compute_mode_t mode,
+                                         int restore_AB, unsigned *ids_out) {
+  PipelineIds ids;
+  const bool batched = !(batch_count == 1 && stridea == 0 && strideb == 0 && stridec == 0);
+  const auto st = cumpsgemm_amd::gemm_pipeline<hipComplex>(
+      handle, op_A, op_B, m, n, k, alpha, a, lda, stridea, b, ldb, strideb, beta, c, ldc, stridec,
+      batch_count, batched, mode, restore_AB != 0, &ids);
+  if (ids_out) {
+    ids_out[0] = ids.a_slot;
+    ids_out[1] = ids.b_slot;
+    ids_out[2] = ids.flag_slot;
+  }
+  return st;
+}
+}

@@ -1,0 +1,604 @@
+/*
+ * CPU oracle for the TCEC GEMM path (TEST INFRASTRUCTURE -- never shipped,
+ * never on the product path).
+ *
+ * This file restates, for host cores and in plain C, the algorithm of the
+ * reference's hot path:
+ *   - the error-corrected split GEMM (reference: src/cumpsgemm_kernel.cuh:58-100
+ *     "mma_smem", src/device_tcec_wrapper.hpp:64-106 which forwards to the
+ *     un-vendored mtk::wmma::tcec library, epilogue src/dmem_accessor.hpp:173-228
+ *     and src/device_common.hpp:47-67),
+ *   - the exponent statistics (src/exp_stats.cu:32-62, :74-184, :187-293, :386-459),
+ *   - the power-of-two scaling (src/dynamic_scaling.cu:15, :75-150),
+ *   - the launch-flag packing (src/dynamic_launch_utils.hpp:10-41,
+ *     src/dynamic_scaling.cu:364-385) and ring ids (src/exp_stats.cu:15-24),
+ *   - the residual metric of the reference's harness (test/main.cu:153-234).
+ *
+ * The arithmetic of the split itself lives in a third-party dependency that is
+ * absent from the reference tree (github.com/wmmae/wmma_extension, namespace
+ * mtk::wmma::tcec, unpinned submodule, .gitmodules:4-6).  Its published
+ * algorithm (Ootomo & Yokota, "Recovering single precision accuracy from Tensor
+ * Cores while surpassing the FP32 theoretical peak performance") is restated:
+ *   hi = fp16_rn(a);  lo = fp16_rn((a - fp32(hi)) * 2^11);
+ *   C  = sum(hi_a*hi_b) + 2^-11 * (sum(lo_a*hi_b) + sum(hi_a*lo_b)),  lo*lo dropped,
+ * products exact in FP32, accumulation FP32 round-to-nearest.
+ *
+ * Pinning status (see tests/test_oracle_*.py):
+ *   - f32->f16 / f32->bf16 converters: pinned (exhaustive against numpy float16,
+ *     closed form for bf16).
+ *   - split: pinned by invariants (exact residual, 2^-22 reconstruction bound).
+ *   - GEMM: pinned at accuracy level (reference's own bar 2^-23*sqrt(K) vs FP64,
+ *     exact integer cases, closed forms); BIT-LEVEL parity with the reference's
+ *     tensor-core accumulation order is "parity unpinned" -- the reference holds
+ *     no golden vectors for it and cannot be built here.
+ *   - stats / scaling / flags / ring ids: pinned (brute-force scalar recount,
+ *     closed forms).
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+#define ORACLE_OP_N 111
+#define ORACLE_OP_T 112
+#define ORACLE_OP_C 113
+
+/* compute modes that the oracle emulates; numeric values follow the
+ * reference's enum (include/cumpsgemm/detail/common.h:6-20) */
+#define ORACLE_MODE_FP16TCEC 1
+#define ORACLE_MODE_TF32TCEC 2 /* served by bf16x3 on CDNA4 */
+#define ORACLE_MODE_FP16TC 3
+#define ORACLE_MODE_TF32TC 4 /* served by bf16x2 on CDNA4 */
+#define ORACLE_MODE_FP32 12  /* plain FP32 multiply-add, sequential in k */
+
+static inline uint32_t f2u(float f) {
+  uint32_t u;
+  memcpy(&u, &f, 4);
+  return u;
+}
+static inline float u2f(uint32_t u) {
+  float f;
+  memcpy(&f, &u, 4);
+  return f;
+}
+
+/* ---------------------------------------------------------------- converters */
+
+/* IEEE binary32 -> binary16, round-to-nearest-even, subnormals kept. */
+uint16_t oracle_f32_to_f16_bits(float f) {
+  const uint32_t x = f2u(f);
+  const uint32_t sign = (x >> 16) & 0x8000u;
+  const uint32_t ax = x & 0x7fffffffu;
+  if (ax > 0x7f800000u) { /* NaN -> quiet NaN, keep top payload bits */
+    return (uint16_t)(sign | 0x7e00u | ((ax >> 13) & 0x1ffu));
+  }
+  if (ax >= 0x477ff000u) { /* >= 65520 rounds to infinity (also Inf) */
+    return (uint16_t)(sign | 0x7c00u);
+  }
+  if (ax <= 0x33000000u) { /* <= 2^-25: rounds to zero (tie goes to even 0) */
+    return (uint16_t)sign;
+  }
+  if (ax < 0x38800000u) { /* subnormal half: |f| < 2^-14 */
+    const int e = (int)(ax >> 23);
+    const uint32_t m = (ax & 0x7fffffu) | 0x800000u;
+    const int shift = 126 - e; /* 14..24 */
+    uint32_t q = m >> shift;
+    const uint32_t rem = m & ((1u << shift) - 1u);
+    const uint32_t half = 1u << (shift - 1);
+    if (rem > half || (rem == half && (q & 1u))) q++;
+    return (uint16_t)(sign | q);
+  }
+  {
+    const uint32_t e = (ax >> 23) - 112u;
+    const uint32_t m = ax & 0x7fffffu;
+    uint32_t q = (e << 10) | (m >> 13);
+    const uint32_t rem = m & 0x1fffu;
+    if (rem > 0x1000u || (rem == 0x1000u && (q & 1u))) q++;
+    return (uint16_t)(sign | q);
+  }
+}
+
+float oracle_f16_bits_to_f32(uint16_t h) {
+  const uint32_t sign = ((uint32_t)h & 0x8000u) << 16;
+  const uint32_t e = (h >> 10) & 0x1fu;
+  const uint32_t m = h & 0x3ffu;
+  if (e == 0x1fu) return u2f(sign | 0x7f800000u | (m << 13));
+  if (e == 0) {
+    if (m == 0) return u2f(sign);
+    /* subnormal: m * 2^-24 */
+    float v = (float)m * 5.9604644775390625e-08f;
+    return (sign ? -v : v);
+  }
+  return u2f(sign | ((e + 112u) << 23) | (m << 13));
+}
+
+/* IEEE binary32 -> bfloat16, round-to-nearest-even. */
+uint16_t oracle_f32_to_bf16_bits(float f) {
+  const uint32_t x = f2u(f);
+  if ((x & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((x >> 16) | 0x0040u);
+  const uint32_t lsb = (x >> 16) & 1u;
+  return (uint16_t)((x + 0x7fffu + lsb) >> 16);
+}
+
+float oracle_bf16_bits_to_f32(uint16_t h) { return u2f((uint32_t)h << 16); }
+
+static inline float rn_f16(float a) {
+  return oracle_f16_bits_to_f32(oracle_f32_to_f16_bits(a));
+}
+static inline float rn_bf16(float a) {
+  return oracle_bf16_bits_to_f32(oracle_f32_to_bf16_bits(a));
+}
+
+/* vectorised helpers for the tests */
+void oracle_f32_to_f16_bits_array(const float *src, uint16_t *dst, size_t n) {
+  for (size_t i = 0; i < n; i++) dst[i] = oracle_f32_to_f16_bits(src[i]);
+}
+void oracle_f32_to_bf16_bits_array(const float *src, uint16_t *dst, size_t n) {
+  for (size_t i = 0; i < n; i++) dst[i] = oracle_f32_to_bf16_bits(src[i]);
+}
+
+/* ---------------------------------------------------------------- the split */
+
+/* hi = fp16(a), lo = fp16((a - hi) * 2^11); both returned widened to FP32. */
+void oracle_split_fp16(const float *a, float *hi, float *lo, size_t n) {
+  for (size_t i = 0; i < n; i++) {
+    const float h = rn_f16(a[i]);
+    hi[i] = h;
+    lo[i] = rn_f16((a[i] - h) * 2048.0f);
+  }
+}
+
+/* a ~= b0 + b1 + b2, each a bfloat16 (RN), residuals exact in FP32. */
+void oracle_split_bf16x3(const float *a, float *b0, float *b1, float *b2,
+                         size_t n) {
+  for (size_t i = 0; i < n; i++) {
+    const float h0 = rn_bf16(a[i]);
+    const float r1 = a[i] - h0;
+    const float h1 = rn_bf16(r1);
+    const float r2 = r1 - h1;
+    b0[i] = h0;
+    b1[i] = h1;
+    b2[i] = rn_bf16(r2);
+  }
+}
+
+/* ---------------------------------------------------------------- GEMM */
+
+/* Gather op(X) (rows x cols, logical) into a dense column-major real plane.
+ * X is column-major with leading dimension ld; elements are `ncomp` floats
+ * (1 real, 2 complex); `comp` selects re/im; conj negates im (OP_C,
+ * reference: src/dmem_accessor.hpp:122-123; for real data OP_C == OP_T,
+ * src/cumpsgemm.cu:48-50). */
+static void gather_plane(float *dst, const float *x, int op, size_t rows,
+                         size_t cols, size_t ld, int ncomp, int comp) {
+  const float sgn = (op == ORACLE_OP_C && comp == 1) ? -1.0f : 1.0f;
+  for (size_t c = 0; c < cols; c++) {
+    for (size_t r = 0; r < rows; r++) {
+      const size_t idx = (op == ORACLE_OP_N) ? (r + c * ld) : (c + r * ld);
+      dst[r + c * rows] = sgn * x[idx * ncomp + comp];
+    }
+  }
+}
+
+typedef struct {
+  int nterms;       /* number of split planes per operand */
+  float *p[3];      /* planes, each rows*cols, column-major */
+} planes_t;
+
+static void split_planes(planes_t *pl, const float *dense, size_t count,
+                         int mode) {
+  pl->nterms = 0;
+  pl->p[0] = pl->p[1] = pl->p[2] = NULL;
+  switch (mode) {
+  case ORACLE_MODE_FP16TCEC:
+    pl->nterms = 2;
+    pl->p[0] = (float *)malloc(count * sizeof(float));
+    pl->p[1] = (float *)malloc(count * sizeof(float));
+    oracle_split_fp16(dense, pl->p[0], pl->p[1], count);
+    break;
+  case ORACLE_MODE_FP16TC:
+    pl->nterms = 1;
+    pl->p[0] = (float *)malloc(count * sizeof(float));
+    for (size_t i = 0; i < count; i++) pl->p[0][i] = rn_f16(dense[i]);
+    break;
+  case ORACLE_MODE_TF32TCEC:
+  case ORACLE_MODE_TF32TC:
+    pl->nterms = 3;
+    pl->p[0] = (float *)malloc(count * sizeof(float));
+    pl->p[1] = (float *)malloc(count * sizeof(float));
+    pl->p[2] = (float *)malloc(count * sizeof(float));
+    oracle_split_bf16x3(dense, pl->p[0], pl->p[1], pl->p[2], count);
+    if (mode == ORACLE_MODE_TF32TC) { /* bf16x2: third term unused */
+      pl->nterms = 2;
+    }
+    break;
+  default: /* FP32 */
+    pl->nterms = 1;
+    pl->p[0] = (float *)malloc(count * sizeof(float));
+    memcpy(pl->p[0], dense, count * sizeof(float));
+    break;
+  }
+}
+
+static void free_planes(planes_t *pl) {
+  for (int i = 0; i < 3; i++) free(pl->p[i]);
+}
+
+/* acc[0..m) (+)= sign * sum_k a[:,k] * b[k]  in FP32, sequential in k.
+ * Products of two fp16/bf16-valued floats are exact in FP32, so a fused
+ * multiply-add and a separate multiply+add give identical bits. */
+static void axpy_cols(float *acc, const float *a, const float *bcol, size_t m,
+                      size_t k, float sign) {
+  for (size_t p = 0; p < k; p++) {
+    const float b = sign * bcol[p];
+    const float *ap = a + p * m;
+    for (size_t i = 0; i < m; i++) acc[i] += ap[i] * b;
+  }
+}
+
+/* One real product op(A) (m x k planes) times op(B) (k x n planes) into
+ * main/corr accumulators for output column j. */
+static void real_product_col(float *main_acc, float *corr_acc,
+                             const planes_t *A, const planes_t *B, size_t m,
+                             size_t k, size_t j, int mode, float sign) {
+  const size_t bo = j * k;
+  switch (mode) {
+  case ORACLE_MODE_FP16TCEC:
+    axpy_cols(main_acc, A->p[0], B->p[0] + bo, m, k, sign); /* hi*hi */
+    axpy_cols(corr_acc, A->p[1], B->p[0] + bo, m, k, sign); /* lo*hi */
+    axpy_cols(corr_acc, A->p[0], B->p[1] + bo, m, k, sign); /* hi*lo */
+    break;
+  case ORACLE_MODE_TF32TCEC: /* bf16x3: all terms with i+j <= 2 */
+    axpy_cols(main_acc, A->p[0], B->p[0] + bo, m, k, sign);
+    axpy_cols(corr_acc, A->p[2], B->p[0] + bo, m, k, sign);
+    axpy_cols(corr_acc, A->p[0], B->p[2] + bo, m, k, sign);
+    axpy_cols(corr_acc, A->p[1], B->p[1] + bo, m, k, sign);
+    axpy_cols(corr_acc, A->p[1], B->p[0] + bo, m, k, sign);
+    axpy_cols(corr_acc, A->p[0], B->p[1] + bo, m, k, sign);
+    break;
+  case ORACLE_MODE_TF32TC: /* bf16x2: b0*b0 + b0*b1 + b1*b0 */
+    axpy_cols(main_acc, A->p[0], B->p[0] + bo, m, k, sign);
+    axpy_cols(corr_acc, A->p[1], B->p[0] + bo, m, k, sign);
+    axpy_cols(corr_acc, A->p[0], B->p[1] + bo, m, k, sign);
+    break;
+  default: /* FP16TC, FP32 */
+    axpy_cols(main_acc, A->p[0], B->p[0] + bo, m, k, sign);
+    break;
+  }
+}
+
+static inline float corr_scale(int mode) {
+  return (mode == ORACLE_MODE_FP16TCEC) ? (1.0f / 2048.0f) : 1.0f;
+}
+
+/* C = alpha * op(A) op(B) + beta * C, column-major, emulating `mode`.
+ * Epilogue as the reference: beta == 0 -> C = acc*alpha and C is never read
+ * (src/dmem_accessor.hpp:281-315), else C = acc*alpha + beta*C (:192-198). */
+void oracle_sgemm(int mode, int op_a, int op_b, size_t m, size_t n, size_t k,
+                  float alpha, const float *a, size_t lda, const float *b,
+                  size_t ldb, float beta, float *c, size_t ldc) {
+  float *da = (float *)malloc(m * k * sizeof(float));
+  float *db = (float *)malloc(k * n * sizeof(float));
+  gather_plane(da, a, op_a == ORACLE_OP_C ? ORACLE_OP_T : op_a, m, k, lda, 1, 0);
+  gather_plane(db, b, op_b == ORACLE_OP_C ? ORACLE_OP_T : op_b, k, n, ldb, 1, 0);
+  planes_t A, B;
+  split_planes(&A, da, m * k, mode);
+  split_planes(&B, db, k * n, mode);
+  free(da);
+  free(db);
+  const float cs = corr_scale(mode);
+#pragma omp parallel
+  {
+    float *main_acc = (float *)malloc(m * sizeof(float));
+    float *corr_acc = (float *)malloc(m * sizeof(float));
+#pragma omp for schedule(static)
+    for (long j = 0; j < (long)n; j++) {
+      memset(main_acc, 0, m * sizeof(float));
+      memset(corr_acc, 0, m * sizeof(float));
+      real_product_col(main_acc, corr_acc, &A, &B, m, k, (size_t)j, mode, 1.0f);
+      for (size_t i = 0; i < m; i++) {
+        const float acc = main_acc[i] + corr_acc[i] * cs;
+        float *cp = c + i + (size_t)j * ldc;
+        if (beta == 0.0f)
+          *cp = acc * alpha;
+        else
+          *cp = acc * alpha + beta * (*cp);
+      }
+    }
+    free(main_acc);
+    free(corr_acc);
+  }
+  free_planes(&A);
+  free_planes(&B);
+}
+
+/* Complex GEMM by the 4-real-product decomposition
+ *   re = ar*br - ai*bi,  im = ar*bi + ai*br,
+ * each real product split-and-corrected on its own.  Data is interleaved
+ * (re, im) float pairs; ld* are in complex elements.  alpha/beta are
+ * {re, im}.  Epilogue: src/device_common.hpp:47-67. */
+void oracle_cgemm(int mode, int op_a, int op_b, size_t m, size_t n, size_t k,
+                  const float *alpha, const float *a, size_t lda,
+                  const float *b, size_t ldb, const float *beta, float *c,
+                  size_t ldc) {
+  float *tmp = (float *)malloc((m * k > k * n ? m * k : k * n) * sizeof(float));
+  planes_t Ar, Ai, Br, Bi;
+  gather_plane(tmp, a, op_a, m, k, lda, 2, 0);
+  split_planes(&Ar, tmp, m * k, mode);
+  gather_plane(tmp, a, op_a, m, k, lda, 2, 1);
+  split_planes(&Ai, tmp, m * k, mode);
+  gather_plane(tmp, b, op_b, k, n, ldb, 2, 0);
+  split_planes(&Br, tmp, k * n, mode);
+  gather_plane(tmp, b, op_b, k, n, ldb, 2, 1);
+  split_planes(&Bi, tmp, k * n, mode);
+  free(tmp);
+  const float cs = corr_scale(mode);
+  const int beta_zero = (beta[0] == 0.0f && beta[1] == 0.0f);
+#pragma omp parallel
+  {
+    float *acc = (float *)malloc(4 * m * sizeof(float));
+    float *re_m = acc, *re_c = acc + m, *im_m = acc + 2 * m, *im_c = acc + 3 * m;
+#pragma omp for schedule(static)
+    for (long j = 0; j < (long)n; j++) {
+      memset(acc, 0, 4 * m * sizeof(float));
+      real_product_col(re_m, re_c, &Ar, &Br, m, k, (size_t)j, mode, 1.0f);
+      real_product_col(re_m, re_c, &Ai, &Bi, m, k, (size_t)j, mode, -1.0f);
+      real_product_col(im_m, im_c, &Ar, &Bi, m, k, (size_t)j, mode, 1.0f);
+      real_product_col(im_m, im_c, &Ai, &Br, m, k, (size_t)j, mode, 1.0f);
+      for (size_t i = 0; i < m; i++) {
+        const float x = re_m[i] + re_c[i] * cs;
+        const float y = im_m[i] + im_c[i] * cs;
+        float *cp = c + 2 * (i + (size_t)j * ldc);
+        /* mul(a, alpha) = (a.x*al.x - a.y*al.y, a.y*al.x + a.x*al.y) */
+        float rx = x * alpha[0] - y * alpha[1];
+        float ry = y * alpha[0] + x * alpha[1];
+        if (!beta_zero) {
+          /* mad(v, alpha, mul(beta, c)) */
+          const float bx = beta[0] * cp[0] - beta[1] * cp[1];
+          const float by = beta[1] * cp[0] + beta[0] * cp[1];
+          rx = x * alpha[0] - y * alpha[1] + bx;
+          ry = y * alpha[0] + x * alpha[1] + by;
+        }
+        cp[0] = rx;
+        cp[1] = ry;
+      }
+    }
+    free(acc);
+  }
+  free_planes(&Ar);
+  free_planes(&Ai);
+  free_planes(&Br);
+  free_planes(&Bi);
+}
+
+/* FP64 reference GEMM of the same FP32 inputs (the harness's
+ * calc_matmul_residual_kernel, test/main.cu:153-202). ncomp = 1 or 2.
+ * Result is double (ncomp doubles per element), dense ld = m. */
+void oracle_gemm_fp64(int ncomp, int op_a, int op_b, size_t m, size_t n,
+                      size_t k, const double *alpha, const float *a, size_t lda,
+                      const float *b, size_t ldb, const double *beta,
+                      const float *c, size_t ldc, double *out) {
+  double *ar = (double *)malloc(m * k * sizeof(double));
+  double *ai = ncomp == 2 ? (double *)malloc(m * k * sizeof(double)) : NULL;
+  double *br = (double *)malloc(k * n * sizeof(double));
+  double *bi = ncomp == 2 ? (double *)malloc(k * n * sizeof(double)) : NULL;
+  float *tmp = (float *)malloc((m * k > k * n ? m * k : k * n) * sizeof(float));
+  const int oa = (ncomp == 1 && op_a == ORACLE_OP_C) ? ORACLE_OP_T : op_a;
+  const int ob = (ncomp == 1 && op_b == ORACLE_OP_C) ? ORACLE_OP_T : op_b;
+  gather_plane(tmp, a, oa, m, k, lda, ncomp, 0);
+  for (size_t i = 0; i < m * k; i++) ar[i] = tmp[i];
+  gather_plane(tmp, b, ob, k, n, ldb, ncomp, 0);
+  for (size_t i = 0; i < k * n; i++) br[i] = tmp[i];
+  if (ncomp == 2) {
+    gather_plane(tmp, a, oa, m, k, lda, ncomp, 1);
+    for (size_t i = 0; i < m * k; i++) ai[i] = tmp[i];
+    gather_plane(tmp, b, ob, k, n, ldb, ncomp, 1);
+    for (size_t i = 0; i < k * n; i++) bi[i] = tmp[i];
+  }
+  free(tmp);
+#pragma omp parallel
+  {
+    double *re = (double *)malloc(2 * m * sizeof(double));
+    double *im = re + m;
+#pragma omp for schedule(static)
+    for (long j = 0; j < (long)n; j++) {
+      for (size_t i = 0; i < 2 * m; i++) re[i] = 0.0;
+      for (size_t p = 0; p < k; p++) {
+        const double bre = br[p + (size_t)j * k];
+        const double *arp = ar + p * m;
+        if (ncomp == 1) {
+          for (size_t i = 0; i < m; i++) re[i] += arp[i] * bre;
+        } else {
+          const double bim = bi[p + (size_t)j * k];
+          const double *aip = ai + p * m;
+          for (size_t i = 0; i < m; i++) {
+            re[i] += arp[i] * bre - aip[i] * bim;
+            im[i] += arp[i] * bim + aip[i] * bre;
+          }
+        }
+      }
+      for (size_t i = 0; i < m; i++) {
+        double *op = out + ncomp * (i + (size_t)j * m);
+        if (ncomp == 1) {
+          double v = re[i] * alpha[0];
+          if (beta[0] != 0.0 && c) v += beta[0] * (double)c[i + (size_t)j * ldc];
+          op[0] = v;
+        } else {
+          double vx = re[i] * alpha[0] - im[i] * alpha[1];
+          double vy = im[i] * alpha[0] + re[i] * alpha[1];
+          if ((beta[0] != 0.0 || beta[1] != 0.0) && c) {
+            const double cx = c[2 * (i + (size_t)j * ldc)];
+            const double cy = c[2 * (i + (size_t)j * ldc) + 1];
+            vx += beta[0] * cx - beta[1] * cy;
+            vy += beta[1] * cx + beta[0] * cy;
+          }
+          op[0] = vx;
+          op[1] = vy;
+        }
+      }
+    }
+    free(re);
+  }
+  free(ar);
+  free(ai);
+  free(br);
+  free(bi);
+}
+
+/* relative Frobenius residual sqrt(sum|ref-c|^2 / sum|ref|^2)
+ * (test/main.cu:196-228). `ref` dense (ld = m), c with ldc; ncomp floats. */
+double oracle_residual(int ncomp, size_t m, size_t n, const double *ref,
+                       const float *c, size_t ldc) {
+  double base = 0.0, diff = 0.0;
+  for (size_t j = 0; j < n; j++) {
+    for (size_t i = 0; i < m; i++) {
+      for (int q = 0; q < ncomp; q++) {
+        const double r = ref[ncomp * (i + j * m) + q];
+        const double d = r - (double)c[ncomp * (i + j * ldc) + q];
+        base += r * r;
+        diff += d * d;
+      }
+    }
+  }
+  return sqrt(diff / base);
+}
+
+/* ---------------------------------------------------------------- exp stats */
+
+typedef struct {
+  uint32_t max_exp_bits; /* bits(maxabs) & 0x7f800000 */
+  uint64_t total;
+  uint64_t underflow;
+  int mode; /* decision: 1 FP16TCEC, 2 TF32TCEC, 11 FP16TCEC_SCALING */
+  int stage2_ran;
+} oracle_exp_stats_t;
+
+#define MODE_FP16TCEC 1
+#define MODE_TF32TCEC 2
+#define MODE_UNDEFINED 10
+#define MODE_FP16TCEC_SCALING 11
+
+/* fmaxf semantics of the device max: NaN operands are ignored. */
+static inline float max_ignore_nan(float a, float b) {
+  if (a != a) return b;
+  if (b != b) return a;
+  return a > b ? a : b;
+}
+
+static void count_pass(const float *ptr, size_t m, size_t n, size_t ld,
+                       size_t batch, size_t stride, int ncomp, float ignore_thr,
+                       float underflow_thr, float *maxabs, uint64_t *total,
+                       uint64_t *under) {
+  /* stride == 0 -> only the first matrix is scanned (src/exp_stats.cu:306) */
+  const size_t nb = (stride == 0) ? 1 : batch;
+  float mx = 0.0f;
+  uint64_t t = 0, u = 0;
+  for (size_t b = 0; b < nb; b++) {
+    const float *mat = ptr + b * stride * ncomp;
+    for (size_t j = 0; j < n; j++) {
+      for (size_t i = 0; i < m; i++) {
+        for (int q = 0; q < ncomp; q++) {
+          const float a = fabsf(mat[(i + j * ld) * ncomp + q]);
+          mx = max_ignore_nan(mx, a);
+          if (a >= ignore_thr) { /* src/exp_stats.cu:40-52 */
+            t++;
+            if (a < underflow_thr) u++;
+          }
+        }
+      }
+    }
+  }
+  *maxabs = mx;
+  *total = t;
+  *under = u;
+}
+
+/* Two-stage statistics + decision (src/exp_stats.cu:74-293, launch arguments
+ * :340-361).  ncomp = 1 float, 2 complex (re and im counted separately,
+ * maximum over max(|re|,|im|), :33-35, :54-62). */
+void oracle_exp_stats(const float *ptr, size_t m, size_t n, size_t ld,
+                      size_t batch, size_t stride, int ncomp, float ignore_thr,
+                      float underflow_thr, float tolerance,
+                      oracle_exp_stats_t *out) {
+  float mx;
+  uint64_t t, u;
+  count_pass(ptr, m, n, ld, batch, stride, ncomp, ignore_thr, underflow_thr, &mx,
+             &t, &u);
+  const uint32_t bits = f2u(mx) & 0x7f800000u;
+  const float max_exp = u2f(bits);
+  out->max_exp_bits = bits;
+  out->stage2_ran = 0;
+  /* decision 1 (src/exp_stats.cu:175-183); the u64 counters are converted to
+   * float by the usual arithmetic conversions */
+  if (((float)u > (float)t * tolerance) || (max_exp > 0.0f && t == 0)) {
+    out->mode = MODE_UNDEFINED;
+    t = 0;
+    u = 0;
+  } else {
+    out->mode = MODE_FP16TCEC;
+  }
+  if (out->mode == MODE_UNDEFINED) {
+    const float it = (ignore_thr / 2) * max_exp;
+    const float ut = (underflow_thr / 2) * max_exp;
+    float dummy;
+    count_pass(ptr, m, n, ld, batch, stride, ncomp, it, ut, &dummy, &t, &u);
+    out->stage2_ran = 1;
+    /* decision 2 (src/exp_stats.cu:287-292) */
+    out->mode = ((float)u <= (float)t * tolerance) ? MODE_FP16TCEC_SCALING
+                                                   : MODE_TF32TCEC;
+  }
+  out->total = t;
+  out->underflow = u;
+}
+
+/* max exponent only (src/exp_stats.cu:386-459) */
+uint32_t oracle_exp_max_bits(const float *ptr, size_t m, size_t n, size_t ld,
+                             size_t batch, size_t stride, int ncomp) {
+  float mx;
+  uint64_t t, u;
+  count_pass(ptr, m, n, ld, batch, stride, ncomp, 0.0f, 0.0f, &mx, &t, &u);
+  return f2u(mx) & 0x7f800000u;
+}
+
+/* ---------------------------------------------------------------- scaling */
+
+/* coefficients (src/dynamic_scaling.cu:15, :93, :106-121, :146) */
+float oracle_scale_ab_coef(float max_exp) { return 16384.0f / max_exp; }
+float oracle_reset_ab_coef(float max_exp) { return max_exp / 16384.0f; }
+float oracle_scale_c_coef(float max_exp_a, float max_exp_b, int use_flag,
+                          int flag) {
+  if (!use_flag) return (float)(max_exp_a * max_exp_b) / (16384.0f * 16384.0f);
+  float coef = 1.0f;
+  if (flag & 0x40) coef *= max_exp_a / 16384.0f; /* scale-A bit */
+  if (flag & 0x20) coef *= max_exp_b / 16384.0f; /* scale-B bit */
+  return coef;
+}
+
+/* in-place multiply of an m x n (ld, batch, stride) view by coef */
+void oracle_scale_matrix(float *ptr, size_t m, size_t n, size_t ld, size_t batch,
+                         size_t stride, int ncomp, float coef) {
+  const size_t nb = (stride == 0) ? 1 : batch;
+  for (size_t b = 0; b < nb; b++) {
+    float *mat = ptr + b * stride * ncomp;
+    for (size_t j = 0; j < n; j++)
+      for (size_t i = 0; i < m; i++)
+        for (int q = 0; q < ncomp; q++) mat[(i + j * ld) * ncomp + q] *= coef;
+  }
+}
+
+/* launch flag = mode (bits 0-4) | scale-B (bit 5) | scale-A (bit 6);
+ * combine rule of src/dynamic_scaling.cu:364-385 */
+int oracle_combine_flag(int mode_a, int mode_b) {
+  if (mode_a == MODE_TF32TCEC || mode_b == MODE_TF32TCEC) return MODE_TF32TCEC;
+  int flag = MODE_FP16TCEC;
+  if (mode_a == MODE_FP16TCEC_SCALING) flag |= 0x40;
+  if (mode_b == MODE_FP16TCEC_SCALING) flag |= 0x20;
+  return flag;
+}
+
+/* ring of result slots: 0 and 1 reserved, 2..len-1 cycle
+ * (src/exp_stats.cu:15-24).  Returns the new current id. */
+uint32_t oracle_next_ring_id(uint32_t current, uint32_t length) {
+  const uint32_t next = current + 1;
+  return next < length ? next : 2;
+}
