@@ -191,7 +191,8 @@ hipblasStatus_t hijack_core(const char *func_name, hipblasHandle_t hb, hipblasOp
     return HIPBLAS_STATUS_INVALID_VALUE;
   }
   const cuMpSGEMM_compute_mode_t mode = query_mode(func_name, hb, op_A, op_B, m, n, k);
-  cuMpSGEMM_handle_t h = global_handle();
+  // a dry run only logs: it must not need a device, so the handle is created after it
+  cuMpSGEMM_handle_t h = (mode == CUMPSGEMM_DRY_RUN) ? g_handle : global_handle();
 
   log_info(std::string(func_name) + " op=(" + op_str(op_A) + ", " + op_str(op_B) + "), shape=(" +
            std::to_string(m) + ", " + std::to_string(n) + ", " + std::to_string(k) + ")" +

@@ -1,0 +1,167 @@
+// Stand-alone hipBLAS client used by tests/test_gpu_hijack.py.  It is linked
+// against the real libhipblas.so; when run under LD_PRELOAD=libcumpsgemm.so the
+// six GEMM entry points below resolve to the interposer instead.  For every
+// call it prints one line:  RESULT <name> status=<s> relerr=<e>
+// where relerr is the relative Frobenius error over sampled entries of C
+// against a double-precision evaluation of the same inputs on the host.
+#include <hip/hip_complex.h>
+#include <hip/hip_runtime.h>
+#include <hipblas/hipblas.h>
+
+#include <cmath>
+#include <complex>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <vector>
+
+#define CHECK_HIP(x)                                                                      \
+  do {                                                                                    \
+    hipError_t e_ = (x);                                                                  \
+    if (e_ != hipSuccess) {                                                               \
+      std::printf("HIP error %s at %s:%d\n", hipGetErrorString(e_), __FILE__, __LINE__); \
+      std::exit(2);                                                                       \
+    }                                                                                     \
+  } while (0)
+
+static uint64_t mix(uint64_t x) {
+  x += 0x9E3779B97F4A7C15ull;
+  x = (x ^ (x >> 30)) * 0xBF58476D1CE4E5B9ull;
+  x = (x ^ (x >> 27)) * 0x94D049BB133111EBull;
+  return x ^ (x >> 31);
+}
+static float unif(uint64_t seed, uint64_t i) {
+  return (float)((double)(mix(seed * 0x100000000ull + i) >> 40) / (1 << 24) * 2.0 - 1.0);
+}
+
+template <class T> struct dev_buf {
+  T *p = nullptr;
+  explicit dev_buf(size_t n) { CHECK_HIP(hipMalloc(&p, n * sizeof(T))); }
+  ~dev_buf() { (void)hipFree(p); }
+};
+
+static void report(const char *name, hipblasStatus_t st, double num, double den) {
+  std::printf("RESULT %s status=%d relerr=%.3e\n", name, (int)st, std::sqrt(num / (den > 0 ? den : 1)));
+  std::fflush(stdout);
+}
+
+int main(int argc, char **argv) {
+  const int n = (argc > 1) ? std::atoi(argv[1]) : 1280; // > 1024 so the default rule engages
+  const int batch = 3;
+  hipblasHandle_t hb;
+  if (hipblasCreate(&hb) != HIPBLAS_STATUS_SUCCESS) {
+    std::printf("hipblasCreate failed\n");
+    return 2;
+  }
+  hipStream_t stream;
+  CHECK_HIP(hipStreamCreate(&stream));
+  hipblasSetStream(hb, stream);
+
+  const size_t e = (size_t)n * n;
+  std::vector<float> ha(e * batch), hb_(e * batch), hc(e * batch);
+  for (size_t i = 0; i < e * batch; i++) {
+    ha[i] = unif(1, i);
+    hb_[i] = unif(2, i);
+  }
+  dev_buf<float> da(e * batch), db(e * batch), dc(e * batch);
+  CHECK_HIP(hipMemcpyAsync(da.p, ha.data(), e * batch * 4, hipMemcpyHostToDevice, stream));
+  CHECK_HIP(hipMemcpyAsync(db.p, hb_.data(), e * batch * 4, hipMemcpyHostToDevice, stream));
+  const float one = 1.0f, zero = 0.0f;
+
+  auto check_real = [&](const char *name, hipblasStatus_t st, int nb, bool trans_a) {
+    CHECK_HIP(hipMemcpyAsync(hc.data(), dc.p, e * nb * 4, hipMemcpyDeviceToHost, stream));
+    CHECK_HIP(hipStreamSynchronize(stream));
+    double num = 0, den = 0;
+    for (int b = 0; b < nb; b++)
+      for (int s = 0; s < 400; s++) {
+        const int i = (int)(mix(s * 2 + 11) % n), j = (int)(mix(s * 2 + 12) % n);
+        double ref = 0;
+        for (int p = 0; p < n; p++) {
+          const double av = trans_a ? ha[b * e + p + (size_t)i * n] : ha[b * e + i + (size_t)p * n];
+          ref += av * (double)hb_[b * e + p + (size_t)j * n];
+        }
+        const double d = ref - (double)hc[b * e + i + (size_t)j * n];
+        num += d * d;
+        den += ref * ref;
+      }
+    report(name, st, num, den);
+  };
+
+  CHECK_HIP(hipMemsetAsync(dc.p, 0, e * batch * 4, stream));
+  hipblasStatus_t st = hipblasSgemm(hb, HIPBLAS_OP_N, HIPBLAS_OP_N, n, n, n, &one, da.p, n, db.p, n, &zero, dc.p, n);
+  check_real("hipblasSgemm", st, 1, false);
+
+  CHECK_HIP(hipMemsetAsync(dc.p, 0, e * batch * 4, stream));
+  st = hipblasSgemm(hb, HIPBLAS_OP_T, HIPBLAS_OP_N, n, n, n, &one, da.p, n, db.p, n, &zero, dc.p, n);
+  check_real("hipblasSgemm_TN", st, 1, true);
+
+  CHECK_HIP(hipMemsetAsync(dc.p, 0, e * batch * 4, stream));
+  st = hipblasSgemmStridedBatched(hb, HIPBLAS_OP_N, HIPBLAS_OP_N, n, n, n, &one, da.p, n, (long long)e, db.p, n,
+                                  (long long)e, &zero, dc.p, n, (long long)e, batch);
+  check_real("hipblasSgemmStridedBatched", st, batch, false);
+
+  CHECK_HIP(hipMemsetAsync(dc.p, 0, e * batch * 4, stream));
+  st = hipblasGemmEx(hb, HIPBLAS_OP_N, HIPBLAS_OP_N, n, n, n, &one, da.p, HIP_R_32F, n, db.p, HIP_R_32F, n, &zero,
+                     dc.p, HIP_R_32F, n, HIPBLAS_COMPUTE_32F, HIPBLAS_GEMM_DEFAULT);
+  check_real("hipblasGemmEx_f32", st, 1, false);
+
+  CHECK_HIP(hipMemsetAsync(dc.p, 0, e * batch * 4, stream));
+  st = hipblasGemmStridedBatchedEx(hb, HIPBLAS_OP_N, HIPBLAS_OP_N, n, n, n, &one, da.p, HIP_R_32F, n, (long long)e,
+                                   db.p, HIP_R_32F, n, (long long)e, &zero, dc.p, HIP_R_32F, n, (long long)e, batch,
+                                   HIPBLAS_COMPUTE_32F, HIPBLAS_GEMM_DEFAULT);
+  check_real("hipblasGemmStridedBatchedEx_f32", st, batch, false);
+
+  // zero-sized call: the interposer answers INVALID_VALUE, hipBLAS succeeds quietly
+  st = hipblasSgemm(hb, HIPBLAS_OP_N, HIPBLAS_OP_N, 0, n, n, &one, da.p, n, db.p, n, &zero, dc.p, n);
+  std::printf("RESULT zero_m status=%d relerr=0\n", (int)st);
+
+  // complex: the float buffers reinterpreted as n/2-column complex matrices
+  {
+    const int nc = n / 2; // complex matrices are n x nc? keep them square: nc x nc
+    const hipComplex cone = make_hipComplex(1.f, 0.f), czero = make_hipComplex(0.f, 0.f);
+    const hipComplex *ca = reinterpret_cast<const hipComplex *>(da.p);
+    const hipComplex *cb = reinterpret_cast<const hipComplex *>(db.p);
+    hipComplex *cc = reinterpret_cast<hipComplex *>(dc.p);
+    CHECK_HIP(hipMemsetAsync(dc.p, 0, e * batch * 4, stream));
+    st = hipblasCgemm(hb, HIPBLAS_OP_C, HIPBLAS_OP_N, nc, nc, nc, &cone, ca, nc, cb, nc, &czero, cc, nc);
+    CHECK_HIP(hipMemcpyAsync(hc.data(), dc.p, (size_t)nc * nc * 8, hipMemcpyDeviceToHost, stream));
+    CHECK_HIP(hipStreamSynchronize(stream));
+    auto A = reinterpret_cast<const std::complex<float> *>(ha.data());
+    auto B = reinterpret_cast<const std::complex<float> *>(hb_.data());
+    auto Cc = reinterpret_cast<const std::complex<float> *>(hc.data());
+    double num = 0, den = 0;
+    for (int s = 0; s < 400; s++) {
+      const int i = (int)(mix(s * 2 + 31) % nc), j = (int)(mix(s * 2 + 32) % nc);
+      std::complex<double> ref = 0;
+      for (int p = 0; p < nc; p++)
+        ref += std::conj(std::complex<double>(A[p + (size_t)i * nc])) * std::complex<double>(B[p + (size_t)j * nc]);
+      num += std::norm(ref - std::complex<double>(Cc[i + (size_t)j * nc]));
+      den += std::norm(ref);
+    }
+    report("hipblasCgemm_CN", st, num, den);
+  }
+
+  // a non-FP32 GemmEx must go to hipBLAS untouched whatever the mode
+  {
+    std::vector<uint16_t> h16(e, 0x3c00 /* 1.0 */);
+    dev_buf<uint16_t> a16(e), b16(e);
+    CHECK_HIP(hipMemcpyAsync(a16.p, h16.data(), e * 2, hipMemcpyHostToDevice, stream));
+    CHECK_HIP(hipMemcpyAsync(b16.p, h16.data(), e * 2, hipMemcpyHostToDevice, stream));
+    CHECK_HIP(hipMemsetAsync(dc.p, 0, e * 4, stream));
+    st = hipblasGemmEx(hb, HIPBLAS_OP_N, HIPBLAS_OP_N, n, n, n, &one, a16.p, HIP_R_16F, n, b16.p, HIP_R_16F, n, &zero,
+                       dc.p, HIP_R_32F, n, HIPBLAS_COMPUTE_32F, HIPBLAS_GEMM_DEFAULT);
+    CHECK_HIP(hipMemcpyAsync(hc.data(), dc.p, e * 4, hipMemcpyDeviceToHost, stream));
+    CHECK_HIP(hipStreamSynchronize(stream));
+    double num = 0, den = 0;
+    for (size_t i = 0; i < e; i += 997) {
+      num += ((double)hc[i] - n) * ((double)hc[i] - n);
+      den += (double)n * n;
+    }
+    report("hipblasGemmEx_f16_in", st, num, den);
+  }
+
+  hipblasDestroy(hb);
+  CHECK_HIP(hipStreamDestroy(stream));
+  std::printf("DONE\n");
+  return 0;
+}

@@ -1,0 +1,180 @@
+"""Parity of the HIP GEMM path (through the C ABI) with the oracle.
+
+Tolerances (floating point, stated by the task): relative Frobenius error of
+the error-corrected modes against an FP64 GEMM of the same inputs must be
+within 2x of a plain FP32 SGEMM's error and below the reference's own bar
+2^-23*sqrt(K) (test/main.cu:68-74); the uncorrected modes below 2^-10*sqrt(K).
+Cases whose result is exactly representable must match the oracle bit for bit.
+"""
+import numpy as np
+import pytest
+
+from cumpsgemm_amd import inputs
+from gpu_util import N, T, C, make_operand, oracle_gemm, rel_diff, run_gemm
+
+pytestmark = pytest.mark.gpu
+
+FP16TCEC, TF32TCEC, FP16TC, TF32TC, FP32 = 1, 2, 3, 4, 12
+
+
+def _gen(cplx):
+    return (lambda s, c: inputs.complex_normal(s, c, 0.6)) if cplx else inputs.uniform
+
+
+def _check(O, handle, dev, mode, opa, opb, m, n, k, cplx, alpha, beta, pads=(0, 0, 0), seed=1):
+    gen = _gen(cplx)
+    a, lda = make_operand(gen, seed, opa, m, k, pads[0])
+    b, ldb = make_operand(gen, seed + 1, opb, k, n, pads[1])
+    ldc = m + pads[2]
+    c0 = gen(seed + 2, ldc * n)
+    c, st = run_gemm(handle, dev, mode, opa, opb, m, n, k, alpha, a, lda, b, ldb, beta, c0, ldc, cplx)
+    assert st == 0
+    ref = O.gemm_fp64(opa, opb, m, n, k, alpha, a, lda, b, ldb, beta, c0, ldc)
+    r_gpu = O.residual(ref, c, m, n, ldc)
+    co = oracle_gemm(O, mode, opa, opb, m, n, k, alpha, a, lda, b, ldb, beta, c0, ldc)
+    r_oracle = O.residual(ref, co, m, n, ldc)
+    cf = oracle_gemm(O, FP32, opa, opb, m, n, k, alpha, a, lda, b, ldb, beta, c0, ldc)
+    r_fp32 = O.residual(ref, cf, m, n, ldc)
+    kk = max(k, 1)
+    if mode in (FP16TCEC, TF32TCEC):
+        # 2x the FP32 error, plus one FP32 rounding of slack for outputs so small
+        # that plain FP32 happens to be exact
+        assert r_gpu <= 2.0 * r_fp32 + 2.0 ** -23, (r_gpu, r_fp32)
+        if alpha == 1.0 and beta == 0.0:  # the conditions of the reference's own bar
+            assert r_gpu < 2.0 ** -23 * np.sqrt(kk)
+        # GPU and oracle run the same algorithm in different summation orders
+        assert rel_diff(c, co, m, n, ldc) < 2.0 ** -21 * np.sqrt(kk)
+    else:
+        assert r_gpu < 2.0 ** -10 * np.sqrt(kk)
+        assert r_gpu <= 1.5 * r_oracle + 1e-7
+    # rows between m and ldc are never written
+    if pads[2]:
+        assert np.array_equal(c.reshape(n, ldc)[:, m:], c0.reshape(n, ldc)[:, m:])
+    return r_gpu
+
+
+@pytest.mark.parametrize("mode", [FP16TCEC, TF32TCEC, FP16TC, TF32TC])
+@pytest.mark.parametrize("opa", [N, T])
+@pytest.mark.parametrize("opb", [N, T])
+def test_sgemm_aligned_all_layouts(O, handle, dev, mode, opa, opb):
+    _check(O, handle, dev, mode, opa, opb, 512, 384, 256, False, 1.0, 0.0)
+
+
+@pytest.mark.parametrize("mode", [FP16TCEC, TF32TCEC])
+@pytest.mark.parametrize("opa", [N, T])
+@pytest.mark.parametrize("opb", [N, T])
+@pytest.mark.parametrize("shape", [(131, 77, 45), (1, 1, 1), (33, 1, 7), (1, 65, 129), (257, 130, 33),
+                                   (64, 64, 1), (5, 300, 1000)])
+def test_sgemm_ragged_padded_alpha_beta(O, handle, dev, mode, opa, opb, shape):
+    m, n, k = shape
+    _check(O, handle, dev, mode, opa, opb, m, n, k, False, 1.5, -0.75, pads=(3, 5, 2))
+
+
+@pytest.mark.parametrize("mode", [FP16TCEC, TF32TCEC, FP16TC, TF32TC])
+@pytest.mark.parametrize("opa", [N, T, C])
+@pytest.mark.parametrize("opb", [N, T, C])
+def test_cgemm_all_ops(O, handle, dev, mode, opa, opb):
+    _check(O, handle, dev, mode, opa, opb, 160, 96, 200, True, 1.0 + 0.5j, 0.25 - 1.0j, pads=(1, 0, 3))
+
+
+@pytest.mark.parametrize("shape", [(96, 80, 72), (3, 2, 5), (129, 65, 31), (512, 512, 64)])
+def test_cgemm_shapes_beta_zero(O, handle, dev, shape):
+    m, n, k = shape
+    _check(O, handle, dev, FP16TCEC, N, N, m, n, k, True, 1.0, 0.0)
+    _check(O, handle, dev, TF32TCEC, C, T, m, n, k, True, -2.0j, 0.0, pads=(2, 2, 2))
+
+
+def test_op_c_on_real_data_is_transpose(O, handle, dev):
+    _check(O, handle, dev, FP16TCEC, C, C, 100, 90, 80, False, 1.0, 0.0)
+
+
+@pytest.mark.parametrize("mode", [FP16TCEC, TF32TCEC, FP16TC, TF32TC])
+@pytest.mark.parametrize("cplx", [False, True])
+def test_exact_integer_products_match_oracle_bitwise(O, handle, dev, mode, cplx):
+    rng = np.random.default_rng(7)
+    m, n, k = 150, 70, 333
+    def ints(count):
+        v = rng.integers(-60, 61, count).astype(np.float32)
+        if cplx:
+            v = (v + 1j * rng.integers(-60, 61, count).astype(np.float32)).astype(np.complex64)
+        return v
+    for opa, opb in ((N, N), (T, N), (N, T), (C, C)):
+        a, b, c0 = ints(m * k), ints(k * n), ints(m * n)
+        lda = m if opa == N else k
+        ldb = k if opb == N else n
+        c, st = run_gemm(handle, dev, mode, opa, opb, m, n, k, 2.0, a, lda, b, ldb, -1.0, c0, m, cplx)
+        co = oracle_gemm(O, mode, opa, opb, m, n, k, 2.0, a, lda, b, ldb, -1.0, c0, m)
+        assert st == 0 and np.array_equal(c, co)
+
+
+def test_subnormal_fp16_terms_are_kept(O, handle, dev):
+    """hi values below 2^-14 are fp16 subnormals; they must not be flushed by the
+    conversion or by the matrix unit: powers of two give an exact result."""
+    m = n = k = 64
+    a = np.full(m * k, 2.0 ** -20, dtype=np.float32)
+    b = np.full(k * n, 2.0 ** -3, dtype=np.float32)
+    c, st = run_gemm(handle, dev, FP16TCEC, N, N, m, n, k, 1.0, a, m, b, k, 0.0, np.zeros(m * n, np.float32), m, False)
+    assert np.array_equal(c, np.full(m * n, k * 2.0 ** -23, dtype=np.float32))
+
+
+def test_beta_zero_ignores_nan_in_c(O, handle, dev):
+    m = n = k = 96
+    a, b = inputs.uniform(1, m * k), inputs.uniform(2, k * n)
+    c0 = np.full(m * n, np.nan, dtype=np.float32)
+    c, st = run_gemm(handle, dev, FP16TCEC, N, N, m, n, k, 1.0, a, m, b, k, 0.0, c0, m, False)
+    assert np.isfinite(c).all()
+
+
+def test_split_k_path_small_output_long_k(O, handle, dev):
+    m, n, k = 64, 48, 8192
+    a, b = inputs.uniform(3, m * k), inputs.uniform(4, k * n)
+    c0 = inputs.uniform(5, m * n)
+    c, st, mid = run_gemm(handle, dev, FP16TCEC, N, N, m, n, k, 1.25, a, m, b, k, 0.5, c0, m, False, want_module_id=True)
+    assert st == 0 and mid >= 100  # split-K took over
+    ref = O.gemm_fp64(N, N, m, n, k, 1.25, a, m, b, k, 0.5, c0, m)
+    cf = oracle_gemm(O, FP32, N, N, m, n, k, 1.25, a, m, b, k, 0.5, c0, m)
+    assert O.residual(ref, c, m, n, m) <= 2.0 * O.residual(ref, cf, m, n, m)
+
+
+@pytest.mark.parametrize("cplx", [False, True])
+def test_strided_batch(O, handle, dev, cplx):
+    m, n, k, batch = 70, 50, 90, 5
+    gen = _gen(cplx)
+    lda, ldb, ldc = m + 2, k, m + 1
+    sa, sb, sc = lda * k + 7, ldb * n, ldc * n + 3
+    a, b, c0 = gen(1, sa * batch), gen(2, sb * batch), gen(3, sc * batch)
+    da, db, dc = dev.up(a), dev.up(b), dev.up(c0)
+    st = handle.gemm_strided_batch(N, N, m, n, k, 1.0, da, lda, sa, db, ldb, sb, 0.5, dc, ldc, sc, batch,
+                                   FP16TCEC, cplx=cplx)
+    assert st == 0
+    c = dev.down(dc, np.complex64 if cplx else np.float32)
+    for i in range(batch):
+        ai, bi, ci0 = a[i * sa:], b[i * sb:], c0[i * sc: i * sc + ldc * n]
+        ref = O.gemm_fp64(N, N, m, n, k, 1.0, ai, lda, bi, ldb, 0.5, ci0, ldc)
+        cf = oracle_gemm(O, FP32, N, N, m, n, k, 1.0, ai, lda, bi, ldb, 0.5, ci0, ldc)
+        got = c[i * sc: i * sc + ldc * n]
+        assert O.residual(ref, got, m, n, ldc) <= 2.0 * O.residual(ref, cf, m, n, ldc)
+    # gaps between batch entries are untouched
+    assert np.array_equal(c[ldc * n: sc], c0[ldc * n: sc])
+
+
+def test_c1_config_1024_cubed(O, handle, dev):
+    """BASELINE config 1: SGEMM NN 1024^3, uniform[-1,1], seeds (1,2)."""
+    m = n = k = 1024
+    a, b = inputs.uniform(1, m * k), inputs.uniform(2, k * n)
+    for mode in (FP16TCEC, TF32TCEC):
+        c, st = run_gemm(handle, dev, mode, N, N, m, n, k, 1.0, a, m, b, k, 0.0, np.zeros(m * n, np.float32), m, False)
+        ref = O.gemm_fp64(N, N, m, n, k, 1.0, a, m, b, k)
+        cf = oracle_gemm(O, FP32, N, N, m, n, k, 1.0, a, m, b, k, 0.0, np.zeros(m * n, np.float32), m)
+        co = oracle_gemm(O, mode, N, N, m, n, k, 1.0, a, m, b, k, 0.0, np.zeros(m * n, np.float32), m)
+        r, rf = O.residual(ref, c, m, n, m), O.residual(ref, cf, m, n, m)
+        assert r <= 2.0 * rf and r < 2.0 ** -23 * 32
+        assert rel_diff(c, co, m, n, m) < 2.0 ** -21 * 32
+
+
+def test_invalid_arguments(handle, dev, cg):
+    x = dev.up(np.zeros(64, np.float32))
+    assert handle.gemm(N, N, 8, 8, 8, 1.0, x, 8, x, 8, 0.0, x, 8, cg.CUBLAS) == cg.STATUS_INVALID_VALUE
+    assert handle.gemm(N, N, 8, 8, 8, 1.0, x, 4, x, 8, 0.0, x, 8, cg.FP16TCEC) == cg.STATUS_INVALID_VALUE
+    assert handle.gemm(N, N, 8, 8, 8, 1.0, x, 8, x, 8, 0.0, x, 7, cg.FP16TCEC) == cg.STATUS_INVALID_VALUE
+    assert handle.gemm(N, N, 0, 8, 8, 1.0, x, 8, x, 8, 0.0, x, 8, cg.FP16TCEC) == cg.STATUS_SUCCESS

@@ -1,0 +1,82 @@
+"""LD_PRELOAD interception of hipBLAS by libcumpsgemm.so, exercised with a
+stand-alone hipBLAS client (tests/native/hijack_probe, linked against the real
+libhipblas.so).  What a drop-in user does: set CUMPSGEMM_COMPUTE_MODE and
+LD_PRELOAD (reference README.md:27-31)."""
+import os
+import re
+import subprocess
+
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+PROBE = os.path.join(ROOT, "tests", "native", "hijack_probe")
+LIB = os.path.join(ROOT, "cumpsgemm_amd", "libcumpsgemm.so")
+
+
+def _probe(env_extra, preload=True):
+    assert os.path.exists(PROBE), "build tests/native/hijack_probe first (make -C tests/native)"
+    env = dict(os.environ)
+    for k in ("CUMPSGEMM_COMPUTE_MODE", "CUMPSGEMM_INFO", "CUMPSGEMM_CUSTOM_GEMM_MX2X2"):
+        env.pop(k, None)
+    env.update(env_extra)
+    if preload:
+        env["LD_PRELOAD"] = LIB + (":" + env["LD_PRELOAD"] if env.get("LD_PRELOAD") else "")
+    r = subprocess.run([PROBE], env=env, text=True, capture_output=True, timeout=300)
+    assert r.returncode == 0 and "DONE" in r.stdout, r.stdout[-2000:] + r.stderr[-2000:]
+    res = {m.group(1): (int(m.group(2)), float(m.group(3)))
+           for m in re.finditer(r"RESULT (\S+) status=(-?\d+) relerr=(\S+)", r.stdout)}
+    logs = [l for l in r.stdout.splitlines() if l.startswith("[cuMpSGEMM")]
+    return res, logs
+
+
+FP32_CALLS = ["hipblasSgemm", "hipblasSgemm_TN", "hipblasSgemmStridedBatched", "hipblasGemmEx_f32",
+              "hipblasGemmStridedBatchedEx_f32", "hipblasCgemm_CN"]
+
+
+def test_without_preload_is_plain_hipblas():
+    res, logs = _probe({"CUMPSGEMM_COMPUTE_MODE": "FP16TC", "CUMPSGEMM_INFO": "1"}, preload=False)
+    assert not logs
+    for name in FP32_CALLS:
+        assert res[name][0] == 0 and res[name][1] < 2e-6
+    assert res["zero_m"][0] == 0
+
+
+def test_preload_fp16tcec_keeps_fp32_accuracy_and_logs_every_call():
+    base, _ = _probe({}, preload=False)
+    res, logs = _probe({"CUMPSGEMM_COMPUTE_MODE": "FP16TCEC", "CUMPSGEMM_INFO": "1"})
+    for name in FP32_CALLS:
+        assert res[name][0] == 0
+        assert res[name][1] <= 2.0 * base[name][1] + 1e-9, (name, res[name], base[name])
+    assert res["zero_m"][0] == 3  # HIPBLAS_STATUS_INVALID_VALUE from the interposer
+    assert res["hipblasGemmEx_f16_in"] == (0, 0.0)  # forwarded untouched
+    text = "\n".join(logs)
+    assert "hipblasSgemm op=(N, N), shape=(1280, 1280, 1280), mode=FP16TCEC[dynamic][exp_stats:0]" in text
+    assert "hipblasSgemm op=(T, N)" in text
+    assert "hipblasSgemmStridedBatched op=(N, N), shape=(1280, 1280, 1280), batch=3, mode=FP16TCEC" in text
+    assert "hipblasGemmEx op=(N, N)" in text and "hipblasGemmStridedBatchedEx op=(N, N)" in text
+    # the complex call is 640^3: the default rule sends small problems to hipBLAS
+    assert "hipblasCgemm op=(C, N), shape=(640, 640, 640), mode=CUBLAS_SIMT" in text
+
+
+def test_preload_uncorrected_mode_is_really_in_the_path():
+    res, _ = _probe({"CUMPSGEMM_COMPUTE_MODE": "FP16TC"})
+    for name in ("hipblasSgemm", "hipblasSgemm_TN", "hipblasSgemmStridedBatched", "hipblasGemmEx_f32"):
+        assert 1e-5 < res[name][1] < 2e-3  # fp16-level error: our kernel ran, not hipBLAS
+    assert res["hipblasCgemm_CN"][1] < 2e-6  # small problem: forwarded
+
+
+@pytest.mark.parametrize("mode", ["TF32TCEC", "FP16TCEC_SCALING", "AUTO"])
+def test_preload_other_modes(mode):
+    base, _ = _probe({}, preload=False)
+    res, logs = _probe({"CUMPSGEMM_COMPUTE_MODE": mode, "CUMPSGEMM_INFO": "1"})
+    for name in FP32_CALLS:
+        assert res[name][0] == 0 and res[name][1] <= 2.0 * base[name][1] + 1e-9
+    assert any(f"mode={mode}" in l for l in logs)
+
+
+def test_preload_dry_run_leaves_c_untouched():
+    res, logs = _probe({"CUMPSGEMM_COMPUTE_MODE": "DRY_RUN", "CUMPSGEMM_INFO": "1"})
+    assert res["hipblasSgemm"] == (0, 1.0)  # C stayed zero: relative error exactly 1
+    assert any("mode=DRY_RUN" in l for l in logs)

@@ -1,0 +1,111 @@
+"""The mode pipelines (FP16TCEC_SCALING, AUTO) end to end on the GPU: the
+statistics and flags they record, restoration of A and B, and the error of the
+result against an FP64 GEMM, next to plain FP16TCEC and plain FP32."""
+import numpy as np
+import pytest
+
+from cumpsgemm_amd import inputs
+from gpu_util import N, T, oracle_gemm
+
+pytestmark = pytest.mark.gpu
+FP16TCEC, TF32TCEC, AUTO, SCALING, FP32 = 1, 2, 9, 11, 12
+
+
+def _pipeline(handle, dev, mode, opa, opb, m, n, k, a, b, cplx=False, restore=True):
+    lda = m if opa == N else k
+    ldb = k if opb == N else n
+    da, db = dev.up(a), dev.up(b)
+    dc = dev.up(np.zeros(m * n, a.dtype))
+    st, ids = handle.gemm_pipeline(opa, opb, m, n, k, 1.0, da, lda, db, ldb, 0.0, dc, m, mode, cplx=cplx,
+                                   restore_ab=restore)
+    assert st == 0
+    dt = np.complex64 if cplx else np.float32
+    return dev.down(dc, dt), dev.down(da, dt), dev.down(db, dt), ids
+
+
+def test_scaling_rescues_tiny_inputs(O, handle, dev):
+    """Inputs ~2^-20: plain FP16TCEC loses the lo term to fp16 underflow; after
+    power-of-two scaling the result is as accurate as FP32."""
+    m = n = k = 384
+    a = (inputs.uniform(1, m * k) * np.float32(2.0 ** -20)).astype(np.float32)
+    b = (inputs.uniform(2, k * n) * np.float32(2.0 ** -18)).astype(np.float32)
+    ref = O.gemm_fp64(N, N, m, n, k, 1.0, a, m, b, k)
+    r_fp32 = O.residual(ref, oracle_gemm(O, FP32, N, N, m, n, k, 1.0, a, m, b, k, 0.0, np.zeros(m * n, np.float32), m), m, n, m)
+    c_plain, _, _, _ = _pipeline(handle, dev, FP16TCEC, N, N, m, n, k, a, b)
+    c_scaled, a_after, b_after, ids = _pipeline(handle, dev, SCALING, N, N, m, n, k, a, b)
+    r_plain, r_scaled = O.residual(ref, c_plain, m, n, m), O.residual(ref, c_scaled, m, n, m)
+    assert r_scaled <= 2.0 * r_fp32
+    assert r_plain > 50 * r_scaled  # the unscaled path visibly degrades
+    # A and B are restored bit-exactly
+    assert np.array_equal(a_after.view(np.uint32), a.view(np.uint32))
+    assert np.array_equal(b_after.view(np.uint32), b.view(np.uint32))
+    assert ids[2] == 1  # forced flag slot
+    assert int(np.float32(handle.get_max_exp(ids[0])).view(np.uint32)) == O.exp_max_bits(a, m, k, m)
+    assert int(np.float32(handle.get_max_exp(ids[1])).view(np.uint32)) == O.exp_max_bits(b, k, n, k)
+    # parity with the oracle's pipeline: scale, TCEC GEMM, unscale
+    L = O.lib()
+    ma, mb = handle.get_max_exp(ids[0]), handle.get_max_exp(ids[1])
+    sa = O.scale_matrix(a.copy(), m, k, m, L.oracle_scale_ab_coef(ma))
+    sb = O.scale_matrix(b.copy(), k, n, k, L.oracle_scale_ab_coef(mb))
+    co = oracle_gemm(O, FP16TCEC, N, N, m, n, k, 1.0, sa, m, sb, k, 0.0, np.zeros(m * n, np.float32), m)
+    O.scale_matrix(co, m, n, m, L.oracle_scale_c_coef(ma, mb, 0, 0))
+    assert np.linalg.norm(co.astype(np.float64) - c_scaled) / np.linalg.norm(co.astype(np.float64)) < 2.0 ** -21 * np.sqrt(k)
+
+
+def test_scaling_without_restore_leaves_scaled_operands(O, handle, dev):
+    m = n = k = 128
+    a = (inputs.uniform(3, m * k) * np.float32(2.0 ** -10)).astype(np.float32)
+    b = inputs.uniform(4, k * n)
+    _, a_after, b_after, ids = _pipeline(handle, dev, SCALING, T, T, m, n, k, a, b, restore=False)
+    ma = handle.get_max_exp(ids[0])
+    assert np.array_equal(a_after, O.scale_matrix(a.copy(), k, m, k, O.lib().oracle_scale_ab_coef(ma)))
+    assert 2.0 ** 14 <= np.abs(b_after).max() < 2.0 ** 15
+
+
+@pytest.mark.parametrize("case", ["unit", "tiny", "wide"])
+def test_auto_mode_decision_and_accuracy(O, handle, dev, case):
+    m = n = k = 320
+    if case == "unit":
+        a, b = inputs.uniform(5, m * k, 0.25, 1.0), inputs.uniform(6, k * n, 0.25, 1.0)
+        want_mode, want_scale = FP16TCEC, (0, 0)
+    elif case == "tiny":
+        a = (inputs.uniform(5, m * k, 0.5, 1.0) * np.float32(2.0 ** -20)).astype(np.float32)
+        b = inputs.uniform(6, k * n, 0.25, 1.0)
+        want_mode, want_scale = FP16TCEC, (1, 0)
+    else:
+        a = inputs.exponent_spread(5, m, k, per_row=True)
+        b = inputs.exponent_spread(6, k, n, per_row=False)
+        want_mode, want_scale = TF32TCEC, (0, 0)
+    c, a_after, b_after, ids = _pipeline(handle, dev, AUTO, N, N, m, n, k, a, b)
+    flag = handle.get_dynamic_launch_flag(ids[2])
+    assert flag & 0x1f == want_mode
+    assert (bool(flag & 0x40), bool(flag & 0x20)) == tuple(bool(x) for x in want_scale)
+    sa, sb = O.exp_stats(a, m, k, m), O.exp_stats(b, k, n, k)
+    assert flag == O.lib().oracle_combine_flag(sa.mode, sb.mode)
+    assert handle.get_exp_stats(ids[0]) == (sa.underflow, sa.total)
+    assert handle.get_exp_stats(ids[1]) == (sb.underflow, sb.total)
+    assert np.array_equal(a_after.view(np.uint32), a.view(np.uint32))
+    assert np.array_equal(b_after.view(np.uint32), b.view(np.uint32))
+    ref = O.gemm_fp64(N, N, m, n, k, 1.0, a, m, b, k)
+    r_fp32 = O.residual(ref, oracle_gemm(O, FP32, N, N, m, n, k, 1.0, a, m, b, k, 0.0, np.zeros(m * n, np.float32), m), m, n, m)
+    assert O.residual(ref, c, m, n, m) <= 2.0 * r_fp32
+
+
+def test_auto_complex_batched(O, handle, dev):
+    m, n, k, batch = 64, 48, 80, 3
+    a = inputs.complex_normal(7, m * k * batch, 2.0 ** -19)
+    b = inputs.complex_normal(8, k * n * batch, 1.0)
+    da, db, dc = dev.up(a), dev.up(b), dev.up(np.zeros(m * n * batch, np.complex64))
+    st, ids = handle.gemm_pipeline(N, N, m, n, k, 1.0, da, m, db, k, 0.0, dc, m, AUTO, cplx=True,
+                                   stridea=m * k, strideb=k * n, stridec=m * n, batch=batch)
+    assert st == 0
+    c = dev.down(dc, np.complex64)
+    flag = handle.get_dynamic_launch_flag(ids[2])
+    sa = O.exp_stats(a, m, k, m, batch=batch, stride=m * k)
+    sb = O.exp_stats(b, k, n, k, batch=batch, stride=k * n)
+    assert flag == O.lib().oracle_combine_flag(sa.mode, sb.mode)
+    assert np.array_equal(dev.down(da, np.complex64), a)
+    for i in range(batch):
+        ref = O.gemm_fp64(N, N, m, n, k, 1.0, a[i * m * k:], m, b[i * k * n:], k)
+        cf = oracle_gemm(O, FP32, N, N, m, n, k, 1.0, a[i * m * k:], m, b[i * k * n:], k, 0.0, np.zeros(m * n, np.complex64), m)
+        assert O.residual(ref, c[i * m * n:(i + 1) * m * n], m, n, m) <= 2.0 * O.residual(ref, cf, m, n, m)
