@@ -1,0 +1,292 @@
+#!/usr/bin/env python3
+"""Headline benchmark: effective FP32 TFLOP/s (2MNK/t) of FP16TCEC SGEMM at
+M=N=K=8192 (NN, uniform[-1,1], alpha=1, beta=0) on one MI355X, with the relative
+Frobenius error against an FP64 GEMM of the same inputs, next to hipBLAS native
+FP32 SGEMM on the same GPU and to the split-and-correct algorithm on host cores.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--full]
+
+One "step" is one GEMM call through the C ABI (cuMpSGEMM_sgemm) with operands
+resident in HBM.  Prints ONE JSON line.  --full adds the other BASELINE
+configurations (layouts, bf16x3, batched CGEMM, scaling pipeline, tall-skinny,
+Mx2x2) under "extra".
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+FP16_MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA
+HBM_PEAK_GBS = 8000.0
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=32)   # the reference times 32 calls (test/main.cu:15)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--size", type=int, default=8192)
+    ap.add_argument("--full", action="store_true")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the host-core baseline")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU (no collectives, no sharding); use --gpus 1")
+
+    import torch
+    import cumpsgemm_amd as cg
+    from cumpsgemm_amd import inputs
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    cg.lib()  # fails loudly if the HIP library has not been built
+    dev = torch.device("cuda:0")
+    stream = torch.cuda.current_stream()
+    h = cg.Handle()
+    h.set_stream(stream)
+
+    n = args.size
+    m = k = n
+    log(f"[bench] generating {n}x{n} inputs (seeds 1, 2)")
+    a_host = inputs.uniform(1, m * k)
+    b_host = inputs.uniform(2, k * n)
+    a = torch.from_numpy(a_host).to(dev)
+    b = torch.from_numpy(b_host).to(dev)
+    c = torch.zeros(m * n, device=dev)
+
+    def timed(fn, steps, warmup):
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        e0.record(stream)
+        for _ in range(steps):
+            fn()
+        e1.record(stream)
+        torch.cuda.synchronize()
+        wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+        return wall_ms, e0.elapsed_time(e1) / steps
+
+    def tcec(mode, opa=cg.OP_N, opb=cg.OP_N):
+        def fn():
+            st = h.gemm(opa, opb, m, n, k, 1.0, a, n, b, n, 0.0, c, n, mode)
+            assert st == 0
+        return fn
+
+    flops = 2.0 * m * n * k
+    log("[bench] FP16TCEC timed region")
+    wall_ms, ev_ms = timed(tcec(cg.FP16TCEC), args.steps, args.warmup)
+    value = flops / (wall_ms * 1e-3) / 1e12
+    kernel_tflops = flops / (ev_ms * 1e-3) / 1e12
+
+    # ---- error against FP64 (rocBLAS DGEMM on widened inputs), same inputs ----
+    log("[bench] FP64 reference")
+    A64 = a.view(n, n).t().double()  # column-major buffer -> logical matrix
+    B64 = b.view(n, n).t().double()
+    ref = A64 @ B64
+    ref_norm = torch.linalg.norm(ref).item()
+
+    def rel_err():
+        got = c.view(n, n).t().double()
+        return (torch.linalg.norm(got - ref) / ref_norm).item()
+
+    tcec(cg.FP16TCEC)()
+    err_tcec = rel_err()
+
+    # ---- hipBLAS native FP32 SGEMM on the same GPU ----
+    log("[bench] hipBLAS SGEMM")
+    hb_tflops, err_sgemm = None, None
+    try:
+        hb = ctypes.CDLL("libhipblas.so")
+        hbh = ctypes.c_void_p()
+        assert hb.hipblasCreate(ctypes.byref(hbh)) == 0
+        hb.hipblasSetStream(hbh, ctypes.c_void_p(stream.cuda_stream))
+        one, zero = ctypes.c_float(1.0), ctypes.c_float(0.0)
+        hb.hipblasSgemm.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                    ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int,
+                                    ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int]
+
+        def sgemm():
+            st = hb.hipblasSgemm(hbh, 111, 111, m, n, k, ctypes.byref(one), a.data_ptr(), n, b.data_ptr(), n,
+                                 ctypes.byref(zero), c.data_ptr(), n)
+            assert st == 0
+        hb_wall, _ = timed(sgemm, max(4, args.steps // 2), 2)
+        hb_tflops = flops / (hb_wall * 1e-3) / 1e12
+        sgemm()
+        err_sgemm = rel_err()
+        hb.hipblasDestroy(hbh)
+    except Exception as e:  # pragma: no cover
+        log(f"[bench] hipBLAS comparison unavailable: {e}")
+
+    extra = {}
+    if args.full:
+        extra = full_suite(torch, cg, inputs, h, dev, stream, timed, log)
+
+    # ---- CPU baseline: the same algorithm on the host cores (oracle, bounded sample) ----
+    cpu = None
+    if not args.no_cpu:
+        log("[bench] CPU baseline (oracle)")
+        from oracle import oracle as O
+        O.lib()
+        cn = 4096 if n >= 4096 else n
+        ca, cb = inputs.uniform(1, cn * cn), inputs.uniform(2, cn * cn)
+        cc = np.zeros(cn * cn, np.float32)
+        cores = int(os.environ.get("OMP_NUM_THREADS", "0")) or min(os.cpu_count() or 1, 16)
+        os.environ["OMP_NUM_THREADS"] = str(cores)
+        t0 = time.perf_counter()
+        O.gemm(O.MODE_FP16TCEC, O.OP_N, O.OP_N, cn, cn, cn, 1.0, ca, cn, cb, cn, 0.0, cc, cn)
+        dt = time.perf_counter() - t0
+        cpu = {"value": round(2.0 * cn ** 3 / dt / 1e12, 5), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+               "sample": f"one FP16TCEC SGEMM NN {cn}^3 (same generator, seeds 1,2) = 1/{(n // cn) ** 3} of the "
+                         f"{n}^3 step, split included, {dt:.1f} s"}
+
+    out = {
+        "metric": "effective FP32 TFLOP/s (2MNK/t) at 8192^3 FP16TCEC + rel. error vs FP64",
+        "value": round(value, 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(wall_ms, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16 (hi/lo split of f32, 3 MFMA products, f32 accumulate)",
+        "data": "synthetic",
+        "config": {"workload": f"C2: SGEMM NN M=N=K={n}, A,B uniform[-1,1] seeds (1,2), alpha=1, beta=0, mode FP16TCEC",
+                   "layout": "NN", "mode": "FP16TCEC"},
+        "rel_error_vs_fp64": err_tcec,
+        "rel_error_hipblas_sgemm_vs_fp64": err_sgemm,
+        "error_ratio_vs_sgemm": (err_tcec / err_sgemm) if err_sgemm else None,
+        "hipblas_sgemm_tflops": round(hb_tflops, 2) if hb_tflops else None,
+        "speedup_vs_hipblas_sgemm": round(value / hb_tflops, 3) if hb_tflops else None,
+        "roofline": {
+            "bound": "mfma",
+            # MFMA flops actually issued = 3 products x algorithmic 2MNK, over the
+            # kernel's average duration between HIP events on the launch stream
+            "achieved": round(3.0 * kernel_tflops, 1),
+            "peak": FP16_MFMA_PEAK_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": round(3.0 * kernel_tflops / FP16_MFMA_PEAK_TFLOPS, 4),
+            "traffic": None,
+            "algorithmic_tflops": round(kernel_tflops, 2),
+            "mfma_products_per_flop": 3,
+            "kernel_ms": round(ev_ms, 4),
+        },
+        "cpu_baseline": cpu,
+    }
+    if extra:
+        out["extra"] = extra
+    print(json.dumps(out), flush=True)
+    h.close()
+
+
+def full_suite(torch, cg, inputs, h, dev, stream, timed, log):
+    """The other BASELINE configurations, reported under "extra"."""
+    res = {}
+
+    def rel_err(got, ref):
+        return (torch.linalg.norm(got - ref) / torch.linalg.norm(ref)).item()
+
+    # C2 layouts and modes at 8192^3
+    n = 8192
+    a = torch.from_numpy(inputs.uniform(1, n * n)).to(dev)
+    b = torch.from_numpy(inputs.uniform(2, n * n)).to(dev)
+    c = torch.zeros(n * n, device=dev)
+    A, B = a.view(n, n).t().double(), b.view(n, n).t().double()
+    refs = {"NN": A @ B, "TN": A.t() @ B, "NT": A @ B.t()}
+    for name, opa, opb in (("NN", cg.OP_N, cg.OP_N), ("TN", cg.OP_T, cg.OP_N), ("NT", cg.OP_N, cg.OP_T)):
+        for mode_name, mode in (("FP16TCEC", cg.FP16TCEC), ("bf16x3", cg.TF32TCEC)):
+            log(f"[bench] C2 {name} {mode_name}")
+            fn = lambda: h.gemm(opa, opb, n, n, n, 1.0, a, n, b, n, 0.0, c, n, mode)
+            wall, ev = timed(fn, 10, 2)
+            res[f"C2_{name}_{mode_name}"] = {"tflops": round(2.0 * n ** 3 / wall / 1e9, 2),
+                                             "rel_error": rel_err(c.view(n, n).t().double(), refs[name])}
+    del refs, A, B, a, b, c
+    torch.cuda.empty_cache()
+
+    # C3: strided-batched CGEMM, batch 64 x 512^3
+    bs, s = 64, 512
+    za = torch.from_numpy(inputs.complex_normal(1, bs * s * s, (1.0 / (2 * s)) ** 0.5).view(np.float32)).to(dev)
+    zb = torch.from_numpy(inputs.complex_normal(2, bs * s * s, (1.0 / (2 * s)) ** 0.5).view(np.float32)).to(dev)
+    zc = torch.zeros(bs * s * s * 2, device=dev)
+    fn = lambda: h.gemm_strided_batch(cg.OP_N, cg.OP_N, s, s, s, 1.0, za, s, s * s, zb, s, s * s, 0.0, zc, s, s * s,
+                                      bs, cg.FP16TCEC, cplx=True)
+    log("[bench] C3 batched CGEMM")
+    wall, ev = timed(fn, 20, 2)
+    ZA = torch.view_as_complex(za.view(bs, s, s, 2)).transpose(1, 2).to(torch.complex128)
+    ZB = torch.view_as_complex(zb.view(bs, s, s, 2)).transpose(1, 2).to(torch.complex128)
+    ZC = torch.view_as_complex(zc.view(bs, s, s, 2)).transpose(1, 2).to(torch.complex128)
+    res["C3_cgemm_batch64_512"] = {"tflops": round(8.0 * s ** 3 * bs / wall / 1e9, 2), "rel_error": rel_err(ZC, ZA @ ZB)}
+
+    # C4: FP16TCEC_SCALING pipeline at 4096^3 with 2^{+-30} row/column exponents
+    n = 4096
+    ea = inputs.exponent_spread(3, n, n, per_row=True)
+    eb = inputs.exponent_spread(4, n, n, per_row=False)
+    a, b = torch.from_numpy(ea).to(dev), torch.from_numpy(eb).to(dev)
+    c = torch.zeros(n * n, device=dev)
+    ref = a.view(n, n).t().double() @ b.view(n, n).t().double()
+    log("[bench] C4 scaling pipeline")
+    fn = lambda: h.gemm_pipeline(cg.OP_N, cg.OP_N, n, n, n, 1.0, a, n, b, n, 0.0, c, n, cg.FP16TCEC_SCALING)
+    wall, ev = timed(fn, 10, 2)
+    err_scaled = rel_err(c.view(n, n).t().double(), ref)
+    h.gemm_pipeline(cg.OP_N, cg.OP_N, n, n, n, 1.0, a, n, b, n, 0.0, c, n, cg.AUTO)
+    err_auto = rel_err(c.view(n, n).t().double(), ref)
+    err_fp32 = rel_err((a.view(n, n).t() @ b.view(n, n).t()).double(), ref)
+    st_ms = timed(lambda: h.exp_stats_ext(n, n, a, n), 20, 3)[1]
+    mx_ms = timed(lambda: h.exp_max_ext(n, n, a, n), 20, 3)[1]
+    sid = h.exp_max_ext(n, n, a, n)
+    sc_ms = timed(lambda: (h.scale_A(sid, 1, n, n, a, n), h.reset_scale_A(sid, 1, n, n, a, n)), 20, 3)[1] / 2
+    nbytes = 4.0 * n * n
+    res["C4_scaling_4096"] = {
+        "pipeline_tflops": round(2.0 * n ** 3 / wall / 1e9, 2), "rel_error_scaling": err_scaled,
+        "rel_error_auto": err_auto, "rel_error_fp32_matmul": err_fp32,
+        "exp_stats_GBs": round(nbytes * 2 / st_ms / 1e6, 1), "exp_max_GBs": round(nbytes / mx_ms / 1e6, 1),
+        "scaling_GBs": round(2 * nbytes / sc_ms / 1e6, 1), "hbm_peak_GBs": HBM_PEAK_GBS}
+    del a, b, c, ref
+    torch.cuda.empty_cache()
+
+    # C5a: tall-skinny 16384 x 16384 x 256
+    mm, kk = 16384, 256
+    a = torch.from_numpy(inputs.uniform(1, mm * kk)).to(dev)
+    b = torch.from_numpy(inputs.uniform(2, kk * mm)).to(dev)
+    c = torch.zeros(mm * mm, device=dev)
+    log("[bench] C5a tall-skinny")
+    fn = lambda: h.gemm(cg.OP_N, cg.OP_N, mm, mm, kk, 1.0, a, mm, b, kk, 0.0, c, mm, cg.FP16TCEC)
+    wall, ev = timed(fn, 10, 2)
+    ref = a.view(kk, mm).t().double() @ b.view(mm, kk).t().double()
+    res["C5a_16384x16384x256"] = {"tflops": round(2.0 * mm * mm * kk / wall / 1e9, 2),
+                                  "rel_error": rel_err(c.view(mm, mm).t().double(), ref)}
+    del a, b, c, ref
+    torch.cuda.empty_cache()
+
+    # C5b: Mx2x2 CGEMM, M = 2^27 (state vector x 2x2 unitary), HBM-bound
+    M = 1 << 27
+    log("[bench] C5b Mx2x2")
+    x = torch.randn(M * 2 * 2, device=dev) * (0.5 ** 0.5)
+    u = torch.from_numpy(inputs.random_unitary_2x2(9).view(np.float32)).to(dev)
+    y = torch.zeros(M * 2 * 2, device=dev)
+    fn = lambda: h.gemm_Mx2x2(cg.OP_N, cg.OP_N, M, 1.0, x, M, u, 2, 0.0, y, M, cplx=True)
+    wall, ev = timed(fn, 10, 2)
+    X = torch.view_as_complex(x.view(2, M, 2)[:, : 1 << 20].contiguous()).t().to(torch.complex128)
+    Y = torch.view_as_complex(y.view(2, M, 2)[:, : 1 << 20].contiguous()).t().to(torch.complex128)
+    U = torch.view_as_complex(u.view(2, 2, 2)).t().to(torch.complex128)
+    res["C5b_cgemm_2^27x2x2"] = {"GBs": round(2.0 * M * 2 * 8 / ev / 1e6, 1), "hbm_peak_GBs": HBM_PEAK_GBS,
+                                 "rel_error_first_2^20_rows": rel_err(Y, X @ U)}
+    return res
+
+
+if __name__ == "__main__":
+    main()

@@ -50,7 +50,7 @@ def lib():
             raise RuntimeError(
                 f"{_LIB} is missing: build it with `make -C {os.path.join(_HERE, 'csrc')}` "
                 "(there is no CPU fallback)")
-        L = ctypes.CDLL(_LIB, mode=ctypes.RTLD_GLOBAL)
+        L = ctypes.CDLL(_LIB)
         _declare(L)
         _lib = L
     return _lib

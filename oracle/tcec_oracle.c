@@ -224,47 +224,68 @@ static void free_planes(planes_t *pl) {
   for (int i = 0; i < 3; i++) free(pl->p[i]);
 }
 
-/* acc[0..m) (+)= sign * sum_k a[:,k] * b[k]  in FP32, sequential in k.
+/* Cache blocking of the CPU loops.  Blocking never changes the result: for
+ * every output element each term's products are still added in ascending k, one
+ * FP32 addition at a time, into that element's own accumulator. */
+#define TILE_M 512
+#define TILE_N 64
+#define TILE_K 256
+
+/* acc[j*mb + i] += sign * sum_k A[i0+i, k] * B[k, j0+j]   (FP32, ascending k).
  * Products of two fp16/bf16-valued floats are exact in FP32, so a fused
  * multiply-add and a separate multiply+add give identical bits. */
-static void axpy_cols(float *acc, const float *a, const float *bcol, size_t m,
-                      size_t k, float sign) {
-  for (size_t p = 0; p < k; p++) {
-    const float b = sign * bcol[p];
-    const float *ap = a + p * m;
-    for (size_t i = 0; i < m; i++) acc[i] += ap[i] * b;
+/* cloned per ISA level and dispatched at load time, so the prebuilt library
+ * runs on any x86-64 host yet vectorises well where it can; -ffp-contract=off
+ * keeps the arithmetic identical across clones */
+__attribute__((target_clones("avx512f", "avx2", "default")))
+static void tile_term(float *acc, const float *a, const float *b, size_t m,
+                      size_t k, size_t i0, size_t mb, size_t j0, size_t nb,
+                      float sign) {
+  for (size_t k0 = 0; k0 < k; k0 += TILE_K) {
+    const size_t k1 = (k0 + TILE_K < k) ? k0 + TILE_K : k;
+    for (size_t j = 0; j < nb; j++) {
+      float *accj = acc + j * mb;
+      const float *bcol = b + (j0 + j) * k;
+      for (size_t p = k0; p < k1; p++) {
+        const float bv = sign * bcol[p];
+        const float *ap = a + p * m + i0;
+        for (size_t i = 0; i < mb; i++) accj[i] += ap[i] * bv;
+      }
+    }
   }
 }
 
-/* One real product op(A) (m x k planes) times op(B) (k x n planes) into
- * main/corr accumulators for output column j. */
-static void real_product_col(float *main_acc, float *corr_acc,
-                             const planes_t *A, const planes_t *B, size_t m,
-                             size_t k, size_t j, int mode, float sign) {
-  const size_t bo = j * k;
+/* One real product op(A) (m x k planes) times op(B) (k x n planes) into the
+ * main / correction accumulators of one output tile. */
+static void real_product_tile(float *main_acc, float *corr_acc,
+                              const planes_t *A, const planes_t *B, size_t m,
+                              size_t k, size_t i0, size_t mb, size_t j0,
+                              size_t nb, int mode, float sign) {
+#define TERM(acc, pa, pb) tile_term(acc, A->p[pa], B->p[pb], m, k, i0, mb, j0, nb, sign)
   switch (mode) {
   case ORACLE_MODE_FP16TCEC:
-    axpy_cols(main_acc, A->p[0], B->p[0] + bo, m, k, sign); /* hi*hi */
-    axpy_cols(corr_acc, A->p[1], B->p[0] + bo, m, k, sign); /* lo*hi */
-    axpy_cols(corr_acc, A->p[0], B->p[1] + bo, m, k, sign); /* hi*lo */
+    TERM(main_acc, 0, 0); /* hi*hi */
+    TERM(corr_acc, 1, 0); /* lo*hi */
+    TERM(corr_acc, 0, 1); /* hi*lo */
     break;
   case ORACLE_MODE_TF32TCEC: /* bf16x3: all terms with i+j <= 2 */
-    axpy_cols(main_acc, A->p[0], B->p[0] + bo, m, k, sign);
-    axpy_cols(corr_acc, A->p[2], B->p[0] + bo, m, k, sign);
-    axpy_cols(corr_acc, A->p[0], B->p[2] + bo, m, k, sign);
-    axpy_cols(corr_acc, A->p[1], B->p[1] + bo, m, k, sign);
-    axpy_cols(corr_acc, A->p[1], B->p[0] + bo, m, k, sign);
-    axpy_cols(corr_acc, A->p[0], B->p[1] + bo, m, k, sign);
+    TERM(main_acc, 0, 0);
+    TERM(corr_acc, 2, 0);
+    TERM(corr_acc, 0, 2);
+    TERM(corr_acc, 1, 1);
+    TERM(corr_acc, 1, 0);
+    TERM(corr_acc, 0, 1);
     break;
   case ORACLE_MODE_TF32TC: /* bf16x2: b0*b0 + b0*b1 + b1*b0 */
-    axpy_cols(main_acc, A->p[0], B->p[0] + bo, m, k, sign);
-    axpy_cols(corr_acc, A->p[1], B->p[0] + bo, m, k, sign);
-    axpy_cols(corr_acc, A->p[0], B->p[1] + bo, m, k, sign);
+    TERM(main_acc, 0, 0);
+    TERM(corr_acc, 1, 0);
+    TERM(corr_acc, 0, 1);
     break;
   default: /* FP16TC, FP32 */
-    axpy_cols(main_acc, A->p[0], B->p[0] + bo, m, k, sign);
+    TERM(main_acc, 0, 0);
     break;
   }
+#undef TERM
 }
 
 static inline float corr_scale(int mode) {
@@ -277,8 +298,8 @@ static inline float corr_scale(int mode) {
 void oracle_sgemm(int mode, int op_a, int op_b, size_t m, size_t n, size_t k,
                   float alpha, const float *a, size_t lda, const float *b,
                   size_t ldb, float beta, float *c, size_t ldc) {
-  float *da = (float *)malloc(m * k * sizeof(float));
-  float *db = (float *)malloc(k * n * sizeof(float));
+  float *da = (float *)malloc((m * k + 1) * sizeof(float));
+  float *db = (float *)malloc((k * n + 1) * sizeof(float));
   gather_plane(da, a, op_a == ORACLE_OP_C ? ORACLE_OP_T : op_a, m, k, lda, 1, 0);
   gather_plane(db, b, op_b == ORACLE_OP_C ? ORACLE_OP_T : op_b, k, n, ldb, 1, 0);
   planes_t A, B;
@@ -287,26 +308,33 @@ void oracle_sgemm(int mode, int op_a, int op_b, size_t m, size_t n, size_t k,
   free(da);
   free(db);
   const float cs = corr_scale(mode);
+  const long tiles_m = (long)((m + TILE_M - 1) / TILE_M);
+  const long tiles_n = (long)((n + TILE_N - 1) / TILE_N);
 #pragma omp parallel
   {
-    float *main_acc = (float *)malloc(m * sizeof(float));
-    float *corr_acc = (float *)malloc(m * sizeof(float));
-#pragma omp for schedule(static)
-    for (long j = 0; j < (long)n; j++) {
-      memset(main_acc, 0, m * sizeof(float));
-      memset(corr_acc, 0, m * sizeof(float));
-      real_product_col(main_acc, corr_acc, &A, &B, m, k, (size_t)j, mode, 1.0f);
-      for (size_t i = 0; i < m; i++) {
-        const float acc = main_acc[i] + corr_acc[i] * cs;
-        float *cp = c + i + (size_t)j * ldc;
-        if (beta == 0.0f)
-          *cp = acc * alpha;
-        else
-          *cp = acc * alpha + beta * (*cp);
+    float *main_acc = (float *)malloc(2 * TILE_M * TILE_N * sizeof(float));
+    float *corr_acc = main_acc + TILE_M * TILE_N;
+#pragma omp for schedule(dynamic) collapse(2)
+    for (long tj = 0; tj < tiles_n; tj++) {
+      for (long ti = 0; ti < tiles_m; ti++) {
+        const size_t i0 = (size_t)ti * TILE_M, j0 = (size_t)tj * TILE_N;
+        const size_t mb = (m - i0 < TILE_M) ? m - i0 : TILE_M;
+        const size_t nb = (n - j0 < TILE_N) ? n - j0 : TILE_N;
+        memset(main_acc, 0, 2 * TILE_M * TILE_N * sizeof(float));
+        real_product_tile(main_acc, corr_acc, &A, &B, m, k, i0, mb, j0, nb, mode, 1.0f);
+        for (size_t j = 0; j < nb; j++) {
+          for (size_t i = 0; i < mb; i++) {
+            const float acc = main_acc[j * mb + i] + corr_acc[j * mb + i] * cs;
+            float *cp = c + (i0 + i) + (j0 + j) * ldc;
+            if (beta == 0.0f)
+              *cp = acc * alpha;
+            else
+              *cp = acc * alpha + beta * (*cp);
+          }
+        }
       }
     }
     free(main_acc);
-    free(corr_acc);
   }
   free_planes(&A);
   free_planes(&B);
@@ -321,7 +349,7 @@ void oracle_cgemm(int mode, int op_a, int op_b, size_t m, size_t n, size_t k,
                   const float *alpha, const float *a, size_t lda,
                   const float *b, size_t ldb, const float *beta, float *c,
                   size_t ldc) {
-  float *tmp = (float *)malloc((m * k > k * n ? m * k : k * n) * sizeof(float));
+  float *tmp = (float *)malloc(((m * k > k * n ? m * k : k * n) + 1) * sizeof(float));
   planes_t Ar, Ai, Br, Bi;
   gather_plane(tmp, a, op_a, m, k, lda, 2, 0);
   split_planes(&Ar, tmp, m * k, mode);
@@ -334,33 +362,43 @@ void oracle_cgemm(int mode, int op_a, int op_b, size_t m, size_t n, size_t k,
   free(tmp);
   const float cs = corr_scale(mode);
   const int beta_zero = (beta[0] == 0.0f && beta[1] == 0.0f);
+  const long tiles_m = (long)((m + TILE_M - 1) / TILE_M);
+  const long tiles_n = (long)((n + TILE_N - 1) / TILE_N);
 #pragma omp parallel
   {
-    float *acc = (float *)malloc(4 * m * sizeof(float));
-    float *re_m = acc, *re_c = acc + m, *im_m = acc + 2 * m, *im_c = acc + 3 * m;
-#pragma omp for schedule(static)
-    for (long j = 0; j < (long)n; j++) {
-      memset(acc, 0, 4 * m * sizeof(float));
-      real_product_col(re_m, re_c, &Ar, &Br, m, k, (size_t)j, mode, 1.0f);
-      real_product_col(re_m, re_c, &Ai, &Bi, m, k, (size_t)j, mode, -1.0f);
-      real_product_col(im_m, im_c, &Ar, &Bi, m, k, (size_t)j, mode, 1.0f);
-      real_product_col(im_m, im_c, &Ai, &Br, m, k, (size_t)j, mode, 1.0f);
-      for (size_t i = 0; i < m; i++) {
-        const float x = re_m[i] + re_c[i] * cs;
-        const float y = im_m[i] + im_c[i] * cs;
-        float *cp = c + 2 * (i + (size_t)j * ldc);
-        /* mul(a, alpha) = (a.x*al.x - a.y*al.y, a.y*al.x + a.x*al.y) */
-        float rx = x * alpha[0] - y * alpha[1];
-        float ry = y * alpha[0] + x * alpha[1];
-        if (!beta_zero) {
-          /* mad(v, alpha, mul(beta, c)) */
-          const float bx = beta[0] * cp[0] - beta[1] * cp[1];
-          const float by = beta[1] * cp[0] + beta[0] * cp[1];
-          rx = x * alpha[0] - y * alpha[1] + bx;
-          ry = y * alpha[0] + x * alpha[1] + by;
+    const size_t T = (size_t)TILE_M * TILE_N;
+    float *acc = (float *)malloc(4 * T * sizeof(float));
+    float *re_m = acc, *re_c = acc + T, *im_m = acc + 2 * T, *im_c = acc + 3 * T;
+#pragma omp for schedule(dynamic) collapse(2)
+    for (long tj = 0; tj < tiles_n; tj++) {
+      for (long ti = 0; ti < tiles_m; ti++) {
+        const size_t i0 = (size_t)ti * TILE_M, j0 = (size_t)tj * TILE_N;
+        const size_t mb = (m - i0 < TILE_M) ? m - i0 : TILE_M;
+        const size_t nb = (n - j0 < TILE_N) ? n - j0 : TILE_N;
+        memset(acc, 0, 4 * T * sizeof(float));
+        real_product_tile(re_m, re_c, &Ar, &Br, m, k, i0, mb, j0, nb, mode, 1.0f);
+        real_product_tile(re_m, re_c, &Ai, &Bi, m, k, i0, mb, j0, nb, mode, -1.0f);
+        real_product_tile(im_m, im_c, &Ar, &Bi, m, k, i0, mb, j0, nb, mode, 1.0f);
+        real_product_tile(im_m, im_c, &Ai, &Br, m, k, i0, mb, j0, nb, mode, 1.0f);
+        for (size_t j = 0; j < nb; j++) {
+          for (size_t i = 0; i < mb; i++) {
+            const float x = re_m[j * mb + i] + re_c[j * mb + i] * cs;
+            const float y = im_m[j * mb + i] + im_c[j * mb + i] * cs;
+            float *cp = c + 2 * ((i0 + i) + (j0 + j) * ldc);
+            /* mul(a, alpha) = (a.x*al.x - a.y*al.y, a.y*al.x + a.x*al.y) */
+            float rx = x * alpha[0] - y * alpha[1];
+            float ry = y * alpha[0] + x * alpha[1];
+            if (!beta_zero) {
+              /* mad(v, alpha, mul(beta, c)) */
+              const float bx = beta[0] * cp[0] - beta[1] * cp[1];
+              const float by = beta[1] * cp[0] + beta[0] * cp[1];
+              rx = x * alpha[0] - y * alpha[1] + bx;
+              ry = y * alpha[0] + x * alpha[1] + by;
+            }
+            cp[0] = rx;
+            cp[1] = ry;
+          }
         }
-        cp[0] = rx;
-        cp[1] = ry;
       }
     }
     free(acc);
