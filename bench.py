@@ -39,6 +39,10 @@ def main():
     ap.add_argument("--size", type=int, default=8192)
     ap.add_argument("--full", action="store_true")
     ap.add_argument("--no-cpu", action="store_true", help="skip the host-core baseline")
+    ap.add_argument("--kernel-only", action="store_true",
+                    help="time the FP16TCEC GEMM only (no FP64 check, hipBLAS or CPU legs): for profilers")
+    ap.add_argument("--op", default="NN", choices=["NN", "TN", "NT", "TT"])
+    ap.add_argument("--mode", default="FP16TCEC", choices=["FP16TCEC", "TF32TCEC", "FP16TC", "TF32TC"])
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (no collectives, no sharding); use --gpus 1")
@@ -79,14 +83,24 @@ def main():
         wall_ms = (time.perf_counter() - t0) * 1e3 / steps
         return wall_ms, e0.elapsed_time(e1) / steps
 
+    flops = 2.0 * m * n * k
+
     def tcec(mode, opa=cg.OP_N, opb=cg.OP_N):
         def fn():
             st = h.gemm(opa, opb, m, n, k, 1.0, a, n, b, n, 0.0, c, n, mode)
             assert st == 0
         return fn
 
-    flops = 2.0 * m * n * k
     log("[bench] FP16TCEC timed region")
+    if args.kernel_only:
+        opa = cg.OP_T if args.op[0] == "T" else cg.OP_N
+        opb = cg.OP_T if args.op[1] == "T" else cg.OP_N
+        wall_ms, ev_ms = timed(tcec(getattr(cg, args.mode), opa, opb), args.steps, args.warmup)
+        print(json.dumps({"kernel_only": True, "op": args.op, "mode": args.mode, "size": n,
+                          "ms_per_step": round(wall_ms, 4), "kernel_ms": round(ev_ms, 4),
+                          "tflops": round(flops / (ev_ms * 1e-3) / 1e12, 2)}), flush=True)
+        h.close()
+        return
     wall_ms, ev_ms = timed(tcec(cg.FP16TCEC), args.steps, args.warmup)
     value = flops / (wall_ms * 1e-3) / 1e12
     kernel_tflops = flops / (ev_ms * 1e-3) / 1e12

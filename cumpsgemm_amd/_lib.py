@@ -50,6 +50,14 @@ def lib():
             raise RuntimeError(
                 f"{_LIB} is missing: build it with `make -C {os.path.join(_HERE, 'csrc')}` "
                 "(there is no CPU fallback)")
+        # A process must end up with ONE HIP runtime.  PyTorch ships its own copy
+        # of libamdhip64 (same SONAME as the system one): if it is going to be
+        # used in this process, let it load first so that this library binds to
+        # the runtime that owns the tensors' memory and streams.
+        try:
+            import torch  # noqa: F401
+        except Exception:
+            pass
         L = ctypes.CDLL(_LIB)
         _declare(L)
         _lib = L

@@ -1,5 +1,11 @@
-// Kernel instances of the tile table for one (precision, element type) pair.
+// Kernel instances of the tile table for one (precision, element type) pair:
+// three tile classes (large, medium, small) for each layout pair.
 #include "gemm_table.hpp"
 namespace cumpsgemm_amd {
-CUMPSGEMM_DEFINE_TABLE(g_tab_fp16tcec_c, CUMPSGEMM_CPLX_ROW, Prec::FP16TCEC)
+#define ROW(AKC, BKC) \
+  { CUMPSGEMM_ENTRY(Prec::FP16TCEC, true, AKC, BKC, 128, 64, 32, 32, 2, true, "c128x64x32_w32x32_deep"), \
+    CUMPSGEMM_ENTRY(Prec::FP16TCEC, true, AKC, BKC, 64, 64, 32, 32, 2, false, "c64x64x32_w32x32"), \
+    CUMPSGEMM_ENTRY(Prec::FP16TCEC, true, AKC, BKC, 32, 32, 32, 32, 2, false, "c32x32x32_w32x32") }
+CUMPSGEMM_DEFINE_TABLE(g_tab_fp16tcec_c, ROW)
+#undef ROW
 } // namespace cumpsgemm_amd

@@ -15,6 +15,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <type_traits>
 
 namespace cumpsgemm_amd {
 
@@ -93,13 +94,35 @@ struct GemmArgs {
 // ---- split one group of 8 FP32 values into NP packed 16-byte plane chunks ----
 template <Prec P> struct splitter;
 
+// hi = fp16(x); lo = fp16((x - hi) * 2^11).  (x - hi) is exact in FP32 and so is
+// the scaling, hence lo = fp16(fma(hi, -2^11, x * 2^11)) is the same value; it
+// is evaluated with the mixed-precision FMA that reads hi straight from its
+// packed fp16 register and writes the fp16 result into the low / high half of
+// the destination: 2.5 vector instructions per element instead of 4.
+__device__ inline uint32_t split_pair_fp16(const float x0, const float x1, uint32_t &lo) {
+  typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
+  typedef float f2_t __attribute__((ext_vector_type(2)));
+  f2_t x = {x0, x1};
+  const uint32_t hi = __builtin_bit_cast(uint32_t, __builtin_convertvector(x, h2_t));
+  const float t0 = x0 * 2048.0f, t1 = x1 * 2048.0f;
+  const float k = -2048.0f;
+  uint32_t l;
+  asm("v_fma_mixlo_f16 %0, %1, %2, %3 op_sel_hi:[1,0,0]" : "=v"(l) : "v"(hi), "s"(k), "v"(t0));
+  asm("v_fma_mixhi_f16 %0, %1, %2, %3 op_sel:[1,0,0] op_sel_hi:[1,0,0]"
+      : "+v"(l)
+      : "v"(hi), "s"(k), "v"(t1));
+  lo = l;
+  return hi;
+}
+
 template <> struct splitter<Prec::FP16TCEC> {
   __device__ static inline void run(const f8_t x, u4_t (&out)[2]) {
-    const h8_t hi = __builtin_convertvector(x, h8_t);
-    const f8_t r = (x - __builtin_convertvector(hi, f8_t)) * 2048.0f;
-    const h8_t lo = __builtin_convertvector(r, h8_t);
-    out[0] = __builtin_bit_cast(u4_t, hi);
-    out[1] = __builtin_bit_cast(u4_t, lo);
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      uint32_t lo;
+      out[0][i] = split_pair_fp16(x[2 * i], x[2 * i + 1], lo);
+      out[1][i] = lo;
+    }
   }
 };
 template <> struct splitter<Prec::FP16TC> {
@@ -144,10 +167,14 @@ __device__ inline f16v_t mfma32(const u4_t a, const u4_t b, const f16v_t c) {
 //   A_KC: op(A) is stored K-contiguous (op T / C); else M-contiguous (op N)
 //   B_KC: op(B) is stored K-contiguous (op N);     else N-contiguous (op T / C)
 //   OCC : waves per SIMD the register allocator must leave room for
+//   DEEP: three LDS buffers and an interleaved instruction schedule (MFMAs with
+//         the staging work dripped in between); otherwise two buffers and
+//         plain program order.
 template <Prec P_, bool CPLX_, bool A_KC_, bool B_KC_, int BM_, int BN_, int WM_,
-          int WN_, int OCC_ = 1>
+          int WN_, int OCC_ = 1, bool DEEP_ = false>
 struct GemmCfg {
   static constexpr int OCC = OCC_;
+  static constexpr bool DEEP = DEEP_;
   static constexpr Prec P = P_;
   static constexpr bool CPLX = CPLX_;
   static constexpr bool A_KC = A_KC_;
@@ -158,24 +185,52 @@ struct GemmCfg {
   static constexpr int TM = WM / 32, TN = WN / 32;
   static constexpr int NP = prec_traits<P>::NP;
   static constexpr int NCOMP = CPLX ? 2 : 1;
-  // LDS row: 32 K-values * 2 bytes + 16 bytes of padding.  The 80-byte pitch
-  // makes both the fragment reads (consecutive rows, same chunk) and the
-  // staging writes sweep all banks.
-  static constexpr int ROW_BYTES = 80;
+  // LDS row: 32 K-values * 2 bytes = four 16-byte chunks, stored at chunk
+  // position (chunk ^ lds_swizzle(row)); see lds_offset().
+  static constexpr int ROW_BYTES = 64;
+  // DEEP workgroups keep three tiles in LDS so that a tile is complete one full
+  // step before it is multiplied and its first fragments can be fetched ahead
+  // of the barrier; the others double-buffer.
+  static constexpr int NSTAGE = DEEP_ ? 3 : 2;
   static constexpr int A_PLANE_BYTES = BM * ROW_BYTES;
   static constexpr int B_PLANE_BYTES = BN * ROW_BYTES;
   static constexpr int A_STAGE_BYTES = A_PLANE_BYTES * NP * NCOMP;
   static constexpr int B_STAGE_BYTES = B_PLANE_BYTES * NP * NCOMP;
   static constexpr int STAGE_BYTES = A_STAGE_BYTES + B_STAGE_BYTES;
-  static constexpr int LDS_BYTES = 2 * STAGE_BYTES;
+  static constexpr int LDS_BYTES = NSTAGE * STAGE_BYTES;
   // staging units: one unit = (row, chunk of 8 K-values)
-  static constexpr int UA = (BM * 4) / NT;
-  static constexpr int UB = (BN * 4) / NT;
-  static_assert((BM * 4) % NT == 0 && (BN * 4) % NT == 0, "tile/threads");
+  // (when a tile has fewer units than the workgroup has threads, the surplus
+  // waves simply stage nothing for that operand)
+  static constexpr int UA = (BM * 4 + NT - 1) / NT;
+  static constexpr int UB = (BN * 4 + NT - 1) / NT;
+  static_assert((BM * 4) % NT == 0 || (BM * 4) < NT, "tile/threads");
+  static_assert((BN * 4) % NT == 0 || (BN * 4) < NT, "tile/threads");
   static_assert(BM % WM == 0 && BN % WN == 0 && WM % 32 == 0 && WN % 32 == 0,
                 "wave tile");
   static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
 };
+
+// Byte offset of (row, 16-byte chunk) inside one LDS plane.  Rows are 64 bytes,
+// i.e. 16 banks; the chunk is XOR-swizzled with row bits chosen such that
+//  - 8 (16) consecutive rows at one logical chunk -- a fragment read, or a
+//    staging write of a row-contiguous tile -- cover all 32 (64) banks,
+//  - 2 (4) consecutive rows x 4 chunks -- a staging write of a K-contiguous
+//    tile -- do too.
+__device__ inline int lds_swizzle(int row) {
+  return (((row >> 1) ^ (row >> 3)) & 1) | (((row >> 2) & 1) << 1);
+}
+__device__ inline int lds_offset(int row, int chunk) {
+  return row * 64 + ((chunk ^ lds_swizzle(row)) << 4);
+}
+
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also fences
+// global memory, which makes every wave wait for its outstanding global loads
+// -- the prefetch of a later K-step -- before it may pass the barrier.
+__device__ inline void block_sync_lds() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
 
 // Map a linear workgroup id to a tile so that (a) workgroups that the
 // dispatcher places on the same XCD (id mod 8) work on neighbouring tiles and
@@ -206,15 +261,23 @@ __device__ inline void map_tile(uint32_t bid, uint32_t tiles_m, uint32_t tiles_n
 // Global -> register staging of one operand tile.
 //   ROWS rows (M for A, N for B) x 32 K-values; U units per thread.
 //   KC:   memory is K-contiguous  -> unit = (row, chunk), chunk fastest over
-//         lanes; each thread reads 8 consecutive elements (vector loads).
+//         lanes; each thread reads 8 consecutive elements (16-byte loads).
 //   !KC:  memory is row-contiguous -> unit = (row, chunk), row fastest over
 //         lanes; each thread reads 8 elements `ld` apart, consecutive lanes
 //         read consecutive addresses.
+// All addresses are "uniform base + per-thread 32-bit offset": the bases live
+// in scalar registers, the offsets are computed once per kernel.
 // Out-of-range elements read as zero, which contributes nothing to the sums.
 // ---------------------------------------------------------------------------
 template <bool CPLX, bool KC, int ROWS, int U, int NT>
 struct tile_loader {
-  // reg[u][comp] holds the 8 K-values of unit u (re or im)
+  static constexpr int NC = CPLX ? 2 : 1;
+  static constexpr int ES = CPLX ? 2 : 1;
+  static constexpr bool PARTIAL = (ROWS * 4) < NT; // fewer units than threads
+
+  // whether this thread stages anything of this operand (wave-uniform)
+  __device__ static inline bool active(int tid) { return !PARTIAL || tid < ROWS * 4; }
+
   __device__ static inline void unit_coords(int u, int tid, int &row, int &chunk) {
     const int id = tid + u * NT;
     if constexpr (KC) {
@@ -226,97 +289,132 @@ struct tile_loader {
     }
   }
 
-  // base points at element (row 0 of the tile, k 0 of the K-step)
-  template <bool FAST>
-  __device__ static inline void load(f8_t (&reg)[U][CPLX ? 2 : 1],
-                                     const float *__restrict__ base, uint64_t ld,
-                                     int rows_left, int k_left, int tid,
-                                     bool conj) {
+  // element offset of unit u from the tile origin
+  __device__ static inline uint32_t unit_offset(int u, int tid, uint32_t ld) {
+    int row, chunk;
+    unit_coords(u, tid, row, chunk);
+    return KC ? (uint32_t)row * ld + (uint32_t)chunk * 8 : (uint32_t)chunk * 8 * ld + (uint32_t)row;
+  }
+
+  // whether every per-thread byte offset of a tile fits 32 bits
+  __device__ static inline bool offsets_fit(uint64_t ld) {
+    const uint64_t span = KC ? (uint64_t)ROWS * ld + 32 : 32 * ld + ROWS;
+    return span * ES * 4 < 0x7fffffffull;
+  }
+
+  // byte offset of unit u from the tile origin
+  __device__ static inline uint32_t unit_byte_offset(int u, int tid, uint32_t ld) {
+    return unit_offset(u, tid, ld) * (uint32_t)(ES * 4);
+  }
+
+  // Staging registers of one thread: the 8 K-values (re, im) of each unit.
+  struct Regs {
+    f8_t v[U][NC];
+  };
+
+  // interior tile: base points at element (row 0 of the tile, k 0 of the K-step).
+  //   !KC: buffer loads -- the descriptor (scalar registers) carries the uniform
+  //        base, the vector offset is the thread's constant byte offset and the
+  //        scalar offset selects the K-line, so no vector ALU work goes into
+  //        addressing; consecutive lanes read consecutive addresses.
+  //   KC:  16-byte global loads at base + constant per-thread offset.
+  // (16-byte *buffer* loads are avoided on purpose: this toolchain narrows them
+  // incorrectly when the loaded vector is taken apart element-wise.)
+  __device__ static inline void load_fast(Regs &reg, const float *__restrict__ base, uint64_t ld,
+                                          const uint32_t (&boff)[U]) {
+    if (!active(threadIdx.x)) return;
+    if constexpr (KC) {
+#pragma unroll
+      for (int u = 0; u < U; u++) {
+        const float4 *p = reinterpret_cast<const float4 *>(reinterpret_cast<const char *>(base) + boff[u]);
+        if constexpr (!CPLX) {
+          const float4 lo = p[0], hi = p[1];
+          reg.v[u][0][0] = lo.x; reg.v[u][0][1] = lo.y; reg.v[u][0][2] = lo.z; reg.v[u][0][3] = lo.w;
+          reg.v[u][0][4] = hi.x; reg.v[u][0][5] = hi.y; reg.v[u][0][6] = hi.z; reg.v[u][0][7] = hi.w;
+        } else {
+#pragma unroll
+          for (int q = 0; q < 4; q++) {
+            const float4 t = p[q];
+            reg.v[u][0][2 * q] = t.x; reg.v[u][1][2 * q] = t.y;
+            reg.v[u][0][2 * q + 1] = t.z; reg.v[u][1][2 * q + 1] = t.w;
+          }
+        }
+      }
+    } else {
+      const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
+          const_cast<float *>(base), 0, 0xffffffff, 0x00020000);
+      const uint32_t line = (uint32_t)ld * (uint32_t)(ES * 4); // bytes between K-lines
+#pragma unroll
+      for (int u = 0; u < U; u++) {
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+#pragma unroll
+          for (int c = 0; c < NC; c++)
+            reg.v[u][c][j] = __builtin_bit_cast(
+                float, __builtin_amdgcn_raw_buffer_load_b32(rsrc, boff[u] + 4 * c, j * line, 0));
+        }
+      }
+    }
+  }
+
+  // The 8 K-values (re, im) of unit u, ready to be split.
+  __device__ static inline void fetch(Regs &reg, int u, bool conj, f8_t &re, f8_t &im) {
+    re = reg.v[u][0];
+    if constexpr (CPLX) {
+      im = reg.v[u][1];
+      if (conj) im = -im;
+    }
+  }
+
+  // edge tile / unaligned / huge ld: element-wise and guarded.  The branches
+  // keep only one load in flight per thread, which keeps this rarely used path
+  // from dictating the kernel's register budget.
+  __device__ static inline void load_guarded(Regs &reg, const float *__restrict__ base, uint64_t ld,
+                                             int rows_left, int k_left, int tid) {
+    if (!active(tid)) return;
 #pragma unroll
     for (int u = 0; u < U; u++) {
       int row, chunk;
       unit_coords(u, tid, row, chunk);
       const int k0 = chunk * 8;
-      if constexpr (!CPLX) {
-        f8_t v;
-        if constexpr (KC) {
-          const float *p = base + (uint64_t)row * ld + k0;
-          if constexpr (FAST) {
-            const float4 lo = *reinterpret_cast<const float4 *>(p);
-            const float4 hi = *reinterpret_cast<const float4 *>(p + 4);
-            v[0] = lo.x; v[1] = lo.y; v[2] = lo.z; v[3] = lo.w;
-            v[4] = hi.x; v[5] = hi.y; v[6] = hi.z; v[7] = hi.w;
+#pragma unroll
+      for (int j = 0; j < 8; j++) {
+        const uint64_t idx = KC ? (uint64_t)row * ld + (k0 + j) : (uint64_t)(k0 + j) * ld + row;
+        float tx = 0.0f, ty = 0.0f;
+        if (row < rows_left && k0 + j < k_left) {
+          if constexpr (!CPLX) {
+            tx = base[idx];
           } else {
-#pragma unroll
-            for (int j = 0; j < 8; j++)
-              v[j] = (row < rows_left && k0 + j < k_left) ? p[j] : 0.0f;
-          }
-        } else {
-          const float *p = base + (uint64_t)k0 * ld + row;
-#pragma unroll
-          for (int j = 0; j < 8; j++) {
-            if constexpr (FAST)
-              v[j] = p[(uint64_t)j * ld];
-            else
-              v[j] = (row < rows_left && k0 + j < k_left) ? p[(uint64_t)j * ld]
-                                                          : 0.0f;
+            const float2 t = reinterpret_cast<const float2 *>(base)[idx];
+            tx = t.x;
+            ty = t.y;
           }
         }
-        reg[u][0] = v;
-      } else {
-        f8_t re, im;
-        const float2 *cb = reinterpret_cast<const float2 *>(base);
-        if constexpr (KC) {
-          const float2 *p = cb + (uint64_t)row * ld + k0;
-          if constexpr (FAST) {
-#pragma unroll
-            for (int j = 0; j < 8; j += 2) {
-              const float4 t = *reinterpret_cast<const float4 *>(p + j);
-              re[j] = t.x; im[j] = t.y; re[j + 1] = t.z; im[j + 1] = t.w;
-            }
-          } else {
-#pragma unroll
-            for (int j = 0; j < 8; j++) {
-              float2 t = make_float2(0.f, 0.f);
-              if (row < rows_left && k0 + j < k_left) t = p[j];
-              re[j] = t.x; im[j] = t.y;
-            }
-          }
-        } else {
-          const float2 *p = cb + (uint64_t)k0 * ld + row;
-#pragma unroll
-          for (int j = 0; j < 8; j++) {
-            float2 t = make_float2(0.f, 0.f);
-            if (FAST || (row < rows_left && k0 + j < k_left))
-              t = p[(uint64_t)j * ld];
-            re[j] = t.x; im[j] = t.y;
-          }
-        }
-        if (conj) im = -im;
-        reg[u][0] = re;
-        reg[u][1] = im;
+        reg.v[u][0][j] = tx;
+        if constexpr (CPLX) reg.v[u][1][j] = ty;
       }
     }
   }
 
   // split and write to LDS: planes laid out [comp][plane][row][chunk]
   template <Prec P>
-  __device__ static inline void store(const f8_t (&reg)[U][CPLX ? 2 : 1],
-                                      char *lds_op, int tid) {
+  __device__ static inline void store(Regs &reg, char *lds_op, int tid, bool conj) {
     constexpr int NP = prec_traits<P>::NP;
-    constexpr int PLANE = ROWS * 80;
+    constexpr int PLANE = ROWS * 64;
+    if (!active(tid)) return;
 #pragma unroll
     for (int u = 0; u < U; u++) {
       int row, chunk;
       unit_coords(u, tid, row, chunk);
+      f8_t part[2];
+      fetch(reg, u, conj, part[0], part[1]);
 #pragma unroll
-      for (int c = 0; c < (CPLX ? 2 : 1); c++) {
+      for (int c = 0; c < NC; c++) {
         u4_t out[NP];
-        splitter<P>::run(reg[u][c], out);
+        splitter<P>::run(part[c], out);
 #pragma unroll
         for (int p = 0; p < NP; p++) {
-          *reinterpret_cast<u4_t *>(lds_op + (c * NP + p) * PLANE + row * 80 +
-                                    chunk * 16) = out[p];
+          *reinterpret_cast<u4_t *>(lds_op + (c * NP + p) * PLANE + lds_offset(row, chunk)) = out[p];
         }
       }
     }
@@ -343,7 +441,7 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave % (BM / Cfg::WM);
   const int wn = wave / (BM / Cfg::WM);
 
@@ -369,22 +467,26 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
   const uint64_t a_kstep = Cfg::A_KC ? (uint64_t)BK * ES : (uint64_t)BK * args.lda * ES;
   const uint64_t b_kstep = Cfg::B_KC ? (uint64_t)BK * ES : (uint64_t)BK * args.ldb * ES;
 
-  const int rows_a = (int)((args.m - m0 < (uint32_t)BM) ? args.m - m0 : BM);
-  const int rows_b = (int)((args.n - n0 < (uint32_t)BN) ? args.n - n0 : BN);
-  // vector loads need 16-byte aligned rows
-  const bool a_vec_ok = !Cfg::A_KC || CPLX
-                            ? (!Cfg::A_KC || ((args.lda & 1) == 0 && ((uintptr_t)a_tile & 15) == 0))
-                            : ((args.lda & 3) == 0 && ((uintptr_t)a_tile & 15) == 0);
-  const bool b_vec_ok = !Cfg::B_KC || CPLX
-                            ? (!Cfg::B_KC || ((args.ldb & 1) == 0 && ((uintptr_t)b_tile & 15) == 0))
-                            : ((args.ldb & 3) == 0 && ((uintptr_t)b_tile & 15) == 0);
-  const bool a_full = (rows_a == BM) && a_vec_ok;
-  const bool b_full = (rows_b == BN) && b_vec_ok;
-
   using LA = tile_loader<CPLX, Cfg::A_KC, BM, Cfg::UA, NT>;
   using LB = tile_loader<CPLX, Cfg::B_KC, BN, Cfg::UB, NT>;
-  f8_t ra[Cfg::UA][NCOMP];
-  f8_t rb[Cfg::UB][NCOMP];
+
+  const int rows_a = (int)((args.m - m0 < (uint32_t)BM) ? args.m - m0 : BM);
+  const int rows_b = (int)((args.n - n0 < (uint32_t)BN) ? args.n - n0 : BN);
+  // 16-byte loads along K need 16-byte aligned rows (4 floats / 2 complex)
+  const bool a_vec_ok = !Cfg::A_KC || (((args.lda * ES) & 3) == 0 && ((uintptr_t)a_tile & 15) == 0);
+  const bool b_vec_ok = !Cfg::B_KC || (((args.ldb * ES) & 3) == 0 && ((uintptr_t)b_tile & 15) == 0);
+  const bool a_full = (rows_a == BM) && a_vec_ok && LA::offsets_fit(args.lda);
+  const bool b_full = (rows_b == BN) && b_vec_ok && LB::offsets_fit(args.ldb);
+
+  uint32_t offa[Cfg::UA], offb[Cfg::UB];
+#pragma unroll
+  for (int u = 0; u < Cfg::UA; u++) offa[u] = LA::unit_byte_offset(u, tid, (uint32_t)args.lda);
+#pragma unroll
+  for (int u = 0; u < Cfg::UB; u++) offb[u] = LB::unit_byte_offset(u, tid, (uint32_t)args.ldb);
+
+  // staging registers: the next tile this wave will split and write to LDS
+  typename LA::Regs ra;
+  typename LB::Regs rb;
 
   // accumulators: [component][main/corr][TN][TM]; MFMA rows run along N and
   // MFMA columns along M so that a lane's 64 outputs of one register are 32
@@ -401,93 +503,190 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
 #pragma unroll
           for (int v = 0; v < 16; v++) acc[q][s][j][i][v] = 0.0f;
 
-  const int nk = (int)((kend - kbeg + BK - 1) / BK);
+  const int klen = (int)(kend - kbeg);
 
-  auto gload = [&](int kt) {
-    const int k_left = (int)(kend - kbeg) - kt * BK;
-    const bool kfull = k_left >= BK;
-    if (a_full && kfull)
-      LA::template load<true>(ra, a_tile + (uint64_t)kt * a_kstep, args.lda, rows_a, k_left, tid, args.conj_a);
-    else
-      LA::template load<false>(ra, a_tile + (uint64_t)kt * a_kstep, args.lda, rows_a, k_left, tid, args.conj_a);
-    if (b_full && kfull)
-      LB::template load<true>(rb, b_tile + (uint64_t)kt * b_kstep, args.ldb, rows_b, k_left, tid, args.conj_b);
-    else
-      LB::template load<false>(rb, b_tile + (uint64_t)kt * b_kstep, args.ldb, rows_b, k_left, tid, args.conj_b);
+  // FAST: interior tile, aligned, full K-step -> unguarded wide loads
+  auto gload = [&](int kt, auto fast_tag) {
+    constexpr bool FAST = decltype(fast_tag)::value;
+    const float *ap = a_tile + (uint64_t)kt * a_kstep;
+    const float *bp = b_tile + (uint64_t)kt * b_kstep;
+    if constexpr (FAST) {
+      LA::load_fast(ra, ap, args.lda, offa);
+      LB::load_fast(rb, bp, args.ldb, offb);
+    } else {
+      const int k_left = klen - kt * BK;
+      LA::load_guarded(ra, ap, args.lda, rows_a, k_left, tid);
+      LB::load_guarded(rb, bp, args.ldb, rows_b, k_left, tid);
+    }
   };
   auto lstore = [&](int stage) {
     char *sa = lds + stage * Cfg::STAGE_BYTES;
     char *sb = sa + Cfg::A_STAGE_BYTES;
-    LA::template store<P>(ra, sa, tid);
-    LB::template store<P>(rb, sb, tid);
+    LA::template store<P>(ra, sa, tid, args.conj_a);
+    LB::template store<P>(rb, sb, tid, args.conj_b);
   };
 
-  gload(0);
-  lstore(0);
-  __syncthreads();
-
-  // per-lane fragment offsets: row = lane % 32, chunk = 2*kk + lane / 32
+  // Per-lane fragment addresses.  Lane l of a 32x32x16 MFMA supplies row
+  // (l % 32) of its operand tile and K-values 8*(l/32).. of the 16-wide slice
+  // kk, i.e. 16-byte chunk 2*kk + l/32.  The swizzle only looks at the low four
+  // row bits, which are the lane's own, so the two slices differ by one XOR.
   const int frag_row = lane & 31;
-  const int frag_chunk = lane >> 5;
-  const int a_frag_off = (wm * Cfg::WM + frag_row) * 80 + frag_chunk * 16;
-  const int b_frag_off = (wn * Cfg::WN + frag_row) * 80 + frag_chunk * 16;
+  const int frag_g = lane >> 5;
+  int a_frag_off[BK / 16], b_frag_off[BK / 16];
+#pragma unroll
+  for (int kk = 0; kk < BK / 16; kk++) {
+    a_frag_off[kk] = lds_offset(wm * Cfg::WM + frag_row, 2 * kk + frag_g);
+    b_frag_off[kk] = lds_offset(wn * Cfg::WN + frag_row, 2 * kk + frag_g);
+  }
 
-  for (int kt = 0; kt < nk; kt++) {
-    const int stage = kt & 1;
-    if (kt + 1 < nk) gload(kt + 1);
-
+  // fragments of one 16-wide K-slice: [component][plane][tile]
+  struct Frags {
+    u4_t a[NCOMP][NP][TM];
+    u4_t b[NCOMP][NP][TN];
+  };
+  auto frag_load = [&](Frags &f, int stage, int kk) {
     const char *sa = lds + stage * Cfg::STAGE_BYTES;
     const char *sb = sa + Cfg::A_STAGE_BYTES;
 #pragma unroll
-    for (int kk = 0; kk < BK / 16; kk++) {
-      u4_t fa[NCOMP][NP][TM];
-      u4_t fb[NCOMP][NP][TN];
+    for (int q = 0; q < NCOMP; q++)
 #pragma unroll
-      for (int q = 0; q < NCOMP; q++)
+      for (int p = 0; p < NP; p++) {
 #pragma unroll
-        for (int p = 0; p < NP; p++) {
+        for (int i = 0; i < TM; i++)
+          f.a[q][p][i] = *reinterpret_cast<const u4_t *>(sa + (q * NP + p) * Cfg::A_PLANE_BYTES +
+                                                         a_frag_off[kk] + i * 32 * 64);
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+          f.b[q][p][j] = *reinterpret_cast<const u4_t *>(sb + (q * NP + p) * Cfg::B_PLANE_BYTES +
+                                                         b_frag_off[kk] + j * 32 * 64);
+      }
+  };
+  auto frag_mma = [&](Frags &f) {
+    if constexpr (!CPLX) {
+#pragma unroll
+      for (int t = 0; t < PT::NPROD; t++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
 #pragma unroll
           for (int i = 0; i < TM; i++)
-            fa[q][p][i] = *reinterpret_cast<const u4_t *>(
-                sa + (q * NP + p) * Cfg::A_PLANE_BYTES + a_frag_off + i * 32 * 80 + kk * 32);
+            acc[0][PT::ACC[t]][j][i] = mfma32<PT::IS_BF16>(
+                f.b[0][PT::PB[t]][j], f.a[0][PT::PA[t]][i], acc[0][PT::ACC[t]][j][i]);
+    } else {
+      // -Im(A) planes for the real part: re = ar*br + (-ai)*bi
+      u4_t fan[NP][TM];
 #pragma unroll
-          for (int j = 0; j < TN; j++)
-            fb[q][p][j] = *reinterpret_cast<const u4_t *>(
-                sb + (q * NP + p) * Cfg::B_PLANE_BYTES + b_frag_off + j * 32 * 80 + kk * 32);
+      for (int p = 0; p < NP; p++)
+#pragma unroll
+        for (int i = 0; i < TM; i++) fan[p][i] = f.a[1][p][i] ^ 0x80008000u;
+#pragma unroll
+      for (int t = 0; t < PT::NPROD; t++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+          for (int i = 0; i < TM; i++) {
+            const int s = PT::ACC[t], pa = PT::PA[t], pb = PT::PB[t];
+            acc[0][s][j][i] = mfma32<PT::IS_BF16>(f.b[0][pb][j], f.a[0][pa][i], acc[0][s][j][i]);
+            acc[1][s][j][i] = mfma32<PT::IS_BF16>(f.b[1][pb][j], f.a[0][pa][i], acc[1][s][j][i]);
+            acc[0][s][j][i] = mfma32<PT::IS_BF16>(f.b[1][pb][j], fan[pa][i], acc[0][s][j][i]);
+            acc[1][s][j][i] = mfma32<PT::IS_BF16>(f.b[0][pb][j], f.a[1][pa][i], acc[1][s][j][i]);
+          }
+    }
+  };
+  static_assert(BK / 16 == 2, "two K-slices per step");
+  auto mma_tile = [&](int stage) {
+    Frags f0, f1;
+    frag_load(f0, stage, 0);
+    frag_load(f1, stage, 1);
+    frag_mma(f0);
+    frag_mma(f1);
+  };
+
+  // The K loop over `nk` steps.  Two separate instances (fast / guarded loads)
+  // keep the rarely used guarded code out of the hot loop.  Loads past the last
+  // tile re-read the last one (never staged), which keeps the loop body free of
+  // conditionals that touch the staging registers.
+  auto pipeline = [&](const int nk, auto fast_tag) {
+    const int last = nk - 1;
+    auto clamp = [&](int kt) { return kt < last ? kt : last; };
+    Frags f0, f1;
+    if constexpr (!Cfg::DEEP) {
+      // Double-buffered: every wave multiplies tile t from one LDS buffer,
+      // stages tile t+1 into the other and prefetches tile t+2 into registers;
+      // one barrier per step.  Overlap of vector and matrix work comes from
+      // co-resident workgroups.
+      gload(0, fast_tag);
+      lstore(0);
+      gload(clamp(1), fast_tag);
+      block_sync_lds();
+      for (int t = 0; t < nk; t++) {
+        const int cur = t & 1;
+        frag_load(f0, cur, 0);
+        frag_load(f1, cur, 1);
+        frag_mma(f0);
+        frag_mma(f1);
+        if (t + 1 < nk) lstore(cur ^ 1);
+        gload(clamp(t + 2), fast_tag);
+        block_sync_lds();
+      }
+    } else {
+      // Three LDS buffers, one barrier per step, every wave does the same work.
+      // In step t a wave
+      //   - multiplies tile t (buffer t%3): the first K-slice from fragments it
+      //     fetched during step t-1, the second from fragments fetched now;
+      //   - splits the tile it holds in registers (t+2) into buffer (t+2)%3,
+      //     last read in step t-1, and reloads the registers with tile t+3;
+      //   - fetches the first K-slice of its fragments of tile t+1, complete
+      //     since the barrier that ended step t-1.
+      // The body is one basic block and the scheduler is told to drip the
+      // vector and memory instructions in between the MFMAs, so that each wave
+      // keeps the matrix pipe busy while it does its share of the staging; the
+      // second wave on the SIMD fills what gaps remain.
+      gload(0, fast_tag);
+      lstore(0);
+      gload(clamp(1), fast_tag);
+      lstore(1);
+      gload(clamp(2), fast_tag);
+      block_sync_lds();
+      frag_load(f0, 0, 0);
+      int b0 = 0, b1 = 1, b2 = 2; // buffers of tiles t, t+1, t+2
+      for (int t = 0; t < nk; t++) {
+        frag_load(f1, b0, 1);
+        frag_mma(f0);
+        frag_mma(f1);
+        lstore(b2);
+        gload(clamp(t + 3), fast_tag);
+        frag_load(f0, b1, 0);
+        if constexpr (decltype(fast_tag)::value) {
+          // 24 (real) MFMAs per step: after each one up to 4 vector ALU
+          // instructions, one LDS access and one global load
+#pragma unroll
+          for (int g = 0; g < 2 * PT::NPROD * TM * TN * (CPLX ? 4 : 1); g++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); // MFMA
+            __builtin_amdgcn_sched_group_barrier(0x002, 4, 0); // VALU
+            __builtin_amdgcn_sched_group_barrier(0x080, 1, 0); // DS
+            __builtin_amdgcn_sched_group_barrier(0x020, 1, 0); // VMEM read
+          }
         }
-      if constexpr (!CPLX) {
-#pragma unroll
-        for (int t = 0; t < PT::NPROD; t++)
-#pragma unroll
-          for (int j = 0; j < TN; j++)
-#pragma unroll
-            for (int i = 0; i < TM; i++)
-              acc[0][PT::ACC[t]][j][i] = mfma32<PT::IS_BF16>(
-                  fb[0][PT::PB[t]][j], fa[0][PT::PA[t]][i], acc[0][PT::ACC[t]][j][i]);
-      } else {
-        // -Im(A) planes for the real part: re = ar*br + (-ai)*bi
-        u4_t fan[NP][TM];
-#pragma unroll
-        for (int p = 0; p < NP; p++)
-#pragma unroll
-          for (int i = 0; i < TM; i++) fan[p][i] = fa[1][p][i] ^ 0x80008000u;
-#pragma unroll
-        for (int t = 0; t < PT::NPROD; t++)
-#pragma unroll
-          for (int j = 0; j < TN; j++)
-#pragma unroll
-            for (int i = 0; i < TM; i++) {
-              const int s = PT::ACC[t], pa = PT::PA[t], pb = PT::PB[t];
-              acc[0][s][j][i] = mfma32<PT::IS_BF16>(fb[0][pb][j], fa[0][pa][i], acc[0][s][j][i]);
-              acc[1][s][j][i] = mfma32<PT::IS_BF16>(fb[1][pb][j], fa[0][pa][i], acc[1][s][j][i]);
-              acc[0][s][j][i] = mfma32<PT::IS_BF16>(fb[1][pb][j], fan[pa][i], acc[0][s][j][i]);
-              acc[1][s][j][i] = mfma32<PT::IS_BF16>(fb[0][pb][j], fa[1][pa][i], acc[1][s][j][i]);
-            }
+        block_sync_lds();
+        const int tmp = b0;
+        b0 = b1;
+        b1 = b2;
+        b2 = tmp;
       }
     }
+  };
 
-    if (kt + 1 < nk) lstore(stage ^ 1);
-    __syncthreads();
+  if (a_full && b_full) {
+    const int nk_full = klen / BK;
+    if (nk_full > 0) pipeline(nk_full, std::true_type{});
+    if (klen % BK != 0) { // ragged K: one more, guarded, step
+      gload(nk_full, std::false_type{});
+      lstore(0);
+      block_sync_lds();
+      mma_tile(0);
+    }
+  } else {
+    pipeline((klen + BK - 1) / BK, std::false_type{});
   }
 
   // ---- epilogue -----------------------------------------------------------

@@ -55,22 +55,12 @@ CUMPSGEMM_DECLARE_TABLE(g_tab_bf16x2_s)
 CUMPSGEMM_DECLARE_TABLE(g_tab_bf16x2_c)
 #undef CUMPSGEMM_DECLARE_TABLE
 
-// Real tiles: {BM, BN, WM, WN, OCC} per class; complex likewise.
-// One row of a table = the same three tile classes for one layout pair.
-#define CUMPSGEMM_REAL_ROW(P, AKC, BKC)                                              \
-  {                                                                                  \
-    make_entry<GemmCfg<P, false, AKC, BKC, 128, 128, 64, 64, 2>>("128x128x32_w64x64"), \
-    make_entry<GemmCfg<P, false, AKC, BKC, 64, 64, 32, 32, 2>>("64x64x32_w32x32"),   \
-    make_entry<GemmCfg<P, false, AKC, BKC, 32, 32, 32, 32, 2>>("32x32x32_w32x32")    \
-  }
-#define CUMPSGEMM_CPLX_ROW(P, AKC, BKC)                                              \
-  {                                                                                  \
-    make_entry<GemmCfg<P, true, AKC, BKC, 64, 64, 32, 32, 2>>("c64x64x32_w32x32"),   \
-    make_entry<GemmCfg<P, true, AKC, BKC, 64, 64, 32, 32, 2>>("c64x64x32_w32x32"),   \
-    make_entry<GemmCfg<P, true, AKC, BKC, 32, 32, 32, 32, 2>>("c32x32x32_w32x32")    \
-  }
-#define CUMPSGEMM_DEFINE_TABLE(sym, ROW, P)                                          \
-  KernelEntry sym[4][kNumTileClasses] = {ROW(P, false, false), ROW(P, true, false), \
-                                         ROW(P, false, true), ROW(P, true, true)};
+// One table = the same three tile classes for each of the four layout pairs.
+// ROW(AKC, BKC) must expand to three make_entry<...>() initialisers.
+#define CUMPSGEMM_DEFINE_TABLE(sym, ROW)                                                       \
+  KernelEntry sym[4][kNumTileClasses] = {ROW(false, false), ROW(true, false), ROW(false, true), \
+                                         ROW(true, true)};
+#define CUMPSGEMM_ENTRY(P, CPLX, AKC, BKC, BM, BN, WM, WN, OCC, DEEP, NAME) \
+  make_entry<GemmCfg<P, CPLX, AKC, BKC, BM, BN, WM, WN, OCC, DEEP>>(NAME)
 
 } // namespace cumpsgemm_amd
