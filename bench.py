@@ -25,6 +25,11 @@ sys.path.insert(0, ROOT)
 
 FP16_MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per 8192^3 FP16TCEC launch from the rocprofv3 FETCH_SIZE + WRITE_SIZE
+# counters, scaled by what the same counters read for a plain copy of known size
+# (profiles/gemm_fp16tcec_8192_nn.md).  This is L2-miss traffic on the fabric
+# (Infinity Cache or HBM); the algorithmic minimum is 3 * 8192^2 * 4 B = 0.805e9.
+GEMM_TRAFFIC_BYTES = 5.70e9
 
 
 def log(*a):
@@ -41,6 +46,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the host-core baseline")
     ap.add_argument("--kernel-only", action="store_true",
                     help="time the FP16TCEC GEMM only (no FP64 check, hipBLAS or CPU legs): for profilers")
+    ap.add_argument("--kernel", default="gemm", choices=["gemm", "copy", "exp_stats", "exp_max", "scale", "mx2x2"],
+                    help="with --kernel-only: which kernel to run (copy = a plain device copy of the "
+                         "same bytes, the reference point for the HBM traffic counters)")
     ap.add_argument("--op", default="NN", choices=["NN", "TN", "NT", "TT"])
     ap.add_argument("--mode", default="FP16TCEC", choices=["FP16TCEC", "TF32TCEC", "FP16TC", "TF32TC"])
     args = ap.parse_args()
@@ -61,6 +69,10 @@ def main():
 
     n = args.size
     m = k = n
+    if args.kernel_only and args.kernel != "gemm":
+        hbm_kernel_only(args, torch, cg, inputs, h, dev, stream)
+        h.close()
+        return
     log(f"[bench] generating {n}x{n} inputs (seeds 1, 2)")
     a_host = inputs.uniform(1, m * k)
     b_host = inputs.uniform(2, k * n)
@@ -154,16 +166,26 @@ def main():
         log("[bench] CPU baseline (oracle)")
         from oracle import oracle as O
         O.lib()
-        cn = 4096 if n >= 4096 else n
-        ca, cb = inputs.uniform(1, cn * cn), inputs.uniform(2, cn * cn)
-        cc = np.zeros(cn * cn, np.float32)
         cores = int(os.environ.get("OMP_NUM_THREADS", "0")) or min(os.cpu_count() or 1, 16)
         os.environ["OMP_NUM_THREADS"] = str(cores)
-        t0 = time.perf_counter()
-        O.gemm(O.MODE_FP16TCEC, O.OP_N, O.OP_N, cn, cn, cn, 1.0, ca, cn, cb, cn, 0.0, cc, cn)
-        dt = time.perf_counter() - t0
+
+        def cpu_run(cn):
+            ca, cb = inputs.uniform(1, cn * cn), inputs.uniform(2, cn * cn)
+            cc = np.zeros(cn * cn, np.float32)
+            t0 = time.perf_counter()
+            O.gemm(O.MODE_FP16TCEC, O.OP_N, O.OP_N, cn, cn, cn, 1.0, ca, cn, cb, cn, 0.0, cc, cn)
+            return time.perf_counter() - t0
+
+        # bounded sample: 1/8 of the step first; the whole step only when the
+        # host cores are fast enough to finish it in about half a minute
+        cn = min(n, 4096)
+        dt = cpu_run(cn)
+        if cn < n and dt * (n // cn) ** 3 < 30.0:
+            cn = n
+            dt = cpu_run(cn)
+        frac = "the whole" if cn == n else f"1/{(n // cn) ** 3} of the"
         cpu = {"value": round(2.0 * cn ** 3 / dt / 1e12, 5), "unit": "TFLOP/s", "cores": cores, "kind": "port",
-               "sample": f"one FP16TCEC SGEMM NN {cn}^3 (same generator, seeds 1,2) = 1/{(n // cn) ** 3} of the "
+               "sample": f"one FP16TCEC SGEMM NN {cn}^3 (same generator, seeds 1,2) = {frac} "
                          f"{n}^3 step, split included, {dt:.1f} s"}
 
     out = {
@@ -188,16 +210,18 @@ def main():
         "speedup_vs_hipblas_sgemm": round(value / hb_tflops, 3) if hb_tflops else None,
         "roofline": {
             "bound": "mfma",
-            # MFMA flops actually issued = 3 products x algorithmic 2MNK, over the
-            # kernel's average duration between HIP events on the launch stream
-            "achieved": round(3.0 * kernel_tflops, 1),
+            # algorithmic flops 2MNK of one launch over the kernel's average
+            # duration between HIP events on the launch stream
+            "achieved": round(kernel_tflops, 2),
             "peak": FP16_MFMA_PEAK_TFLOPS,
             "unit": "TFLOP/s",
-            "frac": round(3.0 * kernel_tflops / FP16_MFMA_PEAK_TFLOPS, 4),
-            "traffic": None,
-            "algorithmic_tflops": round(kernel_tflops, 2),
-            "mfma_products_per_flop": 3,
+            "frac": round(kernel_tflops / FP16_MFMA_PEAK_TFLOPS, 4),
+            "traffic": GEMM_TRAFFIC_BYTES if n == 8192 else None,
             "kernel_ms": round(ev_ms, 4),
+            # the split-and-correct algorithm issues 3 MFMA products per logical product
+            "mfma_products_per_flop": 3,
+            "mfma_issued_tflops": round(3.0 * kernel_tflops, 1),
+            "frac_of_emulation_peak": round(3.0 * kernel_tflops / FP16_MFMA_PEAK_TFLOPS, 4),
         },
         "cpu_baseline": cpu,
     }
@@ -205,6 +229,50 @@ def main():
         out["extra"] = extra
     print(json.dumps(out), flush=True)
     h.close()
+
+
+def hbm_kernel_only(args, torch, cg, inputs, h, dev, stream):
+    """One HBM-bound kernel of the path in a loop, for profilers: --size is the
+    matrix order (mx2x2: log2 of M)."""
+    n = args.size
+    if args.kernel == "mx2x2":
+        M = 1 << n
+        x = torch.randn(M * 4, device=dev)
+        u = torch.from_numpy(inputs.random_unitary_2x2(9).view(np.float32)).to(dev)
+        y = torch.zeros(M * 4, device=dev)
+        nbytes = 2.0 * M * 2 * 8
+        fn = lambda: h.gemm_Mx2x2(cg.OP_N, cg.OP_N, M, 1.0, x, M, u, 2, 0.0, y, M, cplx=True)
+    else:
+        a = torch.from_numpy(inputs.exponent_spread(3, n, n, per_row=True)).to(dev)
+        nbytes = 4.0 * n * n
+        if args.kernel == "copy":
+            d = torch.empty_like(a)
+            nbytes *= 2
+            fn = lambda: d.copy_(a)
+        elif args.kernel == "exp_stats":
+            fn = lambda: h.exp_stats_ext(n, n, a, n)
+        elif args.kernel == "exp_max":
+            fn = lambda: h.exp_max_ext(n, n, a, n)
+        else:
+            sid = h.exp_max_ext(n, n, a, n)
+            nbytes *= 2
+            state = [0]
+
+            def fn():
+                (h.reset_scale_A if state[0] & 1 else h.scale_A)(sid, 1, n, n, a, n)
+                state[0] += 1
+    for _ in range(args.warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record(stream)
+    for _ in range(args.steps):
+        fn()
+    e1.record(stream)
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / args.steps
+    print(json.dumps({"kernel_only": True, "kernel": args.kernel, "size": n, "bytes_per_call": nbytes,
+                      "ms_per_call": round(ms, 5), "GBs": round(nbytes / ms / 1e6, 1)}), flush=True)
 
 
 def full_suite(torch, cg, inputs, h, dev, stream, timed, log):

@@ -18,7 +18,11 @@
 namespace cumpsgemm_amd {
 namespace {
 
-constexpr int kBlock = 256;
+// Few, large workgroups: every workgroup ends with one device-scope release
+// fence and one ticket atomic, and on a multi-XCD part those cost far more than
+// the streaming loop itself when thousands of small workgroups queue up on them.
+constexpr int kBlock = 1024;
+constexpr int kWaves = kBlock / 64;
 
 struct Acc {
   float mx;
@@ -61,21 +65,20 @@ __global__ __launch_bounds__(kBlock) void exp_stats_kernel(
     const unsigned long long nvec = (count_f - head) / 4;
     const unsigned long long gsz = (unsigned long long)gridDim.x * kBlock;
     unsigned long long i = (unsigned long long)blockIdx.x * kBlock + tid;
-    for (; i + 3 * gsz < nvec; i += 4 * gsz) {
-      const float4 v0 = body[i], v1 = body[i + gsz], v2 = body[i + 2 * gsz], v3 = body[i + 3 * gsz];
-      count_one(acc, v0.x, ignore_thr, under_thr); count_one(acc, v0.y, ignore_thr, under_thr);
-      count_one(acc, v0.z, ignore_thr, under_thr); count_one(acc, v0.w, ignore_thr, under_thr);
-      count_one(acc, v1.x, ignore_thr, under_thr); count_one(acc, v1.y, ignore_thr, under_thr);
-      count_one(acc, v1.z, ignore_thr, under_thr); count_one(acc, v1.w, ignore_thr, under_thr);
-      count_one(acc, v2.x, ignore_thr, under_thr); count_one(acc, v2.y, ignore_thr, under_thr);
-      count_one(acc, v2.z, ignore_thr, under_thr); count_one(acc, v2.w, ignore_thr, under_thr);
-      count_one(acc, v3.x, ignore_thr, under_thr); count_one(acc, v3.y, ignore_thr, under_thr);
-      count_one(acc, v3.z, ignore_thr, under_thr); count_one(acc, v3.w, ignore_thr, under_thr);
-    }
-    for (; i < nvec; i += gsz) {
-      const float4 v = body[i];
+    auto count4 = [&](const float4 &v) {
       count_one(acc, v.x, ignore_thr, under_thr); count_one(acc, v.y, ignore_thr, under_thr);
       count_one(acc, v.z, ignore_thr, under_thr); count_one(acc, v.w, ignore_thr, under_thr);
+    };
+    // eight independent 16-byte loads in flight per thread
+    for (; i + 7 * gsz < nvec; i += 8 * gsz) {
+      float4 v[8];
+#pragma unroll
+      for (int j = 0; j < 8; j++) v[j] = body[i + j * gsz];
+#pragma unroll
+      for (int j = 0; j < 8; j++) count4(v[j]);
+    }
+    for (; i < nvec; i += gsz) {
+      count4(body[i]);
     }
     if (blockIdx.x == 0) {
       if (tid < head) count_one(acc, ptr[tid], ignore_thr, under_thr);
@@ -83,11 +86,19 @@ __global__ __launch_bounds__(kBlock) void exp_stats_kernel(
       if (tail0 + tid < count_f) count_one(acc, ptr[tail0 + tid], ignore_thr, under_thr);
     }
   } else {
-    // strided view: one column (of m_f floats) per workgroup iteration
+    // strided view: one column (of m_f floats) per wave iteration
     const unsigned long long ncols = (unsigned long long)n * nbatch;
-    for (unsigned long long col = blockIdx.x; col < ncols; col += gridDim.x) {
+    const unsigned lane = tid & 63;
+    for (unsigned long long col = (unsigned long long)blockIdx.x * kWaves + (tid >> 6); col < ncols;
+         col += (unsigned long long)gridDim.x * kWaves) {
       const float *cp = ptr + (col / n) * stride_f + (col % n) * ld_f;
-      for (unsigned i = tid; i < m_f; i += kBlock) count_one(acc, cp[i], ignore_thr, under_thr);
+      unsigned i = lane;
+      for (; i + 192 < m_f; i += 256) {
+        const float x0 = cp[i], x1 = cp[i + 64], x2 = cp[i + 128], x3 = cp[i + 192];
+        count_one(acc, x0, ignore_thr, under_thr); count_one(acc, x1, ignore_thr, under_thr);
+        count_one(acc, x2, ignore_thr, under_thr); count_one(acc, x3, ignore_thr, under_thr);
+      }
+      for (; i < m_f; i += 64) count_one(acc, cp[i], ignore_thr, under_thr);
     }
   }
 
@@ -115,29 +126,37 @@ __global__ __launch_bounds__(kBlock) void exp_stats_kernel(
       t += s_total[w];
       u += s_under[w];
     }
-    StatsPartial p;
-    p.max_bits = __float_as_uint(mx) & 0x7f800000u;
-    p.pad = 0;
-    p.total = t;
-    p.underflow = u;
-    partials[blockIdx.x] = p;
-    __threadfence();
-    const unsigned arrived = atomicAdd(ticket, 1u);
+    // Publish the partial record with device-scope (write-through) stores, wait
+    // for them to be acknowledged, then take a ticket.  A device-scope release
+    // fence here instead would write back the whole L2 once per workgroup, and
+    // those write-backs serialise: they cost several times the streaming loop.
+    StatsPartial *p = partials + blockIdx.x;
+    __hip_atomic_store(&p->max_bits, __float_as_uint(mx) & 0x7f800000u, __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(&p->total, t, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(&p->underflow, u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_waitcnt(0);
+    const unsigned arrived =
+        __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     s_last = (arrived == gridDim.x - 1);
   }
   __syncthreads();
   if (!s_last) return;
 
-  // last workgroup: fold all partials
+  // last workgroup: fold all partials (device-scope loads, independent of each
+  // other so that they are all in flight together)
   __threadfence();
   unsigned mxb = 0;
   unsigned long long t = 0, u = 0;
   for (unsigned i = tid; i < gridDim.x; i += kBlock) {
-    const volatile StatsPartial *p = partials + i;
-    const unsigned b = p->max_bits;
+    StatsPartial *p = partials + i;
+    const unsigned b = __hip_atomic_load(&p->max_bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const unsigned long long pt = __hip_atomic_load(&p->total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const unsigned long long pu = __hip_atomic_load(&p->underflow, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     mxb = b > mxb ? b : mxb;
-    t += p->total;
-    u += p->underflow;
+    t += pt;
+    u += pu;
   }
 #pragma unroll
   for (int off = 32; off >= 1; off >>= 1) {
@@ -183,7 +202,8 @@ __global__ __launch_bounds__(kBlock) void exp_stats_kernel(
     } else {
       slot->max_exp_bits = mxb;
     }
-    *ticket = 0; // ready for the next pass on this stream
+    // ready for the next pass on this stream
+    __hip_atomic_store(ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __threadfence();
   }
 }
@@ -215,9 +235,11 @@ View make_view(const cuMpSGEMM_handle *h, unsigned m, unsigned n, unsigned ld, u
     blocks = (total_f / 4 + kBlock * 4 - 1) / (kBlock * 4);
   } else {
     v.count_f = 0;
-    blocks = (unsigned long long)n * v.nbatch;
+    blocks = ((unsigned long long)n * v.nbatch + kWaves - 1) / kWaves;
   }
-  const unsigned long long cap = std::min<unsigned long long>((unsigned long long)h->num_cus * 8, kMaxStatsBlocks);
+  // one 16-wave workgroup per CU streams at full HBM rate; more workgroups only
+  // lengthen the serial ticket chain at the end
+  const unsigned long long cap = std::min<unsigned long long>((unsigned long long)h->num_cus, kMaxStatsBlocks);
   v.grid = (unsigned)std::max<unsigned long long>(1, std::min(blocks, cap));
   return v;
 }

@@ -61,15 +61,14 @@ __global__ __launch_bounds__(kBlock) void long2x2_kernel(const LongArgs<E> a) {
                       ((uintptr_t)x % 16) == 0 && ((uintptr_t)y % 16) == 0 &&
                       ((a.x_cs * sizeof(E)) % 16) == 0 && ((a.y_cs * sizeof(E)) % 16) == 0;
   if (vec_ok) {
+    // Every byte is touched once: loads and stores bypass the caches' reuse
+    // policy, and two vectors per column are in flight per thread.
+    typedef float f4_t __attribute__((ext_vector_type(4)));
+    union pack_t { f4_t f; vec_t v; };
     const unsigned long long nv = a.L / V;
-    for (; i < nv; i += gsz) {
-      const vec_t x0 = *reinterpret_cast<const vec_t *>(x + i * V);
-      const vec_t x1 = *reinterpret_cast<const vec_t *>(x + a.x_cs + i * V);
-      vec_t y0, y1;
-      if (!bz) {
-        y0 = *reinterpret_cast<const vec_t *>(y + i * V);
-        y1 = *reinterpret_cast<const vec_t *>(y + a.y_cs + i * V);
-      }
+    auto ldv = [](const E *p) { pack_t t; t.f = __builtin_nontemporal_load(reinterpret_cast<const f4_t *>(p)); return t.v; };
+    auto stv = [](E *p, const vec_t &v) { pack_t t; t.v = v; __builtin_nontemporal_store(t.f, reinterpret_cast<f4_t *>(p)); };
+    auto apply = [&](const vec_t &x0, const vec_t &x1, vec_t &y0, vec_t &y1) {
 #pragma unroll
       for (int v = 0; v < V; v++) {
         const E u0 = cj(x0.e[v], a.conj_x), u1 = cj(x1.e[v], a.conj_x);
@@ -82,8 +81,31 @@ __global__ __launch_bounds__(kBlock) void long2x2_kernel(const LongArgs<E> a) {
         y0.e[v] = r0;
         y1.e[v] = r1;
       }
-      *reinterpret_cast<vec_t *>(y + i * V) = y0;
-      *reinterpret_cast<vec_t *>(y + a.y_cs + i * V) = y1;
+    };
+    for (; i + gsz < nv; i += 2 * gsz) {
+      const unsigned long long j = i + gsz;
+      const vec_t xa0 = ldv(x + i * V), xa1 = ldv(x + a.x_cs + i * V);
+      const vec_t xb0 = ldv(x + j * V), xb1 = ldv(x + a.x_cs + j * V);
+      vec_t ya0, ya1, yb0, yb1;
+      if (!bz) {
+        ya0 = ldv(y + i * V); ya1 = ldv(y + a.y_cs + i * V);
+        yb0 = ldv(y + j * V); yb1 = ldv(y + a.y_cs + j * V);
+      }
+      apply(xa0, xa1, ya0, ya1);
+      apply(xb0, xb1, yb0, yb1);
+      stv(y + i * V, ya0); stv(y + a.y_cs + i * V, ya1);
+      stv(y + j * V, yb0); stv(y + a.y_cs + j * V, yb1);
+    }
+    for (; i < nv; i += gsz) {
+      const vec_t x0 = ldv(x + i * V), x1 = ldv(x + a.x_cs + i * V);
+      vec_t y0, y1;
+      if (!bz) {
+        y0 = ldv(y + i * V);
+        y1 = ldv(y + a.y_cs + i * V);
+      }
+      apply(x0, x1, y0, y1);
+      stv(y + i * V, y0);
+      stv(y + a.y_cs + i * V, y1);
     }
     return;
   }
