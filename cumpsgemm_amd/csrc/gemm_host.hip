@@ -92,11 +92,25 @@ struct Plan {
   unsigned tiles_m, tiles_n, ksplit, k_chunk;
 };
 
+// workgroups of this kernel that one CU holds at a time
+unsigned resident_groups(const KernelEntry *e) {
+  const unsigned by_lds = (160u * 1024u) / (unsigned)e->lds_bytes;
+  const unsigned by_regs = (unsigned)(e->occ * 4 * 64) / (unsigned)e->threads;
+  const unsigned r = by_lds < by_regs ? by_lds : by_regs;
+  return r < 1 ? 1 : r;
+}
+
 // Shape -> tile class and split-K factor.  The reference fills "two waves of
-// SMs" (src/cumpsgemm.cu:252-253, x32 for batches :453-454); here a class is
-// accepted when its tiles give every CU at least one resident workgroup set
-// (occ * 4 / waves-per-group groups per CU), else the next smaller tile is
-// tried; if even the smallest tile leaves CUs idle and K is long, K is split.
+// SMs" with its first candidate or falls back to the second
+// (src/cumpsgemm.cu:252-253, x32 for batches :453-454).  Here every class gets
+// a cost from a small model fitted to measurements on MI355X, and the cheapest
+// wins:
+//   cost = rounds * (K-steps + 4) * tile area * resident groups / efficiency
+// rounds     = how many times the chip's CU slots must be refilled,
+// + 4        = a tile's fixed cost (pipeline fill, write-out) in K-steps,
+// efficiency = sustained MFMA rate relative to the 64x64 wave tile, which has
+//              the fewest LDS fragment reads per MFMA (64x32: 0.83, 32x32: 0.55).
+// If even the chosen class leaves CUs idle and K is long, K is split.
 Plan make_plan(const cuMpSGEMM_handle *h, Prec p, bool cplx, bool a_kc, bool b_kc,
                uint64_t m, uint64_t n, uint64_t k, uint64_t batch, int force_cls) {
   Plan plan{};
@@ -104,12 +118,21 @@ Plan make_plan(const cuMpSGEMM_handle *h, Prec p, bool cplx, bool a_kc, bool b_k
   if (force_cls >= 0) {
     cls = force_cls;
   } else {
-    for (cls = 0; cls < kNumTileClasses - 1; cls++) {
-      const KernelEntry *e = lookup_kernel(p, cplx, a_kc, b_kc, cls);
+    double best = 0.0;
+    for (int c = 0; c < kNumTileClasses; c++) {
+      const KernelEntry *e = lookup_kernel(p, cplx, a_kc, b_kc, c);
       const uint64_t tiles = ((m + e->bm - 1) / e->bm) * ((n + e->bn - 1) / e->bn) * batch;
-      // skip a class whose tile is mostly padding for this shape
-      const bool wasteful = (m * 2 <= (uint64_t)e->bm) || (n * 2 <= (uint64_t)e->bn);
-      if (!wasteful && tiles >= (uint64_t)h->num_cus * 2) break;
+      const unsigned res = resident_groups(e);
+      const uint64_t slots = (uint64_t)h->num_cus * res;
+      const double rounds = (double)((tiles + slots - 1) / slots);
+      const int wave_area = e->wm * e->wn;
+      const double eff = wave_area >= 4096 ? 1.0 : (wave_area >= 2048 ? 0.83 : 0.55);
+      const double steps = (double)((k + 31) / 32) + 4.0;
+      const double cost = rounds * steps * (double)e->bm * e->bn * res / eff;
+      if (c == 0 || cost < best) {
+        best = cost;
+        cls = c;
+      }
     }
   }
   const KernelEntry *e = lookup_kernel(p, cplx, a_kc, b_kc, cls);
@@ -132,6 +155,31 @@ Plan make_plan(const cuMpSGEMM_handle *h, Prec p, bool cplx, bool a_kc, bool b_k
   plan.ksplit = ksplit;
   plan.k_chunk = k_chunk;
   return plan;
+}
+
+// The persistent kernels take no edge tiles: every tile interior, every
+// K-chunk a multiple of the 32-wide step and at least four steps long, rows
+// of a K-contiguous operand 16-byte aligned, per-thread offsets within 31 bits.
+template <class T>
+bool persistent_ok(const KernelEntry *e, bool a_kc, bool b_kc, uint64_t m, uint64_t n, uint64_t k,
+                   const Plan &plan, const T *a, uint64_t lda, uint64_t stridea, const T *b,
+                   uint64_t ldb, uint64_t strideb, uint64_t batch) {
+  constexpr uint64_t ES = sizeof(T) / sizeof(float);
+  if (m % e->bm != 0 || n % e->bn != 0 || k % 32 != 0) return false;
+  const uint64_t last_chunk = k - (uint64_t)(plan.ksplit - 1) * plan.k_chunk;
+  if (plan.k_chunk % 32 != 0 || plan.k_chunk < 128 || last_chunk < 128) return false;
+  auto vec_ok = [&](const T *p, uint64_t ld, uint64_t stride) {
+    return ((ld * ES) % 4 == 0) && ((uintptr_t)p % 16 == 0) && (batch == 1 || (stride * ES) % 4 == 0);
+  };
+  if (a_kc && !vec_ok(a, lda, stridea)) return false;
+  if (b_kc && !vec_ok(b, ldb, strideb)) return false;
+  auto fits = [&](bool kc, uint64_t rows, uint64_t ld) {
+    const uint64_t span = kc ? rows * ld + 32 : 32 * ld + rows;
+    return span * ES * 4 < 0x7fffffffull;
+  };
+  if (!fits(a_kc, (uint64_t)e->bm, lda) || !fits(b_kc, (uint64_t)e->bn, ldb)) return false;
+  if ((uint64_t)plan.tiles_m * plan.tiles_n * batch > 0x7fffffffull) return false;
+  return true;
 }
 
 template <class T> struct scalar_parts;
@@ -205,6 +253,8 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
     if (force_cls < 0 || force_cls >= kNumTileClasses) force_cls = -1;
   }
 
+  const bool no_persist = std::getenv("CUMPSGEMM_NO_PERSISTENT") != nullptr;
+
   ProfileScope prof(h, label);
   const bool beta_zero = args.beta_re == 0.0f && args.beta_im == 0.0f;
 
@@ -240,11 +290,21 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
     }
     args.tiles_m = plan.tiles_m;
     args.tiles_n = plan.tiles_n;
+    args.batch = (uint32_t)batch;
     args.k_chunk = plan.k_chunk;
     args.atomic_out = split ? 1u : 0u;
     args.flag_accept_mask = launches[i].accept;
-    const dim3 grid(plan.tiles_m * plan.tiles_n, (unsigned)batch, plan.ksplit);
-    plan.entry->launch(args, grid, h->stream);
+    const KernelEntry *e = plan.entry;
+    if (e->launch_persistent != nullptr && !no_persist &&
+        persistent_ok<T>(e, a_kc, b_kc, m, n, k, plan, a, lda, stridea, b, ldb, strideb, batch)) {
+      const uint64_t slots = (uint64_t)h->num_cus * resident_groups(e);
+      const uint64_t total = (uint64_t)plan.tiles_m * plan.tiles_n * batch;
+      const dim3 grid((unsigned)std::min(total, slots), 1, plan.ksplit);
+      e->launch_persistent(args, grid, h->stream);
+    } else {
+      const dim3 grid(plan.tiles_m * plan.tiles_n, (unsigned)batch, plan.ksplit);
+      e->launch(args, grid, h->stream);
+    }
     if (used_id != nullptr) {
       *used_id = (mode == CUMPSGEMM_AUTO) ? ~0u : (unsigned)plan.cls + (split ? 100u : 0u);
     }

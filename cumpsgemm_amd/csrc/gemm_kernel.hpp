@@ -84,6 +84,7 @@ struct GemmArgs {
   float alpha_re, alpha_im, beta_re, beta_im;
   uint32_t conj_a, conj_b; // complex only: negate imaginary part on load
   uint32_t tiles_m, tiles_n;
+  uint32_t batch;      // persistent kernels walk (tile, batch) pairs themselves
   uint32_t atomic_out; // split-K: C += alpha*acc with float atomics
   // AUTO mode: device flag consulted before doing any work.  The kernel runs
   // only if ((1u << (flag & 31)) & flag_accept_mask) != 0.
@@ -170,11 +171,19 @@ __device__ inline f16v_t mfma32(const u4_t a, const u4_t b, const f16v_t c) {
 //   DEEP: three LDS buffers and an interleaved instruction schedule (MFMAs with
 //         the staging work dripped in between); otherwise two buffers and
 //         plain program order.
+//   PERSIST (DEEP only): one workgroup per CU slot walks a list of tiles and
+//         keeps the load pipeline running across tile boundaries, so that the
+//         first K-steps of the next tile are already in LDS when the current
+//         tile's results are written out.  Interior tiles only (the host
+//         checks divisibility and alignment).
 template <Prec P_, bool CPLX_, bool A_KC_, bool B_KC_, int BM_, int BN_, int WM_,
-          int WN_, int OCC_ = 1, bool DEEP_ = false>
+          int WN_, int OCC_ = 1, bool DEEP_ = false, bool PERSIST_ = false>
 struct GemmCfg {
+  static_assert(!PERSIST_ || DEEP_, "persistent kernels use the three-buffer pipeline");
+  using persistent_type = GemmCfg<P_, CPLX_, A_KC_, B_KC_, BM_, BN_, WM_, WN_, OCC_, DEEP_, DEEP_>;
   static constexpr int OCC = OCC_;
   static constexpr bool DEEP = DEEP_;
+  static constexpr bool PERSIST = PERSIST_;
   static constexpr Prec P = P_;
   static constexpr bool CPLX = CPLX_;
   static constexpr bool A_KC = A_KC_;
@@ -247,6 +256,32 @@ __device__ inline void map_tile(uint32_t bid, uint32_t tiles_m, uint32_t tiles_n
     // XCD x owns a contiguous range; the first r XCDs own one tile more
     id = xcd * q + (xcd < r ? xcd : r) + loc;
   }
+  constexpr uint32_t GROUP = 8;
+  const uint32_t per_group = GROUP * tiles_n;
+  const uint32_t g = id / per_group;
+  const uint32_t first_m = g * GROUP;
+  const uint32_t gsz = (tiles_m - first_m < GROUP) ? (tiles_m - first_m) : GROUP;
+  const uint32_t in = id % per_group;
+  tm = first_m + in % gsz;
+  tn = in / gsz;
+}
+
+// The same for a list of (tile, batch) pairs: the XCD ranges are cut from the
+// whole list, so that one XCD works on neighbouring tiles of one matrix.
+__device__ inline void map_tile_batched(uint32_t vid, uint32_t tiles_m, uint32_t tiles_n,
+                                        uint32_t batch, uint32_t &tm, uint32_t &tn,
+                                        uint32_t &bat) {
+  const uint32_t per_batch = tiles_m * tiles_n;
+  const uint32_t total = per_batch * batch;
+  constexpr uint32_t NXCD = 8;
+  uint32_t id = vid;
+  if (total >= NXCD * 4) {
+    const uint32_t q = total / NXCD, r = total % NXCD;
+    const uint32_t xcd = vid % NXCD, loc = vid / NXCD;
+    id = xcd * q + (xcd < r ? xcd : r) + loc;
+  }
+  bat = id / per_batch;
+  id -= bat * per_batch;
   constexpr uint32_t GROUP = 8;
   const uint32_t per_group = GROUP * tiles_n;
   const uint32_t g = id / per_group;
@@ -445,25 +480,31 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
   const int wm = wave % (BM / Cfg::WM);
   const int wn = wave / (BM / Cfg::WM);
 
-  uint32_t tile_m, tile_n;
-  map_tile(blockIdx.x, args.tiles_m, args.tiles_n, tile_m, tile_n);
+  // (persistent kernels: the first tile of this workgroup's list; see below)
+  uint32_t tile_m, tile_n, tile_b = blockIdx.y;
+  if constexpr (Cfg::PERSIST) {
+    map_tile_batched(blockIdx.x, args.tiles_m, args.tiles_n, args.batch, tile_m, tile_n, tile_b);
+  } else {
+    map_tile(blockIdx.x, args.tiles_m, args.tiles_n, tile_m, tile_n);
+  }
   const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
   const uint32_t kbeg = blockIdx.z * args.k_chunk;
   const uint32_t kend = (kbeg + args.k_chunk < args.k) ? kbeg + args.k_chunk : args.k;
   if (kbeg >= kend) return;
 
   const float *a = reinterpret_cast<const float *>(args.a) +
-                   (uint64_t)blockIdx.y * args.stride_a * ES;
+                   (uint64_t)tile_b * args.stride_a * ES;
   const float *b = reinterpret_cast<const float *>(args.b) +
-                   (uint64_t)blockIdx.y * args.stride_b * ES;
+                   (uint64_t)tile_b * args.stride_b * ES;
   float *c = reinterpret_cast<float *>(args.c) +
-             (uint64_t)blockIdx.y * args.stride_c * ES;
+             (uint64_t)tile_b * args.stride_c * ES;
 
   // operand tile origins at k = kbeg
   const float *a_tile = Cfg::A_KC ? a + ((uint64_t)m0 * args.lda + kbeg) * ES
                                   : a + ((uint64_t)kbeg * args.lda + m0) * ES;
   const float *b_tile = Cfg::B_KC ? b + ((uint64_t)n0 * args.ldb + kbeg) * ES
                                   : b + ((uint64_t)kbeg * args.ldb + n0) * ES;
+  // (not const: a persistent kernel moves them from tile to tile)
   const uint64_t a_kstep = Cfg::A_KC ? (uint64_t)BK * ES : (uint64_t)BK * args.lda * ES;
   const uint64_t b_kstep = Cfg::B_KC ? (uint64_t)BK * ES : (uint64_t)BK * args.ldb * ES;
 
@@ -601,6 +642,157 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
     frag_mma(f1);
   };
 
+  // ---- epilogue -----------------------------------------------------------
+  // 32x32 accumulator layout: register v of lane l holds
+  //   MFMA row (-> n) = 8*(v/4) + 4*(l/32) + v%4,  MFMA column (-> m) = l%32
+  // so the 32 lanes of a half-wave write 128 contiguous bytes of a C column.
+  // FULL: interior tile, no bounds checks.
+  const bool beta_zero = (args.beta_re == 0.0f) && (!CPLX || args.beta_im == 0.0f);
+  auto epilogue = [&](float *cb, const uint32_t em0, const uint32_t en0, auto full_tag) {
+    constexpr bool FULL = decltype(full_tag)::value;
+#pragma unroll
+    for (int j = 0; j < TN; j++)
+#pragma unroll
+      for (int i = 0; i < TM; i++) {
+        const uint32_t mm = em0 + wm * Cfg::WM + i * 32 + (lane & 31);
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+          const uint32_t nn = en0 + wn * Cfg::WN + j * 32 + 8 * (v / 4) + 4 * (lane >> 5) + (v & 3);
+          if (FULL || (mm < args.m && nn < args.n)) {
+            float *cp = cb + ((uint64_t)nn * args.ldc + mm) * ES;
+            if constexpr (!CPLX) {
+              float x = acc[0][0][j][i][v];
+              if constexpr (PT::NACC == 2) x += acc[0][1][j][i][v] * PT::CORR_SCALE;
+              if (args.atomic_out) {
+                atomicAdd(cp, x * args.alpha_re);
+              } else if (beta_zero) {
+                *cp = x * args.alpha_re;
+              } else {
+                *cp = x * args.alpha_re + args.beta_re * (*cp);
+              }
+            } else {
+              float x = acc[0][0][j][i][v], y = acc[1][0][j][i][v];
+              if constexpr (PT::NACC == 2) {
+                x += acc[0][1][j][i][v] * PT::CORR_SCALE;
+                y += acc[1][1][j][i][v] * PT::CORR_SCALE;
+              }
+              float rx = x * args.alpha_re - y * args.alpha_im;
+              float ry = y * args.alpha_re + x * args.alpha_im;
+              if (args.atomic_out) {
+                atomicAdd(cp, rx);
+                atomicAdd(cp + 1, ry);
+              } else {
+                if (!beta_zero) {
+                  const float2 old = *reinterpret_cast<const float2 *>(cp);
+                  rx = x * args.alpha_re - y * args.alpha_im +
+                       (args.beta_re * old.x - args.beta_im * old.y);
+                  ry = y * args.alpha_re + x * args.alpha_im +
+                       (args.beta_im * old.x + args.beta_re * old.y);
+                }
+                *reinterpret_cast<float2 *>(cp) = make_float2(rx, ry);
+              }
+            }
+          }
+        }
+      }
+  };
+  auto zero_acc = [&]() {
+#pragma unroll
+    for (int q = 0; q < NCOMP; q++)
+#pragma unroll
+      for (int s = 0; s < PT::NACC; s++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+          for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[q][s][j][i][v] = 0.0f;
+  };
+
+  if constexpr (Cfg::PERSIST) {
+    // ---- persistent walk over this workgroup's tiles ----------------------
+    // Tile i of the list is virtual workgroup blockIdx.x + i * gridDim.x.  The
+    // K-steps of all tiles form one stream: the loader runs three steps ahead
+    // of the multiplier straight across tile boundaries, so when a tile's
+    // results are written out the next tile's first steps are already in LDS.
+    // Requires >= 4 K-steps per tile (the loader's "next tile" origin is
+    // refreshed when the multiplier changes tile, three steps after the loader
+    // did).  Every tile is interior and aligned (checked by the host).
+    const uint32_t total = args.tiles_m * args.tiles_n * args.batch;
+    const uint32_t my_tiles = (total - blockIdx.x + gridDim.x - 1) / gridDim.x;
+    const int nk = klen / BK;
+    auto origin = [&](uint32_t i, const float *&at, const float *&bt, float *&ct, uint32_t &om0,
+                      uint32_t &on0) {
+      uint32_t tm, tn, bat;
+      map_tile_batched(blockIdx.x + (i < my_tiles ? i : my_tiles - 1) * gridDim.x, args.tiles_m,
+                       args.tiles_n, args.batch, tm, tn, bat);
+      om0 = tm * BM;
+      on0 = tn * BN;
+      const float *ab = reinterpret_cast<const float *>(args.a) + (uint64_t)bat * args.stride_a * ES;
+      const float *bb = reinterpret_cast<const float *>(args.b) + (uint64_t)bat * args.stride_b * ES;
+      ct = reinterpret_cast<float *>(args.c) + (uint64_t)bat * args.stride_c * ES;
+      at = Cfg::A_KC ? ab + ((uint64_t)om0 * args.lda + kbeg) * ES
+                     : ab + ((uint64_t)kbeg * args.lda + om0) * ES;
+      bt = Cfg::B_KC ? bb + ((uint64_t)on0 * args.ldb + kbeg) * ES
+                     : bb + ((uint64_t)kbeg * args.ldb + on0) * ES;
+    };
+    const float *a_next, *b_next; // origin of the tile after the one being loaded
+    const float *a_unused, *b_unused;
+    float *c_cur = c, *c_unused;
+    uint32_t cm0 = m0, cn0 = n0, u0, u1;
+    origin(1, a_next, b_next, c_unused, u0, u1);
+    int lk = 0;
+    auto gnext = [&]() {
+      gload(0, std::true_type{});
+      lk++;
+      const bool wrap = (lk == nk);
+      a_tile = wrap ? a_next : a_tile + a_kstep;
+      b_tile = wrap ? b_next : b_tile + b_kstep;
+      lk = wrap ? 0 : lk;
+    };
+    Frags f0, f1;
+    gnext();
+    lstore(0);
+    gnext();
+    lstore(1);
+    gnext();
+    block_sync_lds();
+    frag_load(f0, 0, 0);
+    int b0 = 0, b1 = 1, b2 = 2;
+    int ck = 0;
+    uint32_t ct = 0;
+    const uint32_t steps = my_tiles * (uint32_t)nk;
+    for (uint32_t s = 0; s < steps; s++) {
+      frag_load(f1, b0, 1);
+      frag_mma(f0);
+      frag_mma(f1);
+      lstore(b2);
+      gnext();
+      frag_load(f0, b1, 0);
+#pragma unroll
+      for (int g = 0; g < 2 * PT::NPROD * TM * TN * (CPLX ? 4 : 1); g++) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); // MFMA
+        __builtin_amdgcn_sched_group_barrier(0x002, 4, 0); // VALU
+        __builtin_amdgcn_sched_group_barrier(0x080, 1, 0); // DS
+        __builtin_amdgcn_sched_group_barrier(0x020, 1, 0); // VMEM read
+      }
+      block_sync_lds();
+      const int tmp = b0;
+      b0 = b1;
+      b1 = b2;
+      b2 = tmp;
+      if (++ck == nk) { // tile complete: write it out, move on
+        epilogue(c_cur, cm0, cn0, std::true_type{});
+        zero_acc();
+        ck = 0;
+        ct++;
+        origin(ct, a_unused, b_unused, c_cur, cm0, cn0);
+        origin(ct + 1, a_next, b_next, c_unused, u0, u1);
+      }
+    }
+    return;
+  }
+
   // The K loop over `nk` steps.  Two separate instances (fast / guarded loads)
   // keep the rarely used guarded code out of the hot loop.  Loads past the last
   // tile re-read the last one (never staged), which keeps the loop body free of
@@ -689,55 +881,7 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
     pipeline((klen + BK - 1) / BK, std::false_type{});
   }
 
-  // ---- epilogue -----------------------------------------------------------
-  // 32x32 accumulator layout: register v of lane l holds
-  //   MFMA row (-> n) = 8*(v/4) + 4*(l/32) + v%4,  MFMA column (-> m) = l%32
-  const bool beta_zero = (args.beta_re == 0.0f) && (!CPLX || args.beta_im == 0.0f);
-#pragma unroll
-  for (int j = 0; j < TN; j++)
-#pragma unroll
-    for (int i = 0; i < TM; i++) {
-      const uint32_t mm = m0 + wm * Cfg::WM + i * 32 + (lane & 31);
-#pragma unroll
-      for (int v = 0; v < 16; v++) {
-        const uint32_t nn = n0 + wn * Cfg::WN + j * 32 + 8 * (v / 4) + 4 * (lane >> 5) + (v & 3);
-        if (mm < args.m && nn < args.n) {
-          float *cp = c + ((uint64_t)nn * args.ldc + mm) * ES;
-          if constexpr (!CPLX) {
-            float x = acc[0][0][j][i][v];
-            if constexpr (PT::NACC == 2) x += acc[0][1][j][i][v] * PT::CORR_SCALE;
-            if (args.atomic_out) {
-              atomicAdd(cp, x * args.alpha_re);
-            } else if (beta_zero) {
-              *cp = x * args.alpha_re;
-            } else {
-              *cp = x * args.alpha_re + args.beta_re * (*cp);
-            }
-          } else {
-            float x = acc[0][0][j][i][v], y = acc[1][0][j][i][v];
-            if constexpr (PT::NACC == 2) {
-              x += acc[0][1][j][i][v] * PT::CORR_SCALE;
-              y += acc[1][1][j][i][v] * PT::CORR_SCALE;
-            }
-            float rx = x * args.alpha_re - y * args.alpha_im;
-            float ry = y * args.alpha_re + x * args.alpha_im;
-            if (args.atomic_out) {
-              atomicAdd(cp, rx);
-              atomicAdd(cp + 1, ry);
-            } else {
-              if (!beta_zero) {
-                const float2 old = *reinterpret_cast<const float2 *>(cp);
-                rx = x * args.alpha_re - y * args.alpha_im +
-                     (args.beta_re * old.x - args.beta_im * old.y);
-                ry = y * args.alpha_re + x * args.alpha_im +
-                     (args.beta_im * old.x + args.beta_re * old.y);
-              }
-              *reinterpret_cast<float2 *>(cp) = make_float2(rx, ry);
-            }
-          }
-        }
-      }
-    }
+  epilogue(c, m0, n0, std::false_type{});
 }
 
 // C (m x n, ldc, batched) *= beta before a split-K accumulation, or = 0.

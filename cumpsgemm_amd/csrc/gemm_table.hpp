@@ -11,6 +11,9 @@ namespace cumpsgemm_amd {
 
 struct KernelEntry {
   void (*launch)(const GemmArgs &, dim3 grid, hipStream_t stream);
+  // persistent variant (grid.x = CU slots, walks tiles and batches itself), or
+  // nullptr; only for shapes made of interior, aligned tiles
+  void (*launch_persistent)(const GemmArgs &, dim3 grid, hipStream_t stream);
   int bm, bn;      // workgroup tile
   int wm, wn;      // wave tile
   int threads;     // workgroup size
@@ -38,8 +41,16 @@ void launch_cfg(const GemmArgs &args, dim3 grid, hipStream_t stream) {
 }
 
 template <class Cfg> constexpr KernelEntry make_entry(const char *name) {
-  return KernelEntry{&launch_cfg<Cfg>, Cfg::BM,  Cfg::BN,        Cfg::WM,  Cfg::WN,
-                     Cfg::NT,          Cfg::LDS_BYTES, Cfg::OCC, name};
+  if constexpr (Cfg::DEEP) {
+    return KernelEntry{&launch_cfg<Cfg>, &launch_cfg<typename Cfg::persistent_type>,
+                       Cfg::BM,          Cfg::BN,
+                       Cfg::WM,          Cfg::WN,
+                       Cfg::NT,          Cfg::LDS_BYTES,
+                       Cfg::OCC,         name};
+  } else {
+    return KernelEntry{&launch_cfg<Cfg>, nullptr,        Cfg::BM,  Cfg::BN, Cfg::WM,
+                       Cfg::WN,          Cfg::NT,        Cfg::LDS_BYTES, Cfg::OCC, name};
+  }
 }
 
 // Per-(precision, type) tables, one translation unit each (gemm_inst_*.hip).

@@ -178,3 +178,72 @@ def test_invalid_arguments(handle, dev, cg):
     assert handle.gemm(N, N, 8, 8, 8, 1.0, x, 4, x, 8, 0.0, x, 8, cg.FP16TCEC) == cg.STATUS_INVALID_VALUE
     assert handle.gemm(N, N, 8, 8, 8, 1.0, x, 8, x, 8, 0.0, x, 7, cg.FP16TCEC) == cg.STATUS_INVALID_VALUE
     assert handle.gemm(N, N, 0, 8, 8, 1.0, x, 8, x, 8, 0.0, x, 8, cg.FP16TCEC) == cg.STATUS_SUCCESS
+
+
+# ---- persistent (tile-walking) kernels -----------------------------------------
+# Shapes made of interior, aligned tiles run on kernels in which one workgroup
+# per CU slot walks a list of (tile, batch) pairs with the load pipeline running
+# across tile boundaries.  They perform the same arithmetic in the same order as
+# the one-tile-per-workgroup kernels, so the two must agree bit for bit; the
+# environment switches select the tile class and turn the persistent path off.
+def _with_env(monkeypatch, cls, persistent):
+    monkeypatch.setenv("CUMPSGEMM_FORCE_TILE_CLASS", str(cls))
+    if persistent:
+        monkeypatch.delenv("CUMPSGEMM_NO_PERSISTENT", raising=False)
+    else:
+        monkeypatch.setenv("CUMPSGEMM_NO_PERSISTENT", "1")
+
+
+@pytest.mark.parametrize("cls", [0, 1])
+@pytest.mark.parametrize("mode", [FP16TCEC, TF32TCEC])
+@pytest.mark.parametrize("cplx,opa,opb,m,n,k,batch,alpha,beta", [
+    (False, N, N, 4096, 4096, 128, 1, 1.0, 0.0),     # 512 / 1024 tiles of 4 K-steps: every workgroup walks several
+    (False, T, N, 2048, 1024, 160, 3, 0.75, -0.5),   # batches in the walk, beta != 0
+    (False, N, T, 1024, 2048, 352, 2, 1.0, 0.0),
+    (False, T, T, 512, 512, 128, 9, 1.0, 1.0),
+    (True, N, N, 1024, 1024, 128, 3, 1.0, 0.0),
+    (True, C, N, 512, 1024, 192, 5, 0.5, 0.25),
+    (True, N, C, 512, 512, 224, 6, 1.0, 0.0),
+])
+def test_persistent_kernels_match_plain_kernels(O, handle, dev, monkeypatch, cls, mode, cplx, opa, opb,
+                                                m, n, k, batch, alpha, beta):
+    gen = _gen(cplx)
+    ar, ac = (m, k) if opa == N else (k, m)
+    br, bc = (k, n) if opb == N else (n, k)
+    sa, sb, sc = ar * ac, br * bc, m * n
+    a, b, c0 = gen(11, sa * batch), gen(12, sb * batch), gen(13, sc * batch)
+    da, db = dev.up(a), dev.up(b)
+    outs = []
+    for persistent in (True, False):
+        _with_env(monkeypatch, cls, persistent)
+        dc = dev.up(c0)
+        st = handle.gemm_strided_batch(opa, opb, m, n, k, alpha, da, ar, sa, db, br, sb, beta, dc, m, sc,
+                                       batch, mode, cplx=cplx)
+        assert st == 0
+        outs.append(dev.down(dc, np.complex64 if cplx else np.float32))
+    assert np.array_equal(outs[0], outs[1])
+    # and the result is right: last batch entry against FP64 and the FP32 error
+    i = batch - 1
+    ai, bi, ci0 = a[i * sa:(i + 1) * sa], b[i * sb:(i + 1) * sb], c0[i * sc:(i + 1) * sc]
+    ref = O.gemm_fp64(opa, opb, m, n, k, alpha, ai, ar, bi, br, beta, ci0, m)
+    cf = oracle_gemm(O, FP32, opa, opb, m, n, k, alpha, ai, ar, bi, br, beta, ci0, m)
+    got = outs[0][i * sc:(i + 1) * sc]
+    assert O.residual(ref, got, m, n, m) <= 2.0 * O.residual(ref, cf, m, n, m) + 2.0 ** -23
+
+
+def test_persistent_split_k(O, handle, dev, monkeypatch):
+    # few tiles, long K: K is cut into chunks and each chunk's tiles are walked
+    m, n, k = 256, 256, 16384
+    a, b = inputs.uniform(21, m * k), inputs.uniform(22, k * n)
+    c0 = inputs.uniform(23, m * n)
+    outs = []
+    for persistent in (True, False):
+        _with_env(monkeypatch, 1, persistent)
+        c, st, mid = run_gemm(handle, dev, FP16TCEC, N, N, m, n, k, 1.0, a, m, b, k, 0.5, c0, m, False,
+                              want_module_id=True)
+        assert st == 0 and mid == 101
+        outs.append(c)
+    ref = O.gemm_fp64(N, N, m, n, k, 1.0, a, m, b, k, 0.5, c0, m)
+    cf = oracle_gemm(O, FP32, N, N, m, n, k, 1.0, a, m, b, k, 0.5, c0, m)
+    for c in outs:  # atomic accumulation order differs from run to run
+        assert O.residual(ref, c, m, n, m) <= 2.0 * O.residual(ref, cf, m, n, m)
