@@ -82,7 +82,7 @@ struct GemmArgs {
   uint64_t lda, ldb, ldc;                // in elements
   uint64_t stride_a, stride_b, stride_c; // in elements, per blockIdx.y
   float alpha_re, alpha_im, beta_re, beta_im;
-  uint32_t conj_a, conj_b; // complex only: negate imaginary part on load
+  uint32_t conj_a, conj_b; // complex only: op C (the sign is applied when the partial products are combined)
   uint32_t tiles_m, tiles_n;
   uint32_t batch;      // persistent kernels walk (tile, batch) pairs themselves
   uint32_t atomic_out; // split-K: C += alpha*acc with float atomics
@@ -383,22 +383,28 @@ struct tile_loader {
       for (int u = 0; u < U; u++) {
 #pragma unroll
         for (int j = 0; j < 8; j++) {
-#pragma unroll
-          for (int c = 0; c < NC; c++)
-            reg.v[u][c][j] = __builtin_bit_cast(
-                float, __builtin_amdgcn_raw_buffer_load_b32(rsrc, boff[u] + 4 * c, j * line, 0));
+          if constexpr (!CPLX) {
+            reg.v[u][0][j] = __builtin_bit_cast(
+                float, __builtin_amdgcn_raw_buffer_load_b32(rsrc, boff[u], j * line, 0));
+          } else {
+            // one 8-byte load per complex element.  The loaded pair is taken
+            // apart as a 64-bit integer: extracting the elements of the vector
+            // result directly is what this toolchain mis-narrows.
+            typedef unsigned int u2_t __attribute__((ext_vector_type(2)));
+            const u2_t t = __builtin_amdgcn_raw_buffer_load_b64(rsrc, boff[u], j * line, 0);
+            const uint64_t w = __builtin_bit_cast(uint64_t, t);
+            reg.v[u][0][j] = __builtin_bit_cast(float, (uint32_t)w);
+            reg.v[u][1][j] = __builtin_bit_cast(float, (uint32_t)(w >> 32));
+          }
         }
       }
     }
   }
 
   // The 8 K-values (re, im) of unit u, ready to be split.
-  __device__ static inline void fetch(Regs &reg, int u, bool conj, f8_t &re, f8_t &im) {
+  __device__ static inline void fetch(Regs &reg, int u, f8_t &re, f8_t &im) {
     re = reg.v[u][0];
-    if constexpr (CPLX) {
-      im = reg.v[u][1];
-      if (conj) im = -im;
-    }
+    if constexpr (CPLX) im = reg.v[u][1];
   }
 
   // edge tile / unaligned / huge ld: element-wise and guarded.  The branches
@@ -433,7 +439,7 @@ struct tile_loader {
 
   // split and write to LDS: planes laid out [comp][plane][row][chunk]
   template <Prec P>
-  __device__ static inline void store(Regs &reg, char *lds_op, int tid, bool conj) {
+  __device__ static inline void store(Regs &reg, char *lds_op, int tid) {
     constexpr int NP = prec_traits<P>::NP;
     constexpr int PLANE = ROWS * 64;
     if (!active(tid)) return;
@@ -442,7 +448,7 @@ struct tile_loader {
       int row, chunk;
       unit_coords(u, tid, row, chunk);
       f8_t part[2];
-      fetch(reg, u, conj, part[0], part[1]);
+      fetch(reg, u, part[0], part[1]);
 #pragma unroll
       for (int c = 0; c < NC; c++) {
         u4_t out[NP];
@@ -532,9 +538,14 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
   // accumulators: [component][main/corr][TN][TM]; MFMA rows run along N and
   // MFMA columns along M so that a lane's 64 outputs of one register are 32
   // consecutive M-values -> coalesced column-major stores.
-  f16v_t acc[NCOMP][PT::NACC][TN][TM];
+  // Complex: the four real products ar*br, ai*bi, ar*bi, ai*br are kept apart
+  // and combined -- with the signs that op C asks for -- when the tile is
+  // written out, so neither the subtraction nor a conjugation costs a single
+  // vector instruction in the K loop.
+  constexpr int NACCSET = CPLX ? 4 : 1;
+  f16v_t acc[NACCSET][PT::NACC][TN][TM];
 #pragma unroll
-  for (int q = 0; q < NCOMP; q++)
+  for (int q = 0; q < NACCSET; q++)
 #pragma unroll
     for (int s = 0; s < PT::NACC; s++)
 #pragma unroll
@@ -563,8 +574,8 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
   auto lstore = [&](int stage) {
     char *sa = lds + stage * Cfg::STAGE_BYTES;
     char *sb = sa + Cfg::A_STAGE_BYTES;
-    LA::template store<P>(ra, sa, tid, args.conj_a);
-    LB::template store<P>(rb, sb, tid, args.conj_b);
+    LA::template store<P>(ra, sa, tid);
+    LB::template store<P>(rb, sb, tid);
   };
 
   // Per-lane fragment addresses.  Lane l of a 32x32x16 MFMA supplies row
@@ -613,12 +624,6 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
             acc[0][PT::ACC[t]][j][i] = mfma32<PT::IS_BF16>(
                 f.b[0][PT::PB[t]][j], f.a[0][PT::PA[t]][i], acc[0][PT::ACC[t]][j][i]);
     } else {
-      // -Im(A) planes for the real part: re = ar*br + (-ai)*bi
-      u4_t fan[NP][TM];
-#pragma unroll
-      for (int p = 0; p < NP; p++)
-#pragma unroll
-        for (int i = 0; i < TM; i++) fan[p][i] = f.a[1][p][i] ^ 0x80008000u;
 #pragma unroll
       for (int t = 0; t < PT::NPROD; t++)
 #pragma unroll
@@ -627,9 +632,9 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
           for (int i = 0; i < TM; i++) {
             const int s = PT::ACC[t], pa = PT::PA[t], pb = PT::PB[t];
             acc[0][s][j][i] = mfma32<PT::IS_BF16>(f.b[0][pb][j], f.a[0][pa][i], acc[0][s][j][i]);
-            acc[1][s][j][i] = mfma32<PT::IS_BF16>(f.b[1][pb][j], f.a[0][pa][i], acc[1][s][j][i]);
-            acc[0][s][j][i] = mfma32<PT::IS_BF16>(f.b[1][pb][j], fan[pa][i], acc[0][s][j][i]);
-            acc[1][s][j][i] = mfma32<PT::IS_BF16>(f.b[0][pb][j], f.a[1][pa][i], acc[1][s][j][i]);
+            acc[1][s][j][i] = mfma32<PT::IS_BF16>(f.b[1][pb][j], f.a[1][pa][i], acc[1][s][j][i]);
+            acc[2][s][j][i] = mfma32<PT::IS_BF16>(f.b[1][pb][j], f.a[0][pa][i], acc[2][s][j][i]);
+            acc[3][s][j][i] = mfma32<PT::IS_BF16>(f.b[0][pb][j], f.a[1][pa][i], acc[3][s][j][i]);
           }
     }
   };
@@ -648,6 +653,8 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
   // so the 32 lanes of a half-wave write 128 contiguous bytes of a C column.
   // FULL: interior tile, no bounds checks.
   const bool beta_zero = (args.beta_re == 0.0f) && (!CPLX || args.beta_im == 0.0f);
+  const float sgn_a = args.conj_a ? -1.0f : 1.0f, sgn_b = args.conj_b ? -1.0f : 1.0f;
+  const float sgn_ab = sgn_a * sgn_b;
   auto epilogue = [&](float *cb, const uint32_t em0, const uint32_t en0, auto full_tag) {
     constexpr bool FULL = decltype(full_tag)::value;
 #pragma unroll
@@ -671,11 +678,16 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
                 *cp = x * args.alpha_re + args.beta_re * (*cp);
               }
             } else {
-              float x = acc[0][0][j][i][v], y = acc[1][0][j][i][v];
-              if constexpr (PT::NACC == 2) {
-                x += acc[0][1][j][i][v] * PT::CORR_SCALE;
-                y += acc[1][1][j][i][v] * PT::CORR_SCALE;
+              // re = ar*br - sa*sb*ai*bi, im = sb*ar*bi + sa*ai*br with
+              // sa (sb) = -1 when op(A) (op(B)) conjugates
+              float p[4];
+#pragma unroll
+              for (int q = 0; q < 4; q++) {
+                p[q] = acc[q][0][j][i][v];
+                if constexpr (PT::NACC == 2) p[q] += acc[q][1][j][i][v] * PT::CORR_SCALE;
               }
+              const float x = p[0] - sgn_ab * p[1];
+              const float y = sgn_b * p[2] + sgn_a * p[3];
               float rx = x * args.alpha_re - y * args.alpha_im;
               float ry = y * args.alpha_re + x * args.alpha_im;
               if (args.atomic_out) {
@@ -698,7 +710,7 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
   };
   auto zero_acc = [&]() {
 #pragma unroll
-    for (int q = 0; q < NCOMP; q++)
+    for (int q = 0; q < NACCSET; q++)
 #pragma unroll
       for (int s = 0; s < PT::NACC; s++)
 #pragma unroll
