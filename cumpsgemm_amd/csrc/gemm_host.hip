@@ -295,15 +295,24 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
     args.atomic_out = split ? 1u : 0u;
     args.flag_accept_mask = launches[i].accept;
     const KernelEntry *e = plan.entry;
-    if (e->launch_persistent != nullptr && !no_persist &&
+    auto launch_plain = e->launch;
+    auto launch_walk = e->launch_persistent;
+    if (h->fused_scaling && launches[i].p == Prec::FP16TCEC) {
+      launch_plain = e->launch_scaled;
+      launch_walk = e->launch_scaled_persistent;
+      args.scale_max_a = &h->stats_slots[h->fused_slot_a].max_exp_bits;
+      args.scale_max_b = &h->stats_slots[h->fused_slot_b].max_exp_bits;
+      args.scale_flag = h->flag_buffer + h->fused_flag;
+    }
+    if (launch_walk != nullptr && !no_persist &&
         persistent_ok<T>(e, a_kc, b_kc, m, n, k, plan, a, lda, stridea, b, ldb, strideb, batch)) {
       const uint64_t slots = (uint64_t)h->num_cus * resident_groups(e);
       const uint64_t total = (uint64_t)plan.tiles_m * plan.tiles_n * batch;
       const dim3 grid((unsigned)std::min(total, slots), 1, plan.ksplit);
-      e->launch_persistent(args, grid, h->stream);
+      launch_walk(args, grid, h->stream);
     } else {
       const dim3 grid(plan.tiles_m * plan.tiles_n, (unsigned)batch, plan.ksplit);
-      e->launch(args, grid, h->stream);
+      launch_plain(args, grid, h->stream);
     }
     if (used_id != nullptr) {
       *used_id = (mode == CUMPSGEMM_AUTO) ? ~0u : (unsigned)plan.cls + (split ? 100u : 0u);

@@ -90,6 +90,12 @@ struct GemmArgs {
   // only if ((1u << (flag & 31)) & flag_accept_mask) != 0.
   const int *launch_flag;
   uint32_t flag_accept_mask;
+  // SCALED kernels: power-of-two scaling fused into the split (A, B) and the
+  // write-out (C).  The coefficients come from device memory -- the maximum
+  // exponents recorded by the statistics passes and the scale bits of a launch
+  // flag -- so that no host synchronisation is needed.
+  const uint32_t *scale_max_a, *scale_max_b; // bits of 2^floor(log2 max|x|)
+  const int *scale_flag;                     // bit 6: scale A, bit 5: scale B
 };
 
 // ---- split one group of 8 FP32 values into NP packed 16-byte plane chunks ----
@@ -116,12 +122,40 @@ __device__ inline uint32_t split_pair_fp16(const float x0, const float x1, uint3
   return hi;
 }
 
+// The same split of (x * s), s a power of two held in a scalar register (s2048
+// = s * 2^11): hi = fp16(x * s) comes from the mixed-precision FMA as well, so
+// the scaling costs one more instruction per pair, not one per element.
+__device__ inline uint32_t split_pair_fp16_scaled(const float x0, const float x1, const float s,
+                                                  const float s2048, uint32_t &lo) {
+  uint32_t hi;
+  asm("v_fma_mixlo_f16 %0, %1, %2, 0 op_sel_hi:[0,0,0]" : "=v"(hi) : "v"(x0), "s"(s));
+  asm("v_fma_mixhi_f16 %0, %1, %2, 0 op_sel_hi:[0,0,0]" : "+v"(hi) : "v"(x1), "s"(s));
+  const float t0 = x0 * s2048, t1 = x1 * s2048;
+  const float k = -2048.0f;
+  uint32_t l;
+  asm("v_fma_mixlo_f16 %0, %1, %2, %3 op_sel_hi:[1,0,0]" : "=v"(l) : "v"(hi), "s"(k), "v"(t0));
+  asm("v_fma_mixhi_f16 %0, %1, %2, %3 op_sel:[1,0,0] op_sel_hi:[1,0,0]"
+      : "+v"(l)
+      : "v"(hi), "s"(k), "v"(t1));
+  lo = l;
+  return hi;
+}
+
 template <> struct splitter<Prec::FP16TCEC> {
   __device__ static inline void run(const f8_t x, u4_t (&out)[2]) {
 #pragma unroll
     for (int i = 0; i < 4; i++) {
       uint32_t lo;
       out[0][i] = split_pair_fp16(x[2 * i], x[2 * i + 1], lo);
+      out[1][i] = lo;
+    }
+  }
+  __device__ static inline void run_scaled(const f8_t x, u4_t (&out)[2], const float s,
+                                           const float s2048) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      uint32_t lo;
+      out[0][i] = split_pair_fp16_scaled(x[2 * i], x[2 * i + 1], s, s2048, lo);
       out[1][i] = lo;
     }
   }
@@ -176,11 +210,19 @@ __device__ inline f16v_t mfma32(const u4_t a, const u4_t b, const f16v_t c) {
 //         first K-steps of the next tile are already in LDS when the current
 //         tile's results are written out.  Interior tiles only (the host
 //         checks divisibility and alignment).
+//   SCALED (FP16TCEC only): op(A), op(B) are multiplied by powers of two read
+//         from device memory while they are split, and the result by the
+//         inverse product when it is written out (see GemmArgs).
 template <Prec P_, bool CPLX_, bool A_KC_, bool B_KC_, int BM_, int BN_, int WM_,
-          int WN_, int OCC_ = 1, bool DEEP_ = false, bool PERSIST_ = false>
+          int WN_, int OCC_ = 1, bool DEEP_ = false, bool PERSIST_ = false, bool SCALED_ = false>
 struct GemmCfg {
   static_assert(!PERSIST_ || DEEP_, "persistent kernels use the three-buffer pipeline");
-  using persistent_type = GemmCfg<P_, CPLX_, A_KC_, B_KC_, BM_, BN_, WM_, WN_, OCC_, DEEP_, DEEP_>;
+  static_assert(!SCALED_ || P_ == Prec::FP16TCEC, "scaling guards the fp16 range only");
+  using persistent_type =
+      GemmCfg<P_, CPLX_, A_KC_, B_KC_, BM_, BN_, WM_, WN_, OCC_, DEEP_, DEEP_, SCALED_>;
+  using scaled_type = GemmCfg<P_, CPLX_, A_KC_, B_KC_, BM_, BN_, WM_, WN_, OCC_, DEEP_, PERSIST_,
+                              P_ == Prec::FP16TCEC>;
+  static constexpr bool SCALED = SCALED_;
   static constexpr int OCC = OCC_;
   static constexpr bool DEEP = DEEP_;
   static constexpr bool PERSIST = PERSIST_;
@@ -438,8 +480,10 @@ struct tile_loader {
   }
 
   // split and write to LDS: planes laid out [comp][plane][row][chunk]
-  template <Prec P>
-  __device__ static inline void store(Regs &reg, char *lds_op, int tid) {
+  // SCALED: the values are multiplied by s (s2048 = s * 2^11) on the way
+  template <Prec P, bool SCALED = false>
+  __device__ static inline void store(Regs &reg, char *lds_op, int tid, float s = 1.0f,
+                                      float s2048 = 2048.0f) {
     constexpr int NP = prec_traits<P>::NP;
     constexpr int PLANE = ROWS * 64;
     if (!active(tid)) return;
@@ -452,7 +496,11 @@ struct tile_loader {
 #pragma unroll
       for (int c = 0; c < NC; c++) {
         u4_t out[NP];
-        splitter<P>::run(part[c], out);
+        if constexpr (SCALED) {
+          splitter<P>::run_scaled(part[c], out, s, s2048);
+        } else {
+          splitter<P>::run(part[c], out);
+        }
 #pragma unroll
         for (int p = 0; p < NP; p++) {
           *reinterpret_cast<u4_t *>(lds_op + (c * NP + p) * PLANE + lds_offset(row, chunk)) = out[p];
@@ -477,6 +525,26 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
     const int flag = *args.launch_flag;
     if (((1u << (flag & 31)) & args.flag_accept_mask) == 0) return;
   }
+
+  // Fused power-of-two scaling (same coefficients as the stand-alone scaling
+  // kernels: 2^14 / max for a flagged, non-zero operand, and the inverse
+  // product for C).  All uniform, in scalar registers.
+  float coef_a = 1.0f, coef_b = 1.0f, coef_c = 1.0f;
+  if constexpr (Cfg::SCALED) {
+    const int sflag = *args.scale_flag;
+    const float ma = __uint_as_float(*args.scale_max_a), mb = __uint_as_float(*args.scale_max_b);
+    if ((sflag & 0x40) && ma != 0.0f) {
+      coef_a = 16384.0f / ma;
+      coef_c *= ma / 16384.0f;
+    }
+    if ((sflag & 0x20) && mb != 0.0f) {
+      coef_b = 16384.0f / mb;
+      coef_c *= mb / 16384.0f;
+    }
+  }
+  const float coef_a2048 = coef_a * 2048.0f, coef_b2048 = coef_b * 2048.0f;
+  // alpha with the inverse scaling of C folded in (exact: a power of two)
+  const float alpha_re = args.alpha_re * coef_c, alpha_im = args.alpha_im * coef_c;
 
   extern __shared__ __attribute__((aligned(16))) char lds[];
 
@@ -574,8 +642,8 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
   auto lstore = [&](int stage) {
     char *sa = lds + stage * Cfg::STAGE_BYTES;
     char *sb = sa + Cfg::A_STAGE_BYTES;
-    LA::template store<P>(ra, sa, tid);
-    LB::template store<P>(rb, sb, tid);
+    LA::template store<P, Cfg::SCALED>(ra, sa, tid, coef_a, coef_a2048);
+    LB::template store<P, Cfg::SCALED>(rb, sb, tid, coef_b, coef_b2048);
   };
 
   // Per-lane fragment addresses.  Lane l of a 32x32x16 MFMA supplies row
@@ -671,11 +739,11 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
               float x = acc[0][0][j][i][v];
               if constexpr (PT::NACC == 2) x += acc[0][1][j][i][v] * PT::CORR_SCALE;
               if (args.atomic_out) {
-                atomicAdd(cp, x * args.alpha_re);
+                atomicAdd(cp, x * alpha_re);
               } else if (beta_zero) {
-                *cp = x * args.alpha_re;
+                *cp = x * alpha_re;
               } else {
-                *cp = x * args.alpha_re + args.beta_re * (*cp);
+                *cp = x * alpha_re + args.beta_re * (*cp);
               }
             } else {
               // re = ar*br - sa*sb*ai*bi, im = sb*ar*bi + sa*ai*br with
@@ -688,17 +756,17 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
               }
               const float x = p[0] - sgn_ab * p[1];
               const float y = sgn_b * p[2] + sgn_a * p[3];
-              float rx = x * args.alpha_re - y * args.alpha_im;
-              float ry = y * args.alpha_re + x * args.alpha_im;
+              float rx = x * alpha_re - y * alpha_im;
+              float ry = y * alpha_re + x * alpha_im;
               if (args.atomic_out) {
                 atomicAdd(cp, rx);
                 atomicAdd(cp + 1, ry);
               } else {
                 if (!beta_zero) {
                   const float2 old = *reinterpret_cast<const float2 *>(cp);
-                  rx = x * args.alpha_re - y * args.alpha_im +
+                  rx = x * alpha_re - y * alpha_im +
                        (args.beta_re * old.x - args.beta_im * old.y);
-                  ry = y * args.alpha_re + x * args.alpha_im +
+                  ry = y * alpha_re + x * alpha_im +
                        (args.beta_im * old.x + args.beta_re * old.y);
                 }
                 *reinterpret_cast<float2 *>(cp) = make_float2(rx, ry);

@@ -14,6 +14,10 @@ struct KernelEntry {
   // persistent variant (grid.x = CU slots, walks tiles and batches itself), or
   // nullptr; only for shapes made of interior, aligned tiles
   void (*launch_persistent)(const GemmArgs &, dim3 grid, hipStream_t stream);
+  // variants with the power-of-two scaling of A, B and C fused in (FP16TCEC
+  // tables only, else nullptr)
+  void (*launch_scaled)(const GemmArgs &, dim3 grid, hipStream_t stream);
+  void (*launch_scaled_persistent)(const GemmArgs &, dim3 grid, hipStream_t stream);
   int bm, bn;      // workgroup tile
   int wm, wn;      // wave tile
   int threads;     // workgroup size
@@ -41,16 +45,23 @@ void launch_cfg(const GemmArgs &args, dim3 grid, hipStream_t stream) {
 }
 
 template <class Cfg> constexpr KernelEntry make_entry(const char *name) {
-  if constexpr (Cfg::DEEP) {
-    return KernelEntry{&launch_cfg<Cfg>, &launch_cfg<typename Cfg::persistent_type>,
-                       Cfg::BM,          Cfg::BN,
-                       Cfg::WM,          Cfg::WN,
-                       Cfg::NT,          Cfg::LDS_BYTES,
-                       Cfg::OCC,         name};
-  } else {
-    return KernelEntry{&launch_cfg<Cfg>, nullptr,        Cfg::BM,  Cfg::BN, Cfg::WM,
-                       Cfg::WN,          Cfg::NT,        Cfg::LDS_BYTES, Cfg::OCC, name};
+  KernelEntry e{};
+  e.launch = &launch_cfg<Cfg>;
+  if constexpr (Cfg::DEEP) e.launch_persistent = &launch_cfg<typename Cfg::persistent_type>;
+  if constexpr (Cfg::P == Prec::FP16TCEC) {
+    e.launch_scaled = &launch_cfg<typename Cfg::scaled_type>;
+    if constexpr (Cfg::DEEP)
+      e.launch_scaled_persistent = &launch_cfg<typename Cfg::scaled_type::persistent_type>;
   }
+  e.bm = Cfg::BM;
+  e.bn = Cfg::BN;
+  e.wm = Cfg::WM;
+  e.wn = Cfg::WN;
+  e.threads = Cfg::NT;
+  e.lds_bytes = Cfg::LDS_BYTES;
+  e.occ = Cfg::OCC;
+  e.name = name;
+  return e;
 }
 
 // Per-(precision, type) tables, one translation unit each (gemm_inst_*.hip).

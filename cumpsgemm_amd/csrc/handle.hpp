@@ -68,6 +68,12 @@ struct cuMpSGEMM_handle {
   bool flag_enabled = false;
   unsigned flag_enabled_id = 0;
 
+  // While set, FP16TCEC GEMMs apply the power-of-two scaling of these
+  // statistics slots / this launch flag inside the kernel (the mode pipelines
+  // switch it on around their GEMM when A and B are to be left untouched).
+  bool fused_scaling = false;
+  unsigned fused_slot_a = 0, fused_slot_b = 0, fused_flag = 0;
+
   // pinned host word for small read-backs
   unsigned long long *host_scratch = nullptr; // [4]
 

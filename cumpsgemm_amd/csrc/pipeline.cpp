@@ -4,6 +4,7 @@
 // synchronisation.  Follows the orchestration of the reference's interposer,
 // src/cumpsgemm_cublas.cu:446-577 (single) and :836-960 (strided batch).
 #include "pipeline.hpp"
+#include <cstdlib>
 #include "handle.hpp"
 #include <cumpsgemm/cumpsgemm_ext.h>
 
@@ -28,20 +29,40 @@ hipblasStatus_t gemm_pipeline(cuMpSGEMM_handle_t h, hipblasOperation_t op_A,
 
   unsigned a_id = 0, b_id = 0, flag_id = 0;
   const bool scaled = (mode == CUMPSGEMM_AUTO || mode == CUMPSGEMM_FP16TCEC_SCALING);
+  // When A and B are to come out unchanged (restore_AB, the default) the
+  // scaling is fused into the GEMM kernel: A and B are multiplied while they
+  // are split and C on the way out, so A and B are never written and five
+  // read-modify-write passes over A, B and C disappear.  The reference scales
+  // A and B in place through a const_cast and undoes it afterwards
+  // (src/cumpsgemm_cublas.cu:511-518, :562-573); that form is kept for callers
+  // that ask for the scaled operands to be left behind (restore_AB == false).
+  // One deliberate difference: with beta != 0 the fused form computes
+  // alpha*A*B + beta*C, while rescaling the finished C also rescales beta*C.
+  const bool fused = scaled && restore_AB && std::getenv("CUMPSGEMM_NO_FUSED_SCALING") == nullptr;
   if (mode == CUMPSGEMM_AUTO) {
     a_id = cumpsgemm::exp_stats_ext<T>(h, a_rows, a_cols, a, (unsigned)lda, sb, sa_stride);
     b_id = cumpsgemm::exp_stats_ext<T>(h, b_rows, b_cols, b, (unsigned)ldb, sb, sb_stride);
     flag_id = cumpsgemm::get_next_dynamic_launch_buffer_id(h);
     cumpsgemm::set_dynamic_launch_buffer_by_exp_stats(h, flag_id, a_id, b_id);
-    cumpsgemm::scale_A<T>(h, a_id, flag_id, a_rows, a_cols, a, (unsigned)lda, sb, sa_stride);
-    cumpsgemm::scale_B<T>(h, b_id, flag_id, b_rows, b_cols, b, (unsigned)ldb, sb, sb_stride);
+    if (!fused) {
+      cumpsgemm::scale_A<T>(h, a_id, flag_id, a_rows, a_cols, a, (unsigned)lda, sb, sa_stride);
+      cumpsgemm::scale_B<T>(h, b_id, flag_id, b_rows, b_cols, b, (unsigned)ldb, sb, sb_stride);
+    }
     cumpsgemm::set_dynamic_launch_flag_buffer_id(h, flag_id);
   } else if (mode == CUMPSGEMM_FP16TCEC_SCALING) {
     flag_id = 1; // preset: FP16TCEC with both scale bits
     a_id = cumpsgemm::exp_max_ext<T>(h, a_rows, a_cols, a, (unsigned)lda, sb, sa_stride);
     b_id = cumpsgemm::exp_max_ext<T>(h, b_rows, b_cols, b, (unsigned)ldb, sb, sb_stride);
-    cumpsgemm::scale_A<T>(h, a_id, flag_id, a_rows, a_cols, a, (unsigned)lda, sb, sa_stride);
-    cumpsgemm::scale_B<T>(h, b_id, flag_id, b_rows, b_cols, b, (unsigned)ldb, sb, sb_stride);
+    if (!fused) {
+      cumpsgemm::scale_A<T>(h, a_id, flag_id, a_rows, a_cols, a, (unsigned)lda, sb, sa_stride);
+      cumpsgemm::scale_B<T>(h, b_id, flag_id, b_rows, b_cols, b, (unsigned)ldb, sb, sb_stride);
+    }
+  }
+  if (fused) {
+    h->fused_scaling = true;
+    h->fused_slot_a = a_id;
+    h->fused_slot_b = b_id;
+    h->fused_flag = flag_id;
   }
   const cuMpSGEMM_compute_mode_t gemm_mode =
       (mode == CUMPSGEMM_FP16TCEC_SCALING) ? CUMPSGEMM_FP16TCEC : mode;
@@ -53,7 +74,8 @@ hipblasStatus_t gemm_pipeline(cuMpSGEMM_handle_t h, hipblasOperation_t op_A,
     st = cumpsgemm::gemm<T>(h, op_A, op_B, m, n, k, alpha, a, lda, b, ldb, beta, c, ldc,
                             gemm_mode);
   }
-  if (scaled) {
+  h->fused_scaling = false;
+  if (scaled && !fused) {
     cumpsgemm::scale_C<T>(h, a_id, b_id, flag_id, (unsigned)m, (unsigned)n, c, (unsigned)ldc, sb,
                           sc_stride);
     if (restore_AB) {
@@ -62,8 +84,8 @@ hipblasStatus_t gemm_pipeline(cuMpSGEMM_handle_t h, hipblasOperation_t op_A,
       cumpsgemm::reset_scale_B<T>(h, b_id, flag_id, b_rows, b_cols, b, (unsigned)ldb, sb,
                                   sb_stride);
     }
-    if (mode == CUMPSGEMM_AUTO) cumpsgemm::unset_dynamic_launch_flag_buffer_id(h);
   }
+  if (mode == CUMPSGEMM_AUTO) cumpsgemm::unset_dynamic_launch_flag_buffer_id(h);
   if (ids != nullptr) {
     ids->a_slot = a_id;
     ids->b_slot = b_id;

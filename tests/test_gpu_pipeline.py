@@ -109,3 +109,37 @@ def test_auto_complex_batched(O, handle, dev):
         ref = O.gemm_fp64(N, N, m, n, k, 1.0, a[i * m * k:], m, b[i * k * n:], k)
         cf = oracle_gemm(O, FP32, N, N, m, n, k, 1.0, a[i * m * k:], m, b[i * k * n:], k, 0.0, np.zeros(m * n, np.complex64), m)
         assert O.residual(ref, c[i * m * n:(i + 1) * m * n], m, n, m) <= 2.0 * O.residual(ref, cf, m, n, m)
+
+
+@pytest.mark.parametrize("mode", [SCALING, AUTO])
+@pytest.mark.parametrize("cplx,opa,opb,m,n,k", [
+    (False, N, N, 512, 384, 256),    # interior tiles: persistent fused kernels
+    (False, T, N, 200, 130, 100),    # edge tiles
+    (False, N, T, 256, 256, 4096),   # split-K
+    (True, N, N, 256, 128, 192),
+    (True, T, T, 70, 90, 50),
+])
+def test_fused_scaling_matches_in_place_scaling(O, handle, dev, monkeypatch, mode, cplx, opa, opb, m, n, k):
+    """The pipelines scale A, B and C inside the GEMM kernel; the stand-alone
+    passes (scale A, B in place, GEMM, scale C, undo) must give the same bits:
+    every factor is a power of two."""
+    gen = (lambda s, c: inputs.complex_normal(s, c, 1.0)) if cplx else inputs.uniform
+    a = (gen(31, m * k) * np.float32(2.0 ** -21)).astype(np.complex64 if cplx else np.float32)
+    b = (gen(32, k * n) * np.float32(2.0 ** -3)).astype(np.complex64 if cplx else np.float32)
+    outs = []
+    for fused in (True, False):
+        if fused:
+            monkeypatch.delenv("CUMPSGEMM_NO_FUSED_SCALING", raising=False)
+        else:
+            monkeypatch.setenv("CUMPSGEMM_NO_FUSED_SCALING", "1")
+        c, a_after, b_after, ids = _pipeline(handle, dev, mode, opa, opb, m, n, k, a, b, cplx=cplx)
+        assert np.array_equal(a_after.view(np.uint32), a.view(np.uint32))
+        assert np.array_equal(b_after.view(np.uint32), b.view(np.uint32))
+        outs.append(c)
+    if k <= 2048:  # split-K accumulates with atomics: order, hence bits, vary
+        assert np.array_equal(outs[0].view(np.uint32), outs[1].view(np.uint32))
+    ref = O.gemm_fp64(opa, opb, m, n, k, 1.0, a, m if opa == N else k, b, k if opb == N else n)
+    cf = oracle_gemm(O, FP32, opa, opb, m, n, k, 1.0, a, m if opa == N else k, b, k if opb == N else n, 0.0,
+                     np.zeros(m * n, a.dtype), m)
+    for c in outs:
+        assert O.residual(ref, c, m, n, m) <= 2.0 * O.residual(ref, cf, m, n, m)
