@@ -12,6 +12,7 @@
 #include <cumpsgemm/cumpsgemm.hpp>
 #include <cumpsgemm/cumpsgemm_ext.h>
 #include <cumpsgemm/hijack_control.hpp>
+#include <ctime>
 #include <dlfcn.h>
 #include <mutex>
 #include <sstream>
@@ -182,6 +183,49 @@ hipblasStatus_t forward_gemm_sb(hipblasHandle_t hb, hipblasOperation_t op_A,
 }
 
 // One intercepted call.  batched == false: strides are ignored, batch == 1.
+// Per-call wall-clock profiling of intercepted GEMMs, switched on by
+// CUMPSGEMM_ENABLE_CULIP_PROFILING (any value but "0").  The stream is drained
+// before the first and after the second timestamp, and one line
+//   [CULiP Result][<label>] <nanoseconds>ns
+// goes to stdout, with the labels of reference src/cumpsgemm_cublas.cu:270-297,
+// :393-416, :430-441, :648-677, :780-806, :812-822 and the line format of
+// src/culip.cu:19-33 (existing log parsers keep working).
+bool culip_enabled() {
+  const char *v = std::getenv("CUMPSGEMM_ENABLE_CULIP_PROFILING");
+  return v != nullptr && std::string(v) != "0";
+}
+struct CulipScope {
+  bool on;
+  hipStream_t stream;
+  std::string label;
+  struct timespec t0;
+  CulipScope(bool enabled, hipStream_t st, const std::string &name, hipblasOperation_t op_A,
+             hipblasOperation_t op_B, long m, long n, long k, bool batched, long batch)
+      : on(enabled), stream(st) {
+    if (!on) return;
+    char buf[128];
+    if (batched)
+      std::snprintf(buf, sizeof(buf), "%s-%s%s-m%lu-n%lu-k%lu-batchCount%lu", name.c_str(), op_str(op_A),
+                    op_str(op_B), (unsigned long)m, (unsigned long)n, (unsigned long)k,
+                    (unsigned long)batch);
+    else
+      std::snprintf(buf, sizeof(buf), "%s-%s%s-m%lu-n%lu-k%lu", name.c_str(), op_str(op_A), op_str(op_B),
+                    (unsigned long)m, (unsigned long)n, (unsigned long)k);
+    label = buf;
+    (void)hipStreamSynchronize(stream);
+    clock_gettime(CLOCK_MONOTONIC, &t0);
+  }
+  ~CulipScope() {
+    if (!on) return;
+    (void)hipStreamSynchronize(stream);
+    struct timespec t1;
+    clock_gettime(CLOCK_MONOTONIC, &t1);
+    const long ns = ((long)t1.tv_sec - (long)t0.tv_sec) * 1000000000L + ((long)t1.tv_nsec - (long)t0.tv_nsec);
+    std::printf("[CULiP Result][%s] %luns\n", label.c_str(), (unsigned long)ns);
+    std::fflush(stdout);
+  }
+};
+
 template <class T>
 hipblasStatus_t hijack_core(const char *func_name, hipblasHandle_t hb, hipblasOperation_t op_A,
                             hipblasOperation_t op_B, int m, int n, int k, const T *alpha,
@@ -215,7 +259,13 @@ hipblasStatus_t hijack_core(const char *func_name, hipblasHandle_t hb, hipblasOp
   const uint64_t usa = batched ? (uint64_t)sa : 0, usb = batched ? (uint64_t)sb : 0,
                  usc = batched ? (uint64_t)sc : 0;
 
+  const bool culip = culip_enabled();
+  const std::string sc_prefix = std::is_same<T, float>::value ? "s" : "c";
+  const hipStream_t cstream = caller_stream(hb);
+
   if (mx2x2_enabled() && n == 2 && k == 2 && is_pow2((uint64_t)m)) {
+    CulipScope prof(culip, cstream, sc_prefix + (batched ? "gemm_strided_batch_Mx2x2" : "gemm_Mx2x2"), op_A,
+                    op_B, m, n, k, batched, batch);
     log_info(" +---> gemm_Mx2x2");
     if constexpr (std::is_same<T, float>::value)
       return cuMpSGEMM_sgemm_Mx2x2(h, op_A, op_B, m, alpha, a, lda, usa, b, ldb, usb, beta, c, ldc,
@@ -225,6 +275,8 @@ hipblasStatus_t hijack_core(const char *func_name, hipblasHandle_t hb, hipblasOp
                                    usc, nb);
   }
   if (mx2x2_enabled() && m == 2 && k == 2 && is_pow2((uint64_t)n)) {
+    CulipScope prof(culip, cstream, sc_prefix + (batched ? "gemm_strided_batch_2xNx2" : "gemm_2xNx2"), op_A,
+                    op_B, m, n, k, batched, batch);
     log_info(" +---> gemm_2xNx2");
     if constexpr (std::is_same<T, float>::value)
       return cuMpSGEMM_sgemm_2xNx2(h, op_A, op_B, n, alpha, a, lda, usa, b, ldb, usb, beta, c, ldc,
@@ -235,6 +287,7 @@ hipblasStatus_t hijack_core(const char *func_name, hipblasHandle_t hb, hipblasOp
   }
 
   if (forwards_to_hipblas(mode)) {
+    CulipScope prof(culip, cstream, func_name, op_A, op_B, m, n, k, batched, batch);
     const hipblasStatus_t st =
         batched ? forward_gemm_sb<T>(hb, op_A, op_B, m, n, k, alpha, a, lda, sa, b, ldb, sb, beta,
                                      c, ldc, sc, batch)
@@ -254,7 +307,11 @@ hipblasStatus_t hijack_core(const char *func_name, hipblasHandle_t hb, hipblasOp
                                         beta, c, ldc, sc, batch)
                    : forward_gemm<T>(hb, op_A, op_B, m, n, k, alpha, a, lda, b, ldb, beta, c, ldc);
   }
-  // the scaled modes write A and B in place and restore them afterwards
+  CulipScope prof(culip, cstream,
+                  sc_prefix + (batched ? "gemm_stridedBatch_" : "gemm_") +
+                      cuMpSGEMM_get_compute_mode_string(mode),
+                  op_A, op_B, m, n, k, batched, batch);
+  // unless restore_AB is off the scaled modes leave A and B untouched
   return gemm_pipeline<T>(h, op_A, op_B, m, n, k, alpha, const_cast<T *>(a), lda, usa,
                           const_cast<T *>(b), ldb, usb, beta, c, ldc, usc, nb, batched, mode,
                           g_restore_AB, nullptr);
@@ -429,6 +486,27 @@ size_t cuMpSGEMM_hijack_get_last_called_function_str(char *buf, size_t buf_len) 
 }
 void cuMpSGEMM_hijack_clear_last_called_function_str(void) { g_last_called.clear(); }
 int cuMpSGEMM_hijack_is_library_loaded(void) { return 1; }
+void cuMpSGEMM_hijack_set_last_called_function_str(const char *str) {
+  g_last_called = (str != nullptr) ? str : "";
+}
+void cuMpSGEMM_hijack_reset_exp_stats_buffer_id(void) {
+  cumpsgemm::hijack_control::reset_exp_stats_buffer_id();
+}
+void cuMpSGEMM_hijack_set_exp_stats_params(float ignore_threshold, float underflow_threshold,
+                                           float underflow_tolerance_rate) {
+  cumpsgemm::hijack_control::set_exp_stats_params(ignore_threshold, underflow_threshold,
+                                                  underflow_tolerance_rate);
+}
+void cuMpSGEMM_hijack_set_control_function(cuMpSGEMM_control_function_t fn) {
+  if (fn == nullptr) {
+    cumpsgemm::hijack_control::unset_control_function();
+    return;
+  }
+  cumpsgemm::hijack_control::set_control_function(
+      [fn](const int op_A, const int op_B, const unsigned m, const unsigned n, const unsigned k) {
+        return (cuMpSGEMM_compute_mode_t)fn(op_A, op_B, m, n, k);
+      });
+}
 int cuMpSGEMM_hijack_query_compute_mode(const char *func_name, int op_A, int op_B, unsigned m,
                                         unsigned n, unsigned k) {
   return (int)query_mode(func_name, nullptr, (hipblasOperation_t)op_A, (hipblasOperation_t)op_B, m,

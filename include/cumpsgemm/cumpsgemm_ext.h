@@ -162,6 +162,16 @@ void cuMpSGEMM_hijack_set_restore_AB(int enable);
 size_t cuMpSGEMM_hijack_get_last_called_function_str(char *buf, size_t buf_len);
 void cuMpSGEMM_hijack_clear_last_called_function_str(void);
 int cuMpSGEMM_hijack_is_library_loaded(void);
+void cuMpSGEMM_hijack_set_last_called_function_str(const char *str);
+void cuMpSGEMM_hijack_reset_exp_stats_buffer_id(void);
+/* thresholds of the AUTO decision on the interposer's handle (creates it) */
+void cuMpSGEMM_hijack_set_exp_stats_params(float ignore_threshold, float underflow_threshold,
+                                           float underflow_tolerance_rate);
+/* hijack_control::set_control_function with a plain function pointer:
+ * (op_A, op_B, m, n, k) -> cuMpSGEMM_compute_mode_t value; NULL removes it
+ * (reference hijack_control.hpp:28-31, python/src/main.cpp:81-88). */
+typedef int (*cuMpSGEMM_control_function_t)(int op_A, int op_B, unsigned m, unsigned n, unsigned k);
+void cuMpSGEMM_hijack_set_control_function(cuMpSGEMM_control_function_t fn);
 /* The mode the interposer would choose for a call (static mode, control
  * function, rule library, built-in rule -- in that order). */
 int cuMpSGEMM_hijack_query_compute_mode(const char *func_name, int op_A, int op_B, unsigned m,

@@ -80,3 +80,26 @@ def test_preload_dry_run_leaves_c_untouched():
     res, logs = _probe({"CUMPSGEMM_COMPUTE_MODE": "DRY_RUN", "CUMPSGEMM_INFO": "1"})
     assert res["hipblasSgemm"] == (0, 1.0)  # C stayed zero: relative error exactly 1
     assert any("mode=DRY_RUN" in l for l in logs)
+
+
+def test_culip_profiling_lines():
+    """CUMPSGEMM_ENABLE_CULIP_PROFILING prints one '[CULiP Result][label] Nns'
+    line per intercepted call, labels as in the reference
+    (src/cumpsgemm_cublas.cu:430-441, :812-822, :393-398; src/culip.cu:19-33)."""
+    assert os.path.exists(PROBE)
+    env = dict(os.environ)
+    env.update({"CUMPSGEMM_COMPUTE_MODE": "FP16TCEC", "CUMPSGEMM_ENABLE_CULIP_PROFILING": "1"})
+    env["LD_PRELOAD"] = LIB + (":" + env["LD_PRELOAD"] if env.get("LD_PRELOAD") else "")
+    r = subprocess.run([PROBE], env=env, text=True, capture_output=True, timeout=300)
+    assert r.returncode == 0 and "DONE" in r.stdout
+    lines = re.findall(r"^\[CULiP Result\]\[(\S+)\] (\d+)ns$", r.stdout, flags=re.M)
+    labels = [l for l, _ in lines]
+    assert "sgemm_FP16TCEC-NN-m1280-n1280-k1280" in labels
+    assert "sgemm_FP16TCEC-TN-m1280-n1280-k1280" in labels
+    assert "sgemm_stridedBatch_FP16TCEC-NN-m1280-n1280-k1280-batchCount3" in labels
+    assert "hipblasCgemm-CN-m640-n640-k640" in labels  # forwarded call: the symbol's own name
+    assert all(int(ns) > 0 for _, ns in lines)
+    # off by default and with "0"
+    env["CUMPSGEMM_ENABLE_CULIP_PROFILING"] = "0"
+    r0 = subprocess.run([PROBE], env=env, text=True, capture_output=True, timeout=300)
+    assert "[CULiP Result]" not in r0.stdout

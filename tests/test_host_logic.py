@@ -203,3 +203,51 @@ def test_missing_library_fails_loudly(tmp_path):
     r = subprocess.run([sys.executable, "-c", textwrap.dedent(code)], env=env, text=True, capture_output=True)
     assert r.returncode == 0, r.stderr
     assert r.stdout.strip() == "raised: True"
+
+
+# ---- Python control module (counterpart of the reference's pybind11 module,
+# python/src/main.cpp:111-173) ------------------------------------------------
+CTL_PROBE = """
+    import ctypes
+    from cumpsgemm_amd import cumpsgemm_hijack_control as ctl
+    print(ctl.is_library_loaded())
+    q = ctypes.CDLL(None)
+    def query(m):
+        try:
+            f = q.cuMpSGEMM_hijack_query_compute_mode
+        except AttributeError:
+            return -1
+        f.argtypes = [ctypes.c_char_p, ctypes.c_int, ctypes.c_int, ctypes.c_uint, ctypes.c_uint, ctypes.c_uint]
+        return f(b"hipblasSgemm", 111, 111, m, 2048, 2048)
+    print(query(2048))
+    ctl.set_control_function(lambda op_a, op_b, m, n, k: ctl.CUMPSGEMM_TF32TCEC if m == 4096 else ctl.CUMPSGEMM_FP16TC)
+    print(query(4096), query(2048))
+    ctl.set_compute_mode(ctl.CUMPSGEMM_DRY_RUN); print(query(4096))
+    ctl.unset_compute_mode(); ctl.unset_control_function(); print(query(4096))
+    ctl.set_last_called_function_str("abc,N,N,1,2,3,1,FP16TCEC"); print(ctl.get_last_called_function_str())
+    ctl.clear_last_called_function_str(); print(repr(ctl.get_last_called_function_str()))
+    ctl.enable_custom_gemm_Mx2x2(); ctl.disable_custom_gemm_Mx2x2()
+    ctl.disable_restoring_AB_after_scaling(); ctl.enable_restoring_AB_after_scaling()
+    ctl.enable_auto_kernel_selection(); print(ctl.is_auto_kernel_selection_enabled())
+    ctl.set_global_cublas_dim_mn_threshold(256); print(ctl.get_global_cublas_dim_mn_threshold(), ctl.get_global_cublas_dim_k_threshold())
+    print(int(ctl.compute_mode.CUMPSGEMM_AUTO), int(ctl.CUMPSGEMM_CUBLAS_SIMT))
+"""
+
+
+def test_python_control_module_without_preload_is_inert():
+    out = _run(CTL_PROBE, {"CUMPSGEMM_COMPUTE_MODE": "FP16TCEC"}).strip().splitlines()
+    assert out[0] == "False" and out[1] == "-1"
+    assert out[2] == "-1 -1" and out[5] == "" and out[6] == "''"
+    assert out[7] == "True" and out[8] == "256 64" and out[9] == "9 5"
+
+
+def test_python_control_module_drives_the_preloaded_library(cg):
+    preload = cg.lib_path() + (":" + os.environ["LD_PRELOAD"] if os.environ.get("LD_PRELOAD") else "")
+    out = _run(CTL_PROBE, {"CUMPSGEMM_COMPUTE_MODE": "FP16TCEC", "LD_PRELOAD": preload}).strip().splitlines()
+    assert out[0] == "True"
+    assert out[1] == "1"               # rule: env mode for dims > 1024
+    assert out[2] == "2 3"             # control function consulted per call
+    assert out[3] == "8"               # a forced mode outranks it
+    assert out[4] == "1"               # both removed: back to the rule
+    assert out[5] == "abc,N,N,1,2,3,1,FP16TCEC" and out[6] == "''"
+    assert out[7] == "True" and out[8] == "256 64" and out[9] == "9 5"
