@@ -741,7 +741,8 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
               if (args.atomic_out) {
                 atomicAdd(cp, x * alpha_re);
               } else if (beta_zero) {
-                *cp = x * alpha_re;
+                // the result is not read again by this kernel: streaming store
+                __builtin_nontemporal_store(x * alpha_re, cp);
               } else {
                 *cp = x * alpha_re + args.beta_re * (*cp);
               }
@@ -769,7 +770,10 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
                   ry = y * alpha_re + x * alpha_im +
                        (args.beta_im * old.x + args.beta_re * old.y);
                 }
-                *reinterpret_cast<float2 *>(cp) = make_float2(rx, ry);
+                // the result is not read again by this kernel: streaming store
+                typedef float f2v_t __attribute__((ext_vector_type(2)));
+                f2v_t out2 = {rx, ry};
+                __builtin_nontemporal_store(out2, reinterpret_cast<f2v_t *>(cp));
               }
             }
           }
