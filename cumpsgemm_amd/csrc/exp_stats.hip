@@ -118,28 +118,33 @@ __global__ __launch_bounds__(kBlock) void exp_stats_kernel(
     s_under[tid >> 6] = acc.under;
   }
   __syncthreads();
-  if (tid == 0) {
-    float mx = 0.0f;
-    unsigned long long t = 0, u = 0;
-    for (int w = 0; w < kBlock / 64; w++) {
-      mx = fmaxf(mx, s_mx[w]);
-      t += s_total[w];
-      u += s_under[w];
+  if (tid < 64) {
+    // first wave: fold the per-wave results with a second butterfly
+    float mx = tid < kWaves ? s_mx[tid] : 0.0f;
+    unsigned long long t = tid < kWaves ? s_total[tid] : 0ull;
+    unsigned long long u = tid < kWaves ? s_under[tid] : 0ull;
+#pragma unroll
+    for (int off = kWaves / 2; off >= 1; off >>= 1) {
+      mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+      t += __shfl_xor(t, off, 64);
+      u += __shfl_xor(u, off, 64);
     }
-    // Publish the partial record with device-scope (write-through) stores, wait
-    // for them to be acknowledged, then take a ticket.  A device-scope release
-    // fence here instead would write back the whole L2 once per workgroup, and
-    // those write-backs serialise: they cost several times the streaming loop.
-    StatsPartial *p = partials + blockIdx.x;
-    __hip_atomic_store(&p->max_bits, __float_as_uint(mx) & 0x7f800000u, __ATOMIC_RELAXED,
-                       __HIP_MEMORY_SCOPE_AGENT);
-    __hip_atomic_store(&p->total, t, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __hip_atomic_store(&p->underflow, u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-    __builtin_amdgcn_s_waitcnt(0);
-    const unsigned arrived =
-        __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    s_last = (arrived == gridDim.x - 1);
+    if (tid == 0) {
+      // Publish the partial record with device-scope (write-through) stores, wait
+      // for them to be acknowledged, then take a ticket.  A device-scope release
+      // fence here instead would write back the whole L2 once per workgroup, and
+      // those write-backs serialise: they cost several times the streaming loop.
+      StatsPartial *p = partials + blockIdx.x;
+      __hip_atomic_store(&p->max_bits, __float_as_uint(mx) & 0x7f800000u, __ATOMIC_RELAXED,
+                         __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(&p->total, t, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(&p->underflow, u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+      __builtin_amdgcn_s_waitcnt(0);
+      const unsigned arrived =
+          __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      s_last = (arrived == gridDim.x - 1);
+    }
   }
   __syncthreads();
   if (!s_last) return;
@@ -173,13 +178,18 @@ __global__ __launch_bounds__(kBlock) void exp_stats_kernel(
     r_u[tid >> 6] = u;
   }
   __syncthreads();
+  if (tid >= 64) return;
+  mxb = tid < kWaves ? r_mx[tid] : 0u;
+  t = tid < kWaves ? r_t[tid] : 0ull;
+  u = tid < kWaves ? r_u[tid] : 0ull;
+#pragma unroll
+  for (int off = kWaves / 2; off >= 1; off >>= 1) {
+    const unsigned ob = __shfl_xor(mxb, off, 64);
+    mxb = ob > mxb ? ob : mxb;
+    t += __shfl_xor(t, off, 64);
+    u += __shfl_xor(u, off, 64);
+  }
   if (tid == 0) {
-    mxb = 0; t = 0; u = 0;
-    for (int w = 0; w < kBlock / 64; w++) {
-      mxb = r_mx[w] > mxb ? r_mx[w] : mxb;
-      t += r_t[w];
-      u += r_u[w];
-    }
     if (MODE == 0) {
       slot->max_exp_bits = mxb;
       const float max_exp = __uint_as_float(mxb);
