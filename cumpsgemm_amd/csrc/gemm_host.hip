@@ -157,22 +157,17 @@ Plan make_plan(const cuMpSGEMM_handle *h, Prec p, bool cplx, bool a_kc, bool b_k
   return plan;
 }
 
-// The persistent kernels take no edge tiles: every tile interior, every
-// K-chunk a multiple of the 32-wide step and at least four steps long, rows
-// of a K-contiguous operand 16-byte aligned, per-thread offsets within 31 bits.
+// The persistent kernels load without guards: the matrix must be at least one
+// tile wide and high (edge tiles are computed from an origin moved inwards),
+// every K-chunk a multiple of the 32-wide step and at least four steps long,
+// and every per-thread offset must fit 31 bits.
 template <class T>
 bool persistent_ok(const KernelEntry *e, bool a_kc, bool b_kc, uint64_t m, uint64_t n, uint64_t k,
-                   const Plan &plan, const T *a, uint64_t lda, uint64_t stridea, const T *b,
-                   uint64_t ldb, uint64_t strideb, uint64_t batch) {
+                   const Plan &plan, uint64_t lda, uint64_t ldb, uint64_t batch) {
   constexpr uint64_t ES = sizeof(T) / sizeof(float);
-  if (m % e->bm != 0 || n % e->bn != 0 || k % 32 != 0) return false;
+  if (m < (uint64_t)e->bm || n < (uint64_t)e->bn || k % 32 != 0) return false;
   const uint64_t last_chunk = k - (uint64_t)(plan.ksplit - 1) * plan.k_chunk;
   if (plan.k_chunk % 32 != 0 || plan.k_chunk < 128 || last_chunk < 128) return false;
-  auto vec_ok = [&](const T *p, uint64_t ld, uint64_t stride) {
-    return ((ld * ES) % 4 == 0) && ((uintptr_t)p % 16 == 0) && (batch == 1 || (stride * ES) % 4 == 0);
-  };
-  if (a_kc && !vec_ok(a, lda, stridea)) return false;
-  if (b_kc && !vec_ok(b, ldb, strideb)) return false;
   auto fits = [&](bool kc, uint64_t rows, uint64_t ld) {
     const uint64_t span = kc ? rows * ld + 32 : 32 * ld + rows;
     return span * ES * 4 < 0x7fffffffull;
@@ -305,7 +300,7 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
       args.scale_flag = h->flag_buffer + h->fused_flag;
     }
     if (launch_walk != nullptr && !no_persist &&
-        persistent_ok<T>(e, a_kc, b_kc, m, n, k, plan, a, lda, stridea, b, ldb, strideb, batch)) {
+        persistent_ok<T>(e, a_kc, b_kc, m, n, k, plan, lda, ldb, batch)) {
       const uint64_t slots = (uint64_t)h->num_cus * resident_groups(e);
       const uint64_t total = (uint64_t)plan.tiles_m * plan.tiles_n * batch;
       const dim3 grid((unsigned)std::min(total, slots), 1, plan.ksplit);

@@ -403,15 +403,19 @@ struct tile_loader {
     if constexpr (KC) {
 #pragma unroll
       for (int u = 0; u < U; u++) {
-        const float4 *p = reinterpret_cast<const float4 *>(reinterpret_cast<const char *>(base) + boff[u]);
+        // rows of a K-contiguous operand are 16-byte aligned only if ld is a
+        // multiple of 4: the vector type promises 4-byte alignment and leaves
+        // the choice of instruction to the compiler
+        typedef float f4u_t __attribute__((ext_vector_type(4), aligned(4)));
+        const f4u_t *p = reinterpret_cast<const f4u_t *>(reinterpret_cast<const char *>(base) + boff[u]);
         if constexpr (!CPLX) {
-          const float4 lo = p[0], hi = p[1];
+          const f4u_t lo = p[0], hi = p[1];
           reg.v[u][0][0] = lo.x; reg.v[u][0][1] = lo.y; reg.v[u][0][2] = lo.z; reg.v[u][0][3] = lo.w;
           reg.v[u][0][4] = hi.x; reg.v[u][0][5] = hi.y; reg.v[u][0][6] = hi.z; reg.v[u][0][7] = hi.w;
         } else {
 #pragma unroll
           for (int q = 0; q < 4; q++) {
-            const float4 t = p[q];
+            const f4u_t t = p[q];
             reg.v[u][0][2 * q] = t.x; reg.v[u][1][2 * q] = t.y;
             reg.v[u][0][2 * q + 1] = t.z; reg.v[u][1][2 * q + 1] = t.w;
           }
@@ -562,6 +566,14 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
     map_tile(blockIdx.x, args.tiles_m, args.tiles_n, tile_m, tile_n);
   }
   const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
+  // A tile that sticks out over the edge of C is computed from an origin moved
+  // back so that it ends exactly at the edge (when the matrix is at least one
+  // tile wide): every load stays in bounds and unguarded, the rows / columns it
+  // shares with its neighbour are simply not stored again.
+  const bool shift_m = args.m >= (uint32_t)BM, shift_n = args.n >= (uint32_t)BN;
+  auto load_origin_m = [&](uint32_t o) { return (shift_m && o + BM > args.m) ? args.m - BM : o; };
+  auto load_origin_n = [&](uint32_t o) { return (shift_n && o + BN > args.n) ? args.n - BN : o; };
+  const uint32_t ml0 = load_origin_m(m0), nl0 = load_origin_n(n0);
   const uint32_t kbeg = blockIdx.z * args.k_chunk;
   const uint32_t kend = (kbeg + args.k_chunk < args.k) ? kbeg + args.k_chunk : args.k;
   if (kbeg >= kend) return;
@@ -574,10 +586,10 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
              (uint64_t)tile_b * args.stride_c * ES;
 
   // operand tile origins at k = kbeg
-  const float *a_tile = Cfg::A_KC ? a + ((uint64_t)m0 * args.lda + kbeg) * ES
-                                  : a + ((uint64_t)kbeg * args.lda + m0) * ES;
-  const float *b_tile = Cfg::B_KC ? b + ((uint64_t)n0 * args.ldb + kbeg) * ES
-                                  : b + ((uint64_t)kbeg * args.ldb + n0) * ES;
+  const float *a_tile = Cfg::A_KC ? a + ((uint64_t)ml0 * args.lda + kbeg) * ES
+                                  : a + ((uint64_t)kbeg * args.lda + ml0) * ES;
+  const float *b_tile = Cfg::B_KC ? b + ((uint64_t)nl0 * args.ldb + kbeg) * ES
+                                  : b + ((uint64_t)kbeg * args.ldb + nl0) * ES;
   // (not const: a persistent kernel moves them from tile to tile)
   const uint64_t a_kstep = Cfg::A_KC ? (uint64_t)BK * ES : (uint64_t)BK * args.lda * ES;
   const uint64_t b_kstep = Cfg::B_KC ? (uint64_t)BK * ES : (uint64_t)BK * args.ldb * ES;
@@ -585,13 +597,12 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
   using LA = tile_loader<CPLX, Cfg::A_KC, BM, Cfg::UA, NT>;
   using LB = tile_loader<CPLX, Cfg::B_KC, BN, Cfg::UB, NT>;
 
-  const int rows_a = (int)((args.m - m0 < (uint32_t)BM) ? args.m - m0 : BM);
-  const int rows_b = (int)((args.n - n0 < (uint32_t)BN) ? args.n - n0 : BN);
-  // 16-byte loads along K need 16-byte aligned rows (4 floats / 2 complex)
-  const bool a_vec_ok = !Cfg::A_KC || (((args.lda * ES) & 3) == 0 && ((uintptr_t)a_tile & 15) == 0);
-  const bool b_vec_ok = !Cfg::B_KC || (((args.ldb * ES) & 3) == 0 && ((uintptr_t)b_tile & 15) == 0);
-  const bool a_full = (rows_a == BM) && a_vec_ok && LA::offsets_fit(args.lda);
-  const bool b_full = (rows_b == BN) && b_vec_ok && LB::offsets_fit(args.ldb);
+  const int rows_a = (int)((args.m - ml0 < (uint32_t)BM) ? args.m - ml0 : BM);
+  const int rows_b = (int)((args.n - nl0 < (uint32_t)BN) ? args.n - nl0 : BN);
+  // unguarded loads: the (moved) tile lies inside the matrix and every
+  // per-thread offset fits 31 bits
+  const bool a_full = (rows_a == BM) && LA::offsets_fit(args.lda);
+  const bool b_full = (rows_b == BN) && LB::offsets_fit(args.ldb);
 
   uint32_t offa[Cfg::UA], offb[Cfg::UB];
 #pragma unroll
@@ -723,7 +734,10 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
   const bool beta_zero = (args.beta_re == 0.0f) && (!CPLX || args.beta_im == 0.0f);
   const float sgn_a = args.conj_a ? -1.0f : 1.0f, sgn_b = args.conj_b ? -1.0f : 1.0f;
   const float sgn_ab = sgn_a * sgn_b;
-  auto epilogue = [&](float *cb, const uint32_t em0, const uint32_t en0, auto full_tag) {
+  // (em0, en0): origin the tile was computed from; (lo_m, lo_n): first row /
+  // column this tile owns (differs from the origin for a moved edge tile).
+  auto epilogue = [&](float *cb, const uint32_t em0, const uint32_t en0, const uint32_t lo_m,
+                      const uint32_t lo_n, auto full_tag) {
     constexpr bool FULL = decltype(full_tag)::value;
 #pragma unroll
     for (int j = 0; j < TN; j++)
@@ -733,7 +747,7 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
 #pragma unroll
         for (int v = 0; v < 16; v++) {
           const uint32_t nn = en0 + wn * Cfg::WN + j * 32 + 8 * (v / 4) + 4 * (lane >> 5) + (v & 3);
-          if (FULL || (mm < args.m && nn < args.n)) {
+          if (FULL || (mm < args.m && nn < args.n && mm >= lo_m && nn >= lo_n)) {
             float *cp = cb + ((uint64_t)nn * args.ldc + mm) * ES;
             if constexpr (!CPLX) {
               float x = acc[0][0][j][i][v];
@@ -801,17 +815,22 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
     // results are written out the next tile's first steps are already in LDS.
     // Requires >= 4 K-steps per tile (the loader's "next tile" origin is
     // refreshed when the multiplier changes tile, three steps after the loader
-    // did).  Every tile is interior and aligned (checked by the host).
+    // did).  The matrix is at least one tile wide and high and every K-chunk a
+    // multiple of the K-step (checked by the host), so no load needs a guard.
     const uint32_t total = args.tiles_m * args.tiles_n * args.batch;
     const uint32_t my_tiles = (total - blockIdx.x + gridDim.x - 1) / gridDim.x;
     const int nk = klen / BK;
+    // origin of tile i of the list: operand pointers, C, the (possibly moved)
+    // origin it is computed from and the first row / column it owns
     auto origin = [&](uint32_t i, const float *&at, const float *&bt, float *&ct, uint32_t &om0,
-                      uint32_t &on0) {
+                      uint32_t &on0, uint32_t &olo_m, uint32_t &olo_n) {
       uint32_t tm, tn, bat;
       map_tile_batched(blockIdx.x + (i < my_tiles ? i : my_tiles - 1) * gridDim.x, args.tiles_m,
                        args.tiles_n, args.batch, tm, tn, bat);
-      om0 = tm * BM;
-      on0 = tn * BN;
+      olo_m = tm * BM;
+      olo_n = tn * BN;
+      om0 = load_origin_m(olo_m);
+      on0 = load_origin_n(olo_n);
       const float *ab = reinterpret_cast<const float *>(args.a) + (uint64_t)bat * args.stride_a * ES;
       const float *bb = reinterpret_cast<const float *>(args.b) + (uint64_t)bat * args.stride_b * ES;
       ct = reinterpret_cast<float *>(args.c) + (uint64_t)bat * args.stride_c * ES;
@@ -823,8 +842,8 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
     const float *a_next, *b_next; // origin of the tile after the one being loaded
     const float *a_unused, *b_unused;
     float *c_cur = c, *c_unused;
-    uint32_t cm0 = m0, cn0 = n0, u0, u1;
-    origin(1, a_next, b_next, c_unused, u0, u1);
+    uint32_t cm0 = ml0, cn0 = nl0, clo_m = m0, clo_n = n0, u0, u1, u2, u3;
+    origin(1, a_next, b_next, c_unused, u0, u1, u2, u3);
     int lk = 0;
     auto gnext = [&]() {
       gload(0, std::true_type{});
@@ -866,12 +885,16 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
       b1 = b2;
       b2 = tmp;
       if (++ck == nk) { // tile complete: write it out, move on
-        epilogue(c_cur, cm0, cn0, std::true_type{});
+        if (cm0 == clo_m && cn0 == clo_n) {
+          epilogue(c_cur, cm0, cn0, clo_m, clo_n, std::true_type{});
+        } else {
+          epilogue(c_cur, cm0, cn0, clo_m, clo_n, std::false_type{});
+        }
         zero_acc();
         ck = 0;
         ct++;
-        origin(ct, a_unused, b_unused, c_cur, cm0, cn0);
-        origin(ct + 1, a_next, b_next, c_unused, u0, u1);
+        origin(ct, a_unused, b_unused, c_cur, cm0, cn0, clo_m, clo_n);
+        origin(ct + 1, a_next, b_next, c_unused, u0, u1, u2, u3);
       }
     }
     return;
@@ -965,7 +988,11 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
     pipeline((klen + BK - 1) / BK, std::false_type{});
   }
 
-  epilogue(c, m0, n0, std::false_type{});
+  if (ml0 == m0 && nl0 == n0 && rows_a == BM && rows_b == BN) {
+    epilogue(c, ml0, nl0, m0, n0, std::true_type{});
+  } else {
+    epilogue(c, ml0, nl0, m0, n0, std::false_type{});
+  }
 }
 
 // C (m x n, ldc, batched) *= beta before a split-K accumulation, or = 0.

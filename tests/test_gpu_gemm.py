@@ -247,3 +247,38 @@ def test_persistent_split_k(O, handle, dev, monkeypatch):
     cf = oracle_gemm(O, FP32, N, N, m, n, k, 1.0, a, m, b, k, 0.5, c0, m)
     for c in outs:  # atomic accumulation order differs from run to run
         assert O.residual(ref, c, m, n, m) <= 2.0 * O.residual(ref, cf, m, n, m)
+
+
+# ---- edge tiles computed from an origin moved inwards ------------------------------
+# A tile that sticks out over the edge of C is loaded from an origin moved back by
+# the overhang; the rows / columns it shares with its neighbour must not be updated
+# twice (beta != 0, split-K accumulation).  Forced tile classes make sure that large
+# tiles meet small overhangs.
+@pytest.mark.parametrize("cls", [0, 1, 2])
+@pytest.mark.parametrize("cplx,opa,opb,m,n,k,alpha,beta", [
+    (False, N, N, 300, 200, 160, 1.5, -0.5),     # K a multiple of 32: persistent kernels
+    (False, T, N, 257, 129, 96, 1.0, 1.0),
+    (False, N, T, 511, 383, 75, 1.0, 0.25),      # ragged K: one-tile kernels with a guarded tail
+    (False, T, T, 256, 131, 130, 2.0, 0.0),
+    (True, N, N, 200, 150, 128, 1.0 - 0.5j, 0.5 + 0.25j),
+    (True, C, T, 129, 65, 70, 1.0, 1.0),
+    (True, N, C, 70, 260, 64, 0.5j, -1.0),
+])
+def test_edge_tiles_with_beta(O, handle, dev, monkeypatch, cls, cplx, opa, opb, m, n, k, alpha, beta):
+    monkeypatch.setenv("CUMPSGEMM_FORCE_TILE_CLASS", str(cls))
+    _check(O, handle, dev, FP16TCEC, opa, opb, m, n, k, cplx, alpha, beta, pads=(1, 3, 2), seed=41)
+    _check(O, handle, dev, TF32TCEC, opa, opb, m, n, k, cplx, alpha, beta, pads=(0, 0, 0), seed=43)
+
+
+@pytest.mark.parametrize("cls", [0, 1])
+def test_edge_tiles_split_k(O, handle, dev, monkeypatch, cls):
+    monkeypatch.setenv("CUMPSGEMM_FORCE_TILE_CLASS", str(cls))
+    m, n, k = 300, 260, 8192
+    a, b = inputs.uniform(51, m * k), inputs.uniform(52, k * n)
+    c0 = inputs.uniform(53, m * n)
+    c, st, mid = run_gemm(handle, dev, FP16TCEC, N, N, m, n, k, 1.0, a, m, b, k, 0.5, c0, m, False,
+                          want_module_id=True)
+    assert st == 0 and mid == 100 + cls
+    ref = O.gemm_fp64(N, N, m, n, k, 1.0, a, m, b, k, 0.5, c0, m)
+    cf = oracle_gemm(O, FP32, N, N, m, n, k, 1.0, a, m, b, k, 0.5, c0, m)
+    assert O.residual(ref, c, m, n, m) <= 2.0 * O.residual(ref, cf, m, n, m)
