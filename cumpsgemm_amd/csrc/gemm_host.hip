@@ -101,38 +101,55 @@ unsigned resident_groups(const KernelEntry *e) {
 }
 
 // Shape -> tile class and split-K factor.  The reference fills "two waves of
-// SMs" with its first candidate or falls back to the second
-// (src/cumpsgemm.cu:252-253, x32 for batches :453-454).  Here every class gets
-// a cost from a small model fitted to measurements on MI355X, and the cheapest
-// wins:
-//   cost = rounds * (K-steps + 4) * tile area * resident groups / efficiency
+// SMs" with its first candidate or falls back to the second, and splits K for
+// small outputs (src/cumpsgemm.cu:242-253, x32 for batches :453-454).  Here
+// every (class, split) pair gets a cost from a small model fitted to
+// measurements on MI355X, and the cheapest wins:
+//   cost = rounds * (K-steps per chunk + 4) * tile area * resident groups / efficiency
+//          [+ a fixed charge when K is split]
 // rounds     = how many times the chip's CU slots must be refilled,
 // + 4        = a tile's fixed cost (pipeline fill, write-out) in K-steps,
 // efficiency = sustained MFMA rate relative to the 64x64 wave tile, which has
-//              the fewest LDS fragment reads per MFMA (64x32: 0.83, 32x32: 0.55).
-// If even the chosen class leaves CUs idle and K is long, K is split.
+//              the fewest LDS fragment reads per MFMA (64x32: 0.83, 32x32: 0.55),
+// split charge = the extra launch that prepares C (about four K-steps of the
+//              largest tile) plus the atomic write-out, which grows with the
+//              number of chunks adding into the same C.
+// K-chunks are multiples of the 32-wide step and at least four steps long.
 Plan make_plan(const cuMpSGEMM_handle *h, Prec p, bool cplx, bool a_kc, bool b_kc,
-               uint64_t m, uint64_t n, uint64_t k, uint64_t batch, int force_cls) {
+               uint64_t m, uint64_t n, uint64_t k, uint64_t batch, int force_cls, int force_split) {
   Plan plan{};
   int cls = 0;
-  if (force_cls >= 0) {
-    cls = force_cls;
-  } else {
-    double best = 0.0;
-    for (int c = 0; c < kNumTileClasses; c++) {
-      const KernelEntry *e = lookup_kernel(p, cplx, a_kc, b_kc, c);
-      const uint64_t tiles = ((m + e->bm - 1) / e->bm) * ((n + e->bn - 1) / e->bn) * batch;
-      const unsigned res = resident_groups(e);
-      const uint64_t slots = (uint64_t)h->num_cus * res;
-      const double rounds = (double)((tiles + slots - 1) / slots);
-      const int wave_area = e->wm * e->wn;
-      const double eff = wave_area >= 4096 ? 1.0 : (wave_area >= 2048 ? 0.83 : 0.55);
-      const double steps = (double)((k + 31) / 32) + 4.0;
-      const double cost = rounds * steps * (double)e->bm * e->bn * res / eff;
-      if (c == 0 || cost < best) {
+  unsigned ksplit = 1;
+  double best = -1.0;
+  const uint64_t nk = (k + 31) / 32;
+  const uint64_t max_split = std::max<uint64_t>(1, std::min<uint64_t>(k / 128, 64));
+  uint64_t forced_split = 0; // largest power of two <= min(force_split, max_split)
+  if (force_split > 0) {
+    forced_split = 1;
+    while (forced_split * 2 <= (uint64_t)force_split && forced_split * 2 <= max_split) forced_split *= 2;
+  }
+  for (int c = 0; c < kNumTileClasses; c++) {
+    if (force_cls >= 0 && c != force_cls) continue;
+    const KernelEntry *e = lookup_kernel(p, cplx, a_kc, b_kc, c);
+    const uint64_t tiles = ((m + e->bm - 1) / e->bm) * ((n + e->bn - 1) / e->bn) * batch;
+    const unsigned res = resident_groups(e);
+    const uint64_t slots = (uint64_t)h->num_cus * res;
+    const int wave_area = e->wm * e->wn;
+    const double eff = wave_area >= 4096 ? 1.0 : (wave_area >= 2048 ? 0.83 : 0.55);
+    const double unit = (double)e->bm * e->bn * res / eff;
+    const double atomics = (double)m * (double)n * (double)batch * (cplx ? 2.0 : 1.0);
+    for (uint64_t sp = 1; sp <= max_split; sp *= 2) {
+      if (forced_split != 0 && sp != forced_split) continue;
+      const double rounds = (double)((tiles * sp + slots - 1) / slots);
+      const double steps = (double)((nk + sp - 1) / sp) + 4.0;
+      double cost = rounds * steps * unit;
+      if (sp > 1) cost += 4.0 * 256.0 * 128.0 + 0.1 * atomics * (double)sp;
+      if (best < 0.0 || cost < best) {
         best = cost;
         cls = c;
+        ksplit = (unsigned)sp;
       }
+      if (forced_split == 0 && tiles * sp >= slots) break; // more chunks would only add rounds
     }
   }
   const KernelEntry *e = lookup_kernel(p, cplx, a_kc, b_kc, cls);
@@ -140,15 +157,6 @@ Plan make_plan(const cuMpSGEMM_handle *h, Prec p, bool cplx, bool a_kc, bool b_k
   plan.cls = cls;
   plan.tiles_m = (unsigned)((m + e->bm - 1) / e->bm);
   plan.tiles_n = (unsigned)((n + e->bn - 1) / e->bn);
-  const uint64_t tiles = (uint64_t)plan.tiles_m * plan.tiles_n * batch;
-  unsigned ksplit = 1;
-  if (tiles < h->num_cus && k >= 256) {
-    const uint64_t want = ((uint64_t)h->num_cus * 2 + tiles - 1) / tiles;
-    const uint64_t max_by_k = k / 128; // keep at least 4 K-steps per workgroup
-    ksplit = (unsigned)(want < max_by_k ? want : max_by_k);
-    if (ksplit < 1) ksplit = 1;
-    if (ksplit > 64) ksplit = 64;
-  }
   unsigned k_chunk = (unsigned)((k + ksplit - 1) / ksplit);
   k_chunk = (k_chunk + 31) / 32 * 32;
   ksplit = (unsigned)((k + k_chunk - 1) / k_chunk);
@@ -248,6 +256,8 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
     if (force_cls < 0 || force_cls >= kNumTileClasses) force_cls = -1;
   }
 
+  int force_split = 0; // experiments: fix the split-K factor (a power of two)
+  if (const char *f = std::getenv("CUMPSGEMM_FORCE_KSPLIT")) force_split = std::atoi(f);
   const bool no_persist = std::getenv("CUMPSGEMM_NO_PERSISTENT") != nullptr;
 
   ProfileScope prof(h, label);
@@ -263,7 +273,7 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
 
   // AUTO launches two gated kernels that must agree on how C is prepared, so
   // the split-K decision is taken once, from the first candidate.
-  Plan plan0 = make_plan(h, launches[0].p, CPLX, a_kc, b_kc, m, n, k, batch, force_cls);
+  Plan plan0 = make_plan(h, launches[0].p, CPLX, a_kc, b_kc, m, n, k, batch, force_cls, force_split);
   const bool split = plan0.ksplit > 1;
   if (split) {
     const unsigned blocks = (unsigned)std::min<uint64_t>((m * n + 255) / 256, 65535);
@@ -275,7 +285,7 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
 
   for (int i = 0; i < nlaunch; i++) {
     Plan plan = (i == 0) ? plan0
-                         : make_plan(h, launches[i].p, CPLX, a_kc, b_kc, m, n, k, batch, force_cls);
+                         : make_plan(h, launches[i].p, CPLX, a_kc, b_kc, m, n, k, batch, force_cls, force_split);
     if (split) { // same K partition for every candidate
       plan.ksplit = plan0.ksplit;
       plan.k_chunk = plan0.k_chunk;
