@@ -17,6 +17,18 @@
 #include <stdint.h>
 #include <type_traits>
 
+// Instruction mix dripped in after each MFMA of the interleaved K loop (tuning
+// knobs; the defaults are the measured optimum on MI355X).
+#ifndef CUMPSGEMM_SCHED_VALU
+#define CUMPSGEMM_SCHED_VALU 4
+#endif
+#ifndef CUMPSGEMM_SCHED_DS
+#define CUMPSGEMM_SCHED_DS 1
+#endif
+#ifndef CUMPSGEMM_SCHED_VMEM
+#define CUMPSGEMM_SCHED_VMEM 1
+#endif
+
 namespace cumpsgemm_amd {
 
 enum class Prec : int { FP16TCEC = 0, FP16TC = 1, BF16X3 = 2, BF16X2 = 3 };
@@ -875,9 +887,9 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
 #pragma unroll
       for (int g = 0; g < 2 * PT::NPROD * TM * TN * (CPLX ? 4 : 1); g++) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); // MFMA
-        __builtin_amdgcn_sched_group_barrier(0x002, 4, 0); // VALU
-        __builtin_amdgcn_sched_group_barrier(0x080, 1, 0); // DS
-        __builtin_amdgcn_sched_group_barrier(0x020, 1, 0); // VMEM read
+        __builtin_amdgcn_sched_group_barrier(0x002, CUMPSGEMM_SCHED_VALU, 0); // VALU
+        __builtin_amdgcn_sched_group_barrier(0x080, CUMPSGEMM_SCHED_DS, 0); // DS
+        __builtin_amdgcn_sched_group_barrier(0x020, CUMPSGEMM_SCHED_VMEM, 0); // VMEM read
       }
       block_sync_lds();
       const int tmp = b0;
@@ -961,9 +973,9 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
 #pragma unroll
           for (int g = 0; g < 2 * PT::NPROD * TM * TN * (CPLX ? 4 : 1); g++) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); // MFMA
-            __builtin_amdgcn_sched_group_barrier(0x002, 4, 0); // VALU
-            __builtin_amdgcn_sched_group_barrier(0x080, 1, 0); // DS
-            __builtin_amdgcn_sched_group_barrier(0x020, 1, 0); // VMEM read
+            __builtin_amdgcn_sched_group_barrier(0x002, CUMPSGEMM_SCHED_VALU, 0); // VALU
+            __builtin_amdgcn_sched_group_barrier(0x080, CUMPSGEMM_SCHED_DS, 0); // DS
+            __builtin_amdgcn_sched_group_barrier(0x020, CUMPSGEMM_SCHED_VMEM, 0); // VMEM read
           }
         }
         block_sync_lds();
