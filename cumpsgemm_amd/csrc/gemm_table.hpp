@@ -33,13 +33,16 @@ const KernelEntry *lookup_kernel(Prec p, bool cplx, bool a_kc, bool b_kc, int cl
 
 template <class Cfg>
 void launch_cfg(const GemmArgs &args, dim3 grid, hipStream_t stream) {
-  static bool attr_done = false;
-  if (!attr_done) {
-    if (Cfg::LDS_BYTES > 64 * 1024) {
+  if (Cfg::LDS_BYTES > 64 * 1024) {
+    // more than 64 KiB of dynamic LDS must be allowed once per kernel and device
+    static bool attr_done[64] = {};
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    if (dev < 0 || dev >= 64 || !attr_done[dev]) {
       (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_tcec_kernel<Cfg>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES);
+      if (dev >= 0 && dev < 64) attr_done[dev] = true;
     }
-    attr_done = true;
   }
   hipLaunchKernelGGL(gemm_tcec_kernel<Cfg>, grid, dim3(Cfg::NT), Cfg::LDS_BYTES, stream, args);
 }
