@@ -3,6 +3,7 @@
 // src/cumpsgemm.cu:19-605.
 #include "gemm_table.hpp"
 #include "handle.hpp"
+#include "pack_split.hpp"
 #include "utils.hpp"
 #include <cumpsgemm/cumpsgemm.hpp>
 #include <cumpsgemm/cumpsgemm_ext.h>
@@ -271,6 +272,72 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
     return HIPBLAS_STATUS_SUCCESS;
   }
 
+  // Pre-split path (real FP16TCEC): split A and B once, up front, into fp16
+  // planes held in the handle's workspace, and run the kernel that only copies
+  // them into LDS.  Results are bit-identical to the in-loop split (same split,
+  // same order of accumulation).  Measured on MI355X the K loop is limited by
+  // the power the MFMAs draw on real data, not by the split arithmetic, so the
+  // pre-pass (one read + write of A and B) only pays where the in-loop loads are
+  // the slow kind for both operands (A and B both M/N-contiguous, "NT": +15 % at
+  // 8192^3); everywhere else the in-loop kernels are as fast and need no
+  // workspace.  CUMPSGEMM_PACKED=1 / 0 forces / forbids the path.
+  if constexpr (!CPLX) {
+    const char *fp = std::getenv("CUMPSGEMM_PACKED"); // "0" never, "1" whenever possible
+    const bool never = fp != nullptr && fp[0] == '0', always = fp != nullptr && fp[0] == '1';
+    const bool shape_ok = batch == 1 && k >= 128 && (uint64_t)m * n >= (uint64_t)h->num_cus * kPackedBM * kPackedBN;
+    const bool pays = !a_kc && !b_kc && k >= 256 &&
+                      (double)m * (double)n / ((double)m + (double)n) >= 1800.0;
+    if (mode == CUMPSGEMM_FP16TCEC && !h->fused_scaling && !never && shape_ok && (pays || always) &&
+        force_cls <= 0 && force_split <= 1) {
+      const uint32_t mp = packed_rows(m), np = packed_rows(n);
+      const uint64_t a_bytes = packed_bytes(mp, k), b_bytes = packed_bytes(np, k);
+      if (a_bytes + b_bytes <= (16ull << 30) && mp * 64ull < 0xffffffffull && np * 64ull < 0xffffffffull) {
+        if (h->pack_ws_bytes < a_bytes + b_bytes) {
+          // the previous workspace may still be in use by work queued on the stream
+          check_hip(hipStreamSynchronize(h->stream), "sync before growing the pack workspace");
+          if (h->pack_ws != nullptr) (void)hipFree(h->pack_ws);
+          h->pack_ws = nullptr;
+          h->pack_ws_bytes = 0;
+          if (hipMalloc(&h->pack_ws, a_bytes + b_bytes) == hipSuccess) {
+            h->pack_ws_bytes = a_bytes + b_bytes;
+          } else {
+            (void)hipGetLastError();
+            h->pack_ws = nullptr;
+          }
+        }
+        if (h->pack_ws != nullptr) {
+          char *pa = static_cast<char *>(h->pack_ws), *pb = pa + a_bytes;
+          launch_pack_split(h->stream, reinterpret_cast<const float *>(a), a_kc, lda, (uint32_t)m,
+                            (uint32_t)k, pa, mp);
+          launch_pack_split(h->stream, reinterpret_cast<const float *>(b), b_kc, ldb, (uint32_t)n,
+                            (uint32_t)k, pb, np);
+          GemmArgs pargs = args;
+          pargs.a = pa;
+          pargs.b = pb;
+          pargs.lda = mp; // padded row counts of the packed operands
+          pargs.ldb = np;
+          pargs.k = (uint32_t)((k + 31) / 32 * 32); // zero-padded to whole K-steps
+          pargs.k_chunk = pargs.k;
+          pargs.tiles_m = (uint32_t)((m + kPackedBM - 1) / kPackedBM);
+          pargs.tiles_n = (uint32_t)((n + kPackedBN - 1) / kPackedBN);
+          pargs.batch = 1;
+          pargs.atomic_out = 0;
+          pargs.launch_flag = nullptr;
+          const uint64_t total = (uint64_t)pargs.tiles_m * pargs.tiles_n;
+          const dim3 grid((unsigned)std::min<uint64_t>(total, h->num_cus), 1, 1);
+          launch_packed_fp16tcec_s(pargs, grid, h->stream);
+          if (used_id != nullptr) *used_id = 200u; // pre-split path
+          const hipError_t perr = hipGetLastError();
+          if (perr != hipSuccess) {
+            log_error(std::string("packed GEMM launch failed: ") + hipGetErrorString(perr));
+            return HIPBLAS_STATUS_EXECUTION_FAILED;
+          }
+          return HIPBLAS_STATUS_SUCCESS;
+        }
+      }
+    }
+  }
+
   // AUTO launches two gated kernels that must agree on how C is prepared, so
   // the split-K decision is taken once, from the first candidate.
   Plan plan0 = make_plan(h, launches[0].p, CPLX, a_kc, b_kc, m, n, k, batch, force_cls, force_split);
@@ -433,6 +500,7 @@ hipblasStatus_t cuMpSGEMM_destroy(cuMpSGEMM_handle_t handle) {
   (void)hipFree(handle->stats_partials);
   (void)hipFree(handle->stats_ticket);
   (void)hipFree(handle->flag_buffer);
+  if (handle->pack_ws != nullptr) (void)hipFree(handle->pack_ws);
   if (handle->host_scratch) (void)hipHostFree(handle->host_scratch);
   delete handle;
   return HIPBLAS_STATUS_SUCCESS;

@@ -225,9 +225,15 @@ __device__ inline f16v_t mfma32(const u4_t a, const u4_t b, const f16v_t c) {
 //   SCALED (FP16TCEC only): op(A), op(B) are multiplied by powers of two read
 //         from device memory while they are split, and the result by the
 //         inverse product when it is written out (see GemmArgs).
+//   PACKED (persistent, real FP16TCEC): A and B were split beforehand into
+//         fp16 planes laid out as the LDS image of every (tile, K-step), see
+//         pack_split_kernel; staging is a plain 16-byte copy, no arithmetic.
 template <Prec P_, bool CPLX_, bool A_KC_, bool B_KC_, int BM_, int BN_, int WM_,
-          int WN_, int OCC_ = 1, bool DEEP_ = false, bool PERSIST_ = false, bool SCALED_ = false>
+          int WN_, int OCC_ = 1, bool DEEP_ = false, bool PERSIST_ = false, bool SCALED_ = false,
+          bool PACKED_ = false>
 struct GemmCfg {
+  static_assert(!PACKED_ || (PERSIST_ && !CPLX_ && !SCALED_ && P_ == Prec::FP16TCEC), "packed form");
+  static constexpr bool PACKED = PACKED_;
   static_assert(!PERSIST_ || DEEP_, "persistent kernels use the three-buffer pipeline");
   static_assert(!SCALED_ || P_ == Prec::FP16TCEC, "scaling guards the fp16 range only");
   using persistent_type =
@@ -459,6 +465,35 @@ struct tile_loader {
     }
   }
 
+  // Pre-split operand: the planes of one (tile, K-step) are stored as their LDS
+  // image, ROWS * 64 bytes each, `plane_bytes` apart.  Unit u of thread t is the
+  // 16-byte chunk number t + u * NT of every plane; the two chunks (hi, lo)
+  // travel in the unit's staging registers.
+  __device__ static inline void load_packed(Regs &reg, const float *__restrict__ base,
+                                            uint32_t plane_bytes) {
+    if (!active(threadIdx.x)) return;
+    const char *p = reinterpret_cast<const char *>(base);
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      const uint32_t off = (uint32_t)(threadIdx.x + u * NT) * 16u;
+      const float4 hi = *reinterpret_cast<const float4 *>(p + off);
+      const float4 lo = *reinterpret_cast<const float4 *>(p + plane_bytes + off);
+      reg.v[u][0][0] = hi.x; reg.v[u][0][1] = hi.y; reg.v[u][0][2] = hi.z; reg.v[u][0][3] = hi.w;
+      reg.v[u][0][4] = lo.x; reg.v[u][0][5] = lo.y; reg.v[u][0][6] = lo.z; reg.v[u][0][7] = lo.w;
+    }
+  }
+  __device__ static inline void store_packed(Regs &reg, char *lds_op, int tid) {
+    constexpr int PLANE = ROWS * 64;
+    if (!active(tid)) return;
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      const int off = (tid + u * NT) * 16;
+      const f8_t v = reg.v[u][0];
+      *reinterpret_cast<float4 *>(lds_op + off) = make_float4(v[0], v[1], v[2], v[3]);
+      *reinterpret_cast<float4 *>(lds_op + PLANE + off) = make_float4(v[4], v[5], v[6], v[7]);
+    }
+  }
+
   // The 8 K-values (re, im) of unit u, ready to be split.
   __device__ static inline void fetch(Regs &reg, int u, f8_t &re, f8_t &im) {
     re = reg.v[u][0];
@@ -582,7 +617,9 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
   // back so that it ends exactly at the edge (when the matrix is at least one
   // tile wide): every load stays in bounds and unguarded, the rows / columns it
   // shares with its neighbour are simply not stored again.
-  const bool shift_m = args.m >= (uint32_t)BM, shift_n = args.n >= (uint32_t)BN;
+  // (pre-split operands are padded to whole tiles instead)
+  const bool shift_m = !Cfg::PACKED && args.m >= (uint32_t)BM;
+  const bool shift_n = !Cfg::PACKED && args.n >= (uint32_t)BN;
   auto load_origin_m = [&](uint32_t o) { return (shift_m && o + BM > args.m) ? args.m - BM : o; };
   auto load_origin_n = [&](uint32_t o) { return (shift_n && o + BN > args.n) ? args.n - BN : o; };
   const uint32_t ml0 = load_origin_m(m0), nl0 = load_origin_n(n0);
@@ -603,8 +640,19 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
   const float *b_tile = Cfg::B_KC ? b + ((uint64_t)nl0 * args.ldb + kbeg) * ES
                                   : b + ((uint64_t)kbeg * args.ldb + nl0) * ES;
   // (not const: a persistent kernel moves them from tile to tile)
-  const uint64_t a_kstep = Cfg::A_KC ? (uint64_t)BK * ES : (uint64_t)BK * args.lda * ES;
-  const uint64_t b_kstep = Cfg::B_KC ? (uint64_t)BK * ES : (uint64_t)BK * args.ldb * ES;
+  // Pre-split operands: lda / ldb are the padded row counts; one K-step holds
+  // NP planes of (rows x 64 bytes), i.e. 16 floats per row and plane.
+  auto packed_origin = [&](const float *base, uint64_t rows_pad, uint32_t row0) {
+    return base + ((uint64_t)(kbeg / BK) * NP * rows_pad + row0) * 16;
+  };
+  if constexpr (Cfg::PACKED) {
+    a_tile = packed_origin(a, args.lda, ml0);
+    b_tile = packed_origin(b, args.ldb, nl0);
+  }
+  const uint64_t a_kstep = Cfg::PACKED ? (uint64_t)NP * args.lda * 16
+                           : Cfg::A_KC ? (uint64_t)BK * ES : (uint64_t)BK * args.lda * ES;
+  const uint64_t b_kstep = Cfg::PACKED ? (uint64_t)NP * args.ldb * 16
+                           : Cfg::B_KC ? (uint64_t)BK * ES : (uint64_t)BK * args.ldb * ES;
 
   using LA = tile_loader<CPLX, Cfg::A_KC, BM, Cfg::UA, NT>;
   using LB = tile_loader<CPLX, Cfg::B_KC, BN, Cfg::UB, NT>;
@@ -653,7 +701,10 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
     constexpr bool FAST = decltype(fast_tag)::value;
     const float *ap = a_tile + (uint64_t)kt * a_kstep;
     const float *bp = b_tile + (uint64_t)kt * b_kstep;
-    if constexpr (FAST) {
+    if constexpr (Cfg::PACKED) {
+      LA::load_packed(ra, ap, (uint32_t)args.lda * 64u);
+      LB::load_packed(rb, bp, (uint32_t)args.ldb * 64u);
+    } else if constexpr (FAST) {
       LA::load_fast(ra, ap, args.lda, offa);
       LB::load_fast(rb, bp, args.ldb, offb);
     } else {
@@ -665,8 +716,13 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
   auto lstore = [&](int stage) {
     char *sa = lds + stage * Cfg::STAGE_BYTES;
     char *sb = sa + Cfg::A_STAGE_BYTES;
-    LA::template store<P, Cfg::SCALED>(ra, sa, tid, coef_a, coef_a2048);
-    LB::template store<P, Cfg::SCALED>(rb, sb, tid, coef_b, coef_b2048);
+    if constexpr (Cfg::PACKED) {
+      LA::store_packed(ra, sa, tid);
+      LB::store_packed(rb, sb, tid);
+    } else {
+      LA::template store<P, Cfg::SCALED>(ra, sa, tid, coef_a, coef_a2048);
+      LB::template store<P, Cfg::SCALED>(rb, sb, tid, coef_b, coef_b2048);
+    }
   };
 
   // Per-lane fragment addresses.  Lane l of a 32x32x16 MFMA supplies row
@@ -846,10 +902,15 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
       const float *ab = reinterpret_cast<const float *>(args.a) + (uint64_t)bat * args.stride_a * ES;
       const float *bb = reinterpret_cast<const float *>(args.b) + (uint64_t)bat * args.stride_b * ES;
       ct = reinterpret_cast<float *>(args.c) + (uint64_t)bat * args.stride_c * ES;
-      at = Cfg::A_KC ? ab + ((uint64_t)om0 * args.lda + kbeg) * ES
-                     : ab + ((uint64_t)kbeg * args.lda + om0) * ES;
-      bt = Cfg::B_KC ? bb + ((uint64_t)on0 * args.ldb + kbeg) * ES
-                     : bb + ((uint64_t)kbeg * args.ldb + on0) * ES;
+      if constexpr (Cfg::PACKED) {
+        at = packed_origin(ab, args.lda, om0);
+        bt = packed_origin(bb, args.ldb, on0);
+      } else {
+        at = Cfg::A_KC ? ab + ((uint64_t)om0 * args.lda + kbeg) * ES
+                       : ab + ((uint64_t)kbeg * args.lda + om0) * ES;
+        bt = Cfg::B_KC ? bb + ((uint64_t)on0 * args.ldb + kbeg) * ES
+                       : bb + ((uint64_t)kbeg * args.ldb + on0) * ES;
+      }
     };
     const float *a_next, *b_next; // origin of the tile after the one being loaded
     const float *a_unused, *b_unused;
@@ -897,7 +958,7 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
       b1 = b2;
       b2 = tmp;
       if (++ck == nk) { // tile complete: write it out, move on
-        if (cm0 == clo_m && cn0 == clo_n) {
+        if (cm0 == clo_m && cn0 == clo_n && cm0 + BM <= args.m && cn0 + BN <= args.n) {
           epilogue(c_cur, cm0, cn0, clo_m, clo_n, std::true_type{});
         } else {
           epilogue(c_cur, cm0, cn0, clo_m, clo_n, std::false_type{});

@@ -80,6 +80,10 @@ CUMPSGEMM_DECLARE_TABLE(g_tab_bf16x2_s)
 CUMPSGEMM_DECLARE_TABLE(g_tab_bf16x2_c)
 #undef CUMPSGEMM_DECLARE_TABLE
 
+// Real FP16TCEC, 256x128 tile, persistent, operands pre-split by launch_pack_split.
+void launch_packed_fp16tcec_s(const GemmArgs &args, dim3 grid, hipStream_t stream);
+constexpr int kPackedBM = 256, kPackedBN = 128;
+
 // One table = the same three tile classes for each of the four layout pairs.
 // ROW(AKC, BKC) must expand to three make_entry<...>() initialisers.
 #define CUMPSGEMM_DEFINE_TABLE(sym, ROW)                                                       \

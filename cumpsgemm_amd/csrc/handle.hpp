@@ -74,6 +74,11 @@ struct cuMpSGEMM_handle {
   bool fused_scaling = false;
   unsigned fused_slot_a = 0, fused_slot_b = 0, fused_flag = 0;
 
+  // workspace of the pre-split (packed) GEMM path: grows on demand, freed with
+  // the handle
+  void *pack_ws = nullptr;
+  unsigned long long pack_ws_bytes = 0;
+
   // pinned host word for small read-backs
   unsigned long long *host_scratch = nullptr; // [4]
 

@@ -1,0 +1,59 @@
+// Pre-split of a whole FP32 operand into fp16 hi / lo planes for the packed
+// FP16TCEC kernels.  For large problems every element of A is otherwise split
+// once per column of tiles (and B once per row of tiles) inside the GEMM's K
+// loop; doing it once up front takes the vector arithmetic out of that loop.
+//
+// Output layout (the LDS image of every (tile, K-step), so that staging in the
+// GEMM is a linear 16-byte copy):
+//   dst[kb][plane][row][64 bytes],  kb = K-step (32 values), plane 0 = hi, 1 = lo,
+//   row < rows_pad (a multiple of 256, rows >= `rows` and K-values >= `k` are
+//   zero), and inside a row the 16-byte chunk c (8 K-values) sits at position
+//   c ^ lds_swizzle(row).
+// HBM-bound: reads 4 bytes and writes 4 bytes per element.
+#include "gemm_kernel.hpp"
+#include "pack_split.hpp"
+
+namespace cumpsgemm_amd {
+namespace {
+constexpr int kRowsPerBlock = 64;
+
+// KC: the source is K-contiguous (element (row, kk) at src[row * ld + kk]);
+// else row-contiguous (src[kk * ld + row]).
+template <bool KC>
+__global__ __launch_bounds__(256) void pack_split_kernel(const float *__restrict__ src, uint64_t ld,
+                                                         uint32_t rows, uint32_t k,
+                                                         char *__restrict__ dst, uint32_t rows_pad) {
+  const uint32_t kb = blockIdx.y;
+  const uint32_t t = threadIdx.x;
+  // lanes run along the contiguous direction of the source
+  const uint32_t row = blockIdx.x * kRowsPerBlock + (KC ? t / 4 : t % kRowsPerBlock);
+  const uint32_t chunk = KC ? t % 4 : t / kRowsPerBlock;
+  const uint32_t k0 = kb * 32 + chunk * 8;
+  f8_t x;
+#pragma unroll
+  for (int j = 0; j < 8; j++) {
+    const uint32_t kk = k0 + j;
+    float v = 0.0f;
+    if (row < rows && kk < k) v = KC ? src[(uint64_t)row * ld + kk] : src[(uint64_t)kk * ld + row];
+    x[j] = v;
+  }
+  u4_t out[2];
+  splitter<Prec::FP16TCEC>::run(x, out);
+  char *p = dst + ((uint64_t)kb * 2 * rows_pad + row) * 64 + ((chunk ^ (uint32_t)lds_swizzle((int)row)) << 4);
+  *reinterpret_cast<u4_t *>(p) = out[0];
+  *reinterpret_cast<u4_t *>(p + (uint64_t)rows_pad * 64) = out[1];
+}
+} // namespace
+
+void launch_pack_split(hipStream_t stream, const float *src, bool k_contiguous, uint64_t ld,
+                       uint32_t rows, uint32_t k, void *dst, uint32_t rows_pad) {
+  const dim3 grid(rows_pad / kRowsPerBlock, (k + 31) / 32);
+  if (k_contiguous) {
+    hipLaunchKernelGGL(pack_split_kernel<true>, grid, dim3(256), 0, stream, src, ld, rows, k,
+                       static_cast<char *>(dst), rows_pad);
+  } else {
+    hipLaunchKernelGGL(pack_split_kernel<false>, grid, dim3(256), 0, stream, src, ld, rows, k,
+                       static_cast<char *>(dst), rows_pad);
+  }
+}
+} // namespace cumpsgemm_amd

@@ -1,0 +1,12 @@
+// Pre-split of an FP32 operand into fp16 planes (see pack_split.hip).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <cstdint>
+
+namespace cumpsgemm_amd {
+// bytes of the packed form of a (rows x k) operand
+inline uint64_t packed_bytes(uint64_t rows_pad, uint64_t k) { return ((k + 31) / 32) * 2 * rows_pad * 64; }
+inline uint32_t packed_rows(uint64_t rows) { return (uint32_t)((rows + 255) / 256 * 256); }
+void launch_pack_split(hipStream_t stream, const float *src, bool k_contiguous, uint64_t ld,
+                       uint32_t rows, uint32_t k, void *dst, uint32_t rows_pad);
+} // namespace cumpsgemm_amd

@@ -282,3 +282,33 @@ def test_edge_tiles_split_k(O, handle, dev, monkeypatch, cls):
     ref = O.gemm_fp64(N, N, m, n, k, 1.0, a, m, b, k, 0.5, c0, m)
     cf = oracle_gemm(O, FP32, N, N, m, n, k, 1.0, a, m, b, k, 0.5, c0, m)
     assert O.residual(ref, c, m, n, m) <= 2.0 * O.residual(ref, cf, m, n, m)
+
+
+# ---- pre-split (packed) path ------------------------------------------------------
+# Large real FP16TCEC problems split A and B once into fp16 planes (workspace of the
+# handle) and run a kernel that only copies them into LDS.  Same split, same order of
+# accumulation: the result must equal the in-loop kernels' bit for bit.
+@pytest.mark.parametrize("opa,opb,m,n,k,pads,alpha,beta", [
+    (N, N, 4096, 4096, 256, (0, 0, 0), 1.0, 0.0),
+    (T, N, 4000, 3000, 300, (1, 3, 2), 1.5, -0.5),     # ragged M, N, K and odd leading dimensions
+    (N, T, 2304, 4100, 1000, (0, 5, 0), 1.0, 1.0),
+    (T, T, 3333, 2777, 129, (2, 0, 1), -1.0, 0.25),
+])
+def test_packed_path_matches_in_loop_split(O, handle, dev, monkeypatch, opa, opb, m, n, k, pads, alpha, beta):
+    a, lda = make_operand(inputs.uniform, 61, opa, m, k, pads[0])
+    b, ldb = make_operand(inputs.uniform, 62, opb, k, n, pads[1])
+    ldc = m + pads[2]
+    c0 = inputs.uniform(63, ldc * n)
+    outs = []
+    for packed in ("1", "0"):
+        monkeypatch.setenv("CUMPSGEMM_PACKED", packed)
+        c, st, mid = run_gemm(handle, dev, FP16TCEC, opa, opb, m, n, k, alpha, a, lda, b, ldb, beta, c0, ldc, False,
+                              want_module_id=True)
+        assert st == 0 and (mid == 200) == (packed == "1")
+        outs.append(c)
+    assert np.array_equal(outs[0].view(np.uint32), outs[1].view(np.uint32))
+    ref = O.gemm_fp64(opa, opb, m, n, k, alpha, a, lda, b, ldb, beta, c0, ldc)
+    cf = oracle_gemm(O, FP32, opa, opb, m, n, k, alpha, a, lda, b, ldb, beta, c0, ldc)
+    assert O.residual(ref, outs[0], m, n, ldc) <= 2.0 * O.residual(ref, cf, m, n, ldc)
+    if pads[2]:
+        assert np.array_equal(outs[0].reshape(n, ldc)[:, m:], c0.reshape(n, ldc)[:, m:])
