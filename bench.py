@@ -50,6 +50,9 @@ def main():
                     help="with --kernel-only: which kernel to run (copy = a plain device copy of the "
                          "same bytes, the reference point for the HBM traffic counters)")
     ap.add_argument("--op", default="NN", choices=["NN", "TN", "NT", "TT"])
+    ap.add_argument("--data", default="uniform", choices=["uniform", "zeros", "ones", "ints", "fp16"],
+                    help="with --kernel-only: operand values (the part is power-limited and the MFMAs' "
+                         "draw depends on how many operand bits toggle)")
     ap.add_argument("--mode", default="FP16TCEC", choices=["FP16TCEC", "TF32TCEC", "FP16TC", "TF32TC"])
     args = ap.parse_args()
     if args.gpus != 1:
@@ -79,6 +82,15 @@ def main():
     a = torch.from_numpy(a_host).to(dev)
     b = torch.from_numpy(b_host).to(dev)
     c = torch.zeros(m * n, device=dev)
+    if args.kernel_only and args.data != "uniform":
+        if args.data == "zeros":
+            a.zero_(), b.zero_()
+        elif args.data == "ones":
+            a.fill_(1.0), b.fill_(1.0)
+        elif args.data == "ints":
+            a, b = torch.round(a * 8), torch.round(b * 8)
+        else:  # values an fp16 holds exactly: the lo planes of the split are zero
+            a, b = a.half().float(), b.half().float()
 
     def timed(fn, steps, warmup):
         for _ in range(warmup):
@@ -108,7 +120,7 @@ def main():
         opa = cg.OP_T if args.op[0] == "T" else cg.OP_N
         opb = cg.OP_T if args.op[1] == "T" else cg.OP_N
         wall_ms, ev_ms = timed(tcec(getattr(cg, args.mode), opa, opb), args.steps, args.warmup)
-        print(json.dumps({"kernel_only": True, "op": args.op, "mode": args.mode, "size": n,
+        print(json.dumps({"kernel_only": True, "op": args.op, "mode": args.mode, "size": n, "data": args.data,
                           "ms_per_step": round(wall_ms, 4), "kernel_ms": round(ev_ms, 4),
                           "tflops": round(flops / (ev_ms * 1e-3) / 1e12, 2)}), flush=True)
         h.close()
