@@ -91,6 +91,7 @@ struct Plan {
   const KernelEntry *entry;
   int cls;
   unsigned tiles_m, tiles_n, ksplit, k_chunk;
+  double cost; // of the cost model below; comparable between shapes
 };
 
 // workgroups of this kernel that one CU holds at a time
@@ -163,6 +164,7 @@ Plan make_plan(const cuMpSGEMM_handle *h, Prec p, bool cplx, bool a_kc, bool b_k
   ksplit = (unsigned)((k + k_chunk - 1) / k_chunk);
   plan.ksplit = ksplit;
   plan.k_chunk = k_chunk;
+  plan.cost = best;
   return plan;
 }
 
@@ -201,7 +203,7 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
                          const T *b, uint64_t ldb, uint64_t strideb, const T *beta, T *c,
                          uint64_t ldc, uint64_t stridec, uint64_t batch,
                          cuMpSGEMM_compute_mode_t mode, unsigned *used_id,
-                         const char *label) {
+                         const char *label, int depth = 0) {
   constexpr bool CPLX = std::is_same<T, hipComplex>::value;
   if (h == nullptr || alpha == nullptr || beta == nullptr) return HIPBLAS_STATUS_INVALID_VALUE;
   if (m == 0 || n == 0 || batch == 0) return HIPBLAS_STATUS_SUCCESS;
@@ -261,6 +263,13 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
   if (const char *f = std::getenv("CUMPSGEMM_FORCE_KSPLIT")) force_split = std::atoi(f);
   const bool no_persist = std::getenv("CUMPSGEMM_NO_PERSISTENT") != nullptr;
 
+  // the two halves of a column split are timed as one call, by the outer level
+  struct ProfilerPause {
+    cuMpSGEMM_handle *h;
+    bool was, active;
+    ~ProfilerPause() { if (active) h->profiler.enabled = was; }
+  } pause{h, h->profiler.enabled, depth > 0};
+  if (depth > 0) h->profiler.enabled = false;
   ProfileScope prof(h, label);
   const bool beta_zero = args.beta_re == 0.0f && args.beta_im == 0.0f;
 
@@ -342,6 +351,33 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
   // the split-K decision is taken once, from the first candidate.
   Plan plan0 = make_plan(h, launches[0].p, CPLX, a_kc, b_kc, m, n, k, batch, force_cls, force_split);
   const bool split = plan0.ksplit > 1;
+
+  // A tile count just above a multiple of the chip's CU slots leaves most CUs
+  // idle for the last round.  C's columns are independent, so such a problem is
+  // cut in two: a first part whose tiles fill whole rounds, and the remaining
+  // columns, planned on their own (typically with K split to fill the chip).
+  if (!split && batch == 1 && depth == 0 && k >= 256 && std::getenv("CUMPSGEMM_NO_COLUMN_SPLIT") == nullptr) {
+    const KernelEntry *e0 = plan0.entry;
+    const uint64_t slots = (uint64_t)h->num_cus * resident_groups(e0);
+    const uint64_t tiles = (uint64_t)plan0.tiles_m * plan0.tiles_n;
+    const uint64_t full = tiles / slots;
+    const uint64_t cols1 = (full * slots) / plan0.tiles_m; // tile columns of the first part
+    if (full >= 1 && tiles % slots != 0 && cols1 >= 1 && cols1 < plan0.tiles_n) {
+      const uint64_t n1 = cols1 * (uint64_t)e0->bn, n2 = n - n1;
+      const double c1 = make_plan(h, launches[0].p, CPLX, a_kc, b_kc, m, n1, k, 1, force_cls, force_split).cost;
+      const double c2 = make_plan(h, launches[0].p, CPLX, a_kc, b_kc, m, n2, k, 1, force_cls, force_split).cost;
+      const double extra_launch = 3.0 * 256.0 * 128.0;
+      if (c1 + c2 + extra_launch < 0.93 * plan0.cost) {
+        const T *b2 = b_kc ? b + n1 * ldb : b + n1; // op(B) = N: columns of B; else rows of B^T
+        hipblasStatus_t st = run_gemm<T>(h, op_A, op_B, m, n1, k, alpha, a, lda, stridea, b, ldb, strideb,
+                                         beta, c, ldc, stridec, 1, mode, used_id, label, 1);
+        if (st != HIPBLAS_STATUS_SUCCESS) return st;
+        return run_gemm<T>(h, op_A, op_B, m, n2, k, alpha, a, lda, stridea, b2, ldb, strideb, beta,
+                           c + n1 * ldc, ldc, stridec, 1, mode, nullptr, label, 1);
+      }
+    }
+  }
+
   if (split) {
     const unsigned blocks = (unsigned)std::min<uint64_t>((m * n + 255) / 256, 65535);
     hipLaunchKernelGGL(prescale_c_kernel<CPLX>, dim3(blocks, (unsigned)batch), dim3(256), 0,

@@ -312,3 +312,37 @@ def test_packed_path_matches_in_loop_split(O, handle, dev, monkeypatch, opa, opb
     assert O.residual(ref, outs[0], m, n, ldc) <= 2.0 * O.residual(ref, cf, m, n, ldc)
     if pads[2]:
         assert np.array_equal(outs[0].reshape(n, ldc)[:, m:], c0.reshape(n, ldc)[:, m:])
+
+
+# ---- column split for a partial last round --------------------------------------
+# When the tile count is just above a multiple of the CU slots, C is cut into two
+# column blocks that are planned separately.  Same numbers as the single launch up
+# to the accumulation order of a split-K second part.
+@pytest.mark.parametrize("cplx,opa,opb,m,n,k,alpha,beta", [
+    (False, N, N, 3072, 3072, 512, 1.0, 0.0),
+    (False, T, T, 2560, 2700, 384, 1.5, -0.5),
+    (False, N, T, 3000, 3000, 300, 1.0, 1.0),
+    (True, N, N, 2048, 1300, 256, 1.0 + 0.5j, 0.5),
+    (True, C, T, 1536, 1700, 320, 1.0, 0.0),
+])
+def test_column_split_matches_single_launch(O, handle, dev, monkeypatch, cplx, opa, opb, m, n, k, alpha, beta):
+    gen = _gen(cplx)
+    a, lda = make_operand(gen, 71, opa, m, k, 1)
+    b, ldb = make_operand(gen, 72, opb, k, n, 2)
+    ldc = m + 3
+    c0 = gen(73, ldc * n)
+    outs = []
+    for single in (False, True):
+        if single:
+            monkeypatch.setenv("CUMPSGEMM_NO_COLUMN_SPLIT", "1")
+        else:
+            monkeypatch.delenv("CUMPSGEMM_NO_COLUMN_SPLIT", raising=False)
+        c, st = run_gemm(handle, dev, FP16TCEC, opa, opb, m, n, k, alpha, a, lda, b, ldb, beta, c0, ldc, cplx)
+        assert st == 0
+        outs.append(c)
+    assert rel_diff(outs[0], outs[1], m, n, ldc) < 2.0 ** -22 * np.sqrt(k)
+    ref = O.gemm_fp64(opa, opb, m, n, k, alpha, a, lda, b, ldb, beta, c0, ldc)
+    cf = oracle_gemm(O, FP32, opa, opb, m, n, k, alpha, a, lda, b, ldb, beta, c0, ldc)
+    for c in outs:
+        assert O.residual(ref, c, m, n, ldc) <= 2.0 * O.residual(ref, cf, m, n, ldc) + 2.0 ** -23
+        assert np.array_equal(c.reshape(n, ldc)[:, m:], c0.reshape(n, ldc)[:, m:])
