@@ -57,14 +57,20 @@ __global__ __launch_bounds__(kBlock) void scaling_kernel(
     const unsigned long long nvec = (count_f - head) / 4;
     const unsigned long long gsz = (unsigned long long)gridDim.x * kBlock;
     unsigned long long i = (unsigned long long)blockIdx.x * kBlock + tid;
-    for (; i + 3 * gsz < nvec; i += 4 * gsz) {
-      float4 v0 = body[i], v1 = body[i + gsz], v2 = body[i + 2 * gsz], v3 = body[i + 3 * gsz];
+    // contiguous chunks of 4 * kBlock vectors per workgroup: the grid streams
+    // one compact window at a time
+    constexpr unsigned long long kChunk = 4ull * kBlock;
+    const unsigned long long nfull = nvec / kChunk;
+    for (unsigned long long c = blockIdx.x; c < nfull; c += gridDim.x) {
+      float4 *cp = body + c * kChunk + tid;
+      float4 v0 = cp[0], v1 = cp[kBlock], v2 = cp[2 * kBlock], v3 = cp[3 * kBlock];
       v0.x *= coef; v0.y *= coef; v0.z *= coef; v0.w *= coef;
       v1.x *= coef; v1.y *= coef; v1.z *= coef; v1.w *= coef;
       v2.x *= coef; v2.y *= coef; v2.z *= coef; v2.w *= coef;
       v3.x *= coef; v3.y *= coef; v3.z *= coef; v3.w *= coef;
-      body[i] = v0; body[i + gsz] = v1; body[i + 2 * gsz] = v2; body[i + 3 * gsz] = v3;
+      cp[0] = v0; cp[kBlock] = v1; cp[2 * kBlock] = v2; cp[3 * kBlock] = v3;
     }
+    i += nfull * kChunk;
     for (; i < nvec; i += gsz) {
       float4 v = body[i];
       v.x *= coef; v.y *= coef; v.z *= coef; v.w *= coef;

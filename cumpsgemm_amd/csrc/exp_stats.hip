@@ -69,14 +69,21 @@ __global__ __launch_bounds__(kBlock) void exp_stats_kernel(
       count_one(acc, v.x, ignore_thr, under_thr); count_one(acc, v.y, ignore_thr, under_thr);
       count_one(acc, v.z, ignore_thr, under_thr); count_one(acc, v.w, ignore_thr, under_thr);
     };
-    // eight independent 16-byte loads in flight per thread
-    for (; i + 7 * gsz < nvec; i += 8 * gsz) {
+    // Eight independent 16-byte loads in flight per thread.  A workgroup takes
+    // contiguous chunks of 8 * kBlock vectors, so that what the whole grid
+    // streams at any moment is one compact window (windows a power-of-two
+    // stride apart would fall on the same memory channels).
+    constexpr unsigned long long kChunk = 8ull * kBlock;
+    const unsigned long long nfull = nvec / kChunk;
+    for (unsigned long long c = blockIdx.x; c < nfull; c += gridDim.x) {
+      const float4 *cp = body + c * kChunk + tid;
       float4 v[8];
 #pragma unroll
-      for (int j = 0; j < 8; j++) v[j] = body[i + j * gsz];
+      for (int j = 0; j < 8; j++) v[j] = cp[j * kBlock];
 #pragma unroll
       for (int j = 0; j < 8; j++) count4(v[j]);
     }
+    i += nfull * kChunk;
     for (; i < nvec; i += gsz) {
       count4(body[i]);
     }
