@@ -346,3 +346,37 @@ def test_column_split_matches_single_launch(O, handle, dev, monkeypatch, cplx, o
     for c in outs:
         assert O.residual(ref, c, m, n, ldc) <= 2.0 * O.residual(ref, cf, m, n, ldc) + 2.0 ** -23
         assert np.array_equal(c.reshape(n, ldc)[:, m:], c0.reshape(n, ldc)[:, m:])
+
+
+# ---- degenerate and skinny shapes ----------------------------------------------------
+@pytest.mark.parametrize("cplx", [False, True])
+def test_k_zero_scales_c(O, handle, dev, cplx):
+    m, n = 37, 21
+    gen = _gen(cplx)
+    c0 = gen(81, (m + 2) * n)
+    x = gen(82, 64)
+    beta = (0.5 - 0.25j) if cplx else -1.5
+    c, st = run_gemm(handle, dev, FP16TCEC, N, N, m, n, 0, 1.0, x, m, x, 1, beta, c0, m + 2, cplx)
+    assert st == 0
+    want = c0.copy().reshape(n, m + 2)
+    want[:, :m] = (want[:, :m].astype(np.complex128 if cplx else np.float64) * beta).astype(c0.dtype)
+    assert np.allclose(c.reshape(n, m + 2), want, rtol=1e-6, atol=0)
+    assert np.array_equal(c.reshape(n, m + 2)[:, m:], c0.reshape(n, m + 2)[:, m:])
+
+
+@pytest.mark.parametrize("mode", [FP16TCEC, TF32TCEC])
+@pytest.mark.parametrize("opa,opb,m,n,k", [
+    (N, N, 1, 4096, 4096),      # row vector times matrix
+    (T, N, 4096, 1, 300),       # matrix times column vector
+    (N, T, 5, 7, 10000),        # tiny output, long K: split-K with guarded loads
+    (T, T, 3, 1, 1),
+    (N, N, 2000, 3, 64),
+    (N, N, 31, 33, 17),
+])
+def test_skinny_shapes(O, handle, dev, mode, opa, opb, m, n, k):
+    _check(O, handle, dev, mode, opa, opb, m, n, k, False, 1.25, 0.5, pads=(1, 2, 3), seed=91)
+
+
+def test_skinny_complex(O, handle, dev):
+    _check(O, handle, dev, FP16TCEC, C, N, 1, 513, 700, True, 1.0 - 1.0j, 0.5j, pads=(0, 1, 2), seed=93)
+    _check(O, handle, dev, TF32TCEC, N, C, 257, 2, 90, True, 1.0, 0.0, pads=(3, 0, 0), seed=95)
