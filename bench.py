@@ -7,7 +7,7 @@ FP32 SGEMM on the same GPU and to the split-and-correct algorithm on host cores.
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--full]
 
 One "step" is one GEMM call through the C ABI (cuMpSGEMM_sgemm) with operands
-resident in HBM.  Prints ONE JSON line.  --full adds the other BASELINE
+resident in HBM.  Prints ONE JSON line.  --full adds the other benchmark
 configurations (layouts, bf16x3, batched CGEMM, scaling pipeline, tall-skinny,
 Mx2x2) under "extra".
 """
@@ -288,7 +288,7 @@ def hbm_kernel_only(args, torch, cg, inputs, h, dev, stream):
 
 
 def full_suite(torch, cg, inputs, h, dev, stream, timed, log):
-    """The other BASELINE configurations, reported under "extra"."""
+    """The other benchmark configurations (C2 layouts, C3, C4, C5a, C5b), reported under "extra"."""
     res = {}
 
     def rel_err(got, ref):

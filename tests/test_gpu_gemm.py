@@ -159,7 +159,7 @@ def test_strided_batch(O, handle, dev, cplx):
 
 
 def test_c1_config_1024_cubed(O, handle, dev):
-    """BASELINE config 1: SGEMM NN 1024^3, uniform[-1,1], seeds (1,2)."""
+    """Benchmark configuration C1: SGEMM NN 1024^3, uniform[-1,1], seeds (1,2)."""
     m = n = k = 1024
     a, b = inputs.uniform(1, m * k), inputs.uniform(2, k * n)
     for mode in (FP16TCEC, TF32TCEC):

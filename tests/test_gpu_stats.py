@@ -92,7 +92,7 @@ def test_three_way_decision(O, handle, dev):
 
 
 def test_c4_config_stats_bit_exact(O, handle, dev):
-    """BASELINE config 4 inputs (4096^2, per-row / per-column exponents in [-30, 30])."""
+    """Benchmark configuration C4 inputs (4096^2, per-row / per-column exponents in [-30, 30])."""
     a = inputs.exponent_spread(3, 4096, 4096, per_row=True)
     b = inputs.exponent_spread(4, 4096, 4096, per_row=False)
     _cmp_stats(O, handle, dev, a, 4096, 4096, 4096)
