@@ -380,3 +380,25 @@ def test_skinny_shapes(O, handle, dev, mode, opa, opb, m, n, k):
 def test_skinny_complex(O, handle, dev):
     _check(O, handle, dev, FP16TCEC, C, N, 1, 513, 700, True, 1.0 - 1.0j, 0.5j, pads=(0, 1, 2), seed=93)
     _check(O, handle, dev, TF32TCEC, N, C, 257, 2, 90, True, 1.0, 0.0, pads=(3, 0, 0), seed=95)
+
+
+def test_huge_leading_dimension_uses_64_bit_addressing(O, handle, dev, torch_gpu):
+    """lda = 2^29: the per-thread byte offsets of a tile no longer fit 31 bits and
+    the kernels must fall back to 64-bit element addressing."""
+    torch = torch_gpu
+    m, n, k, lda = 64, 48, 2, 1 << 29
+    a_small = inputs.uniform(97, m * k).reshape(k, m)           # column-major: column j at a[j]
+    b = inputs.uniform(98, k * n)
+    da = torch.zeros((k - 1) * lda + m, device=dev.dev)         # 2 GiB of floats
+    for j in range(k):
+        da[j * lda: j * lda + m] = torch.from_numpy(a_small[j]).to(dev.dev)
+    db, dc = dev.up(b), dev.up(np.zeros(m * n, np.float32))
+    for opa, ld_used in ((N, lda),):
+        st = handle.gemm(opa, N, m, n, k, 1.0, da, ld_used, db, k, 0.0, dc, m, FP16TCEC)
+        assert st == 0
+        c = dev.down(dc)
+        ref = O.gemm_fp64(N, N, m, n, k, 1.0, a_small.reshape(-1), m, b, k)
+        cf = oracle_gemm(O, FP32, N, N, m, n, k, 1.0, a_small.reshape(-1), m, b, k, 0.0, np.zeros(m * n, np.float32), m)
+        assert O.residual(ref, c, m, n, m) <= 2.0 * O.residual(ref, cf, m, n, m) + 2.0 ** -23
+    del da
+    torch.cuda.empty_cache()
