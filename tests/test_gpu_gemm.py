@@ -402,3 +402,26 @@ def test_huge_leading_dimension_uses_64_bit_addressing(O, handle, dev, torch_gpu
         assert O.residual(ref, c, m, n, m) <= 2.0 * O.residual(ref, cf, m, n, m) + 2.0 ** -23
     del da
     torch.cuda.empty_cache()
+
+
+def test_seeded_random_shapes_all_paths(O, handle, dev):
+    """Forty seeded random problems (shape, layout, mode, type, scalars, padding):
+    whatever kernel form the planner picks -- one-tile or persistent, split-K,
+    column split, moved edge tiles -- the result must meet the accuracy bars."""
+    rng = np.random.default_rng(20240611)
+    dims = [1, 2, 31, 32, 33, 64, 100, 127, 128, 129, 200, 255, 256, 257, 300, 384, 512, 640, 700, 1000]
+    for case in range(40):
+        m, n, k = (int(rng.choice(dims)) for _ in range(3))
+        if case % 8 == 0:
+            k = int(rng.choice([2048, 4096, 6000]))      # long K: split-K candidates
+        if case % 10 == 5:
+            m, n = 2560, int(rng.choice([1300, 2700]))     # column split candidates
+            k = int(rng.choice([256, 288]))
+        cplx = bool(rng.integers(0, 2))
+        ops = [N, T, C] if cplx else [N, T]
+        opa, opb = int(rng.choice(ops)), int(rng.choice(ops))
+        mode = int(rng.choice([FP16TCEC, TF32TCEC, FP16TCEC, FP16TC, TF32TC]))
+        alpha = complex(rng.normal(), rng.normal()) if cplx else float(rng.normal())
+        beta = 0.0 if rng.integers(0, 3) == 0 else (complex(rng.normal(), rng.normal()) if cplx else float(rng.normal()))
+        pads = tuple(int(x) for x in rng.integers(0, 4, 3))
+        _check(O, handle, dev, mode, opa, opb, m, n, k, cplx, alpha, beta, pads=pads, seed=1000 + case)
