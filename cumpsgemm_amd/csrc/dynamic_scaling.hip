@@ -250,7 +250,13 @@ unsigned cuMpSGEMM_get_current_dynamic_launch_buffer_id(cuMpSGEMM_handle_t h) {
 unsigned cuMpSGEMM_get_next_dynamic_launch_buffer_id(cuMpSGEMM_handle_t h) {
   return cumpsgemm::get_next_dynamic_launch_buffer_id(h);
 }
-int cuMpSGEMM_get_dynamic_launch_flag(cuMpSGEMM_handle_t h, unsigned id) { return read_flag(h, id); }
+int cuMpSGEMM_get_dynamic_launch_flag(cuMpSGEMM_handle_t h, unsigned id) {
+  try { // no exception may cross the C boundary
+    return read_flag(h, id);
+  } catch (const std::exception &) {
+    return 0;
+  }
+}
 void cuMpSGEMM_set_dynamic_launch_buffer_by_exp_stats(cuMpSGEMM_handle_t h, unsigned flag_id,
                                                       unsigned a_id, unsigned b_id) {
   cumpsgemm::set_dynamic_launch_buffer_by_exp_stats(h, flag_id, a_id, b_id);

@@ -418,17 +418,33 @@ unsigned cuMpSGEMM_exp_max_ext_c(cuMpSGEMM_handle_t h, unsigned m, unsigned n,
                                  unsigned stride) {
   return cumpsgemm::exp_max_ext<hipComplex>(h, m, n, ptr, ld, batch, stride);
 }
+// The read-backs synchronise the stream and the C++ forms throw when HIP
+// reports an error; no exception may cross the C boundary, so the C forms log
+// (check_hip already has) and return zeros / UNDEFINED instead.
 void cuMpSGEMM_get_exp_stats(cuMpSGEMM_handle_t h, unsigned id, uint64_t *underflow,
                              uint64_t *total) {
-  const auto r = cumpsgemm::get_exp_stats(h, id);
-  *underflow = r.first;
-  *total = r.second;
+  *underflow = 0;
+  *total = 0;
+  try {
+    const auto r = cumpsgemm::get_exp_stats(h, id);
+    *underflow = r.first;
+    *total = r.second;
+  } catch (const std::exception &) {
+  }
 }
 float cuMpSGEMM_get_max_exp(cuMpSGEMM_handle_t h, unsigned id) {
-  return cumpsgemm::get_max_exp(h, id);
+  try {
+    return cumpsgemm::get_max_exp(h, id);
+  } catch (const std::exception &) {
+    return 0.0f;
+  }
 }
 int cuMpSGEMM_get_exp_stats_compute_mode_level(cuMpSGEMM_handle_t h, unsigned id) {
-  return (int)cumpsgemm::get_exp_stats_compute_mode_level(h, id);
+  try {
+    return (int)cumpsgemm::get_exp_stats_compute_mode_level(h, id);
+  } catch (const std::exception &) {
+    return (int)CUMPSGEMM_UNDEFINED;
+  }
 }
 void cuMpSGEMM_set_exp_stats_params(cuMpSGEMM_handle_t h, float ignore_threshold,
                                     float underflow_threshold, float tolerance) {

@@ -303,7 +303,10 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
       if (a_bytes + b_bytes <= (16ull << 30) && mp * 64ull < 0xffffffffull && np * 64ull < 0xffffffffull) {
         if (h->pack_ws_bytes < a_bytes + b_bytes) {
           // the previous workspace may still be in use by work queued on the stream
-          check_hip(hipStreamSynchronize(h->stream), "sync before growing the pack workspace");
+          if (hipStreamSynchronize(h->stream) != hipSuccess) {
+            log_error("stream synchronisation failed before growing the pack workspace");
+            return HIPBLAS_STATUS_EXECUTION_FAILED;
+          }
           if (h->pack_ws != nullptr) (void)hipFree(h->pack_ws);
           h->pack_ws = nullptr;
           h->pack_ws_bytes = 0;
