@@ -9,8 +9,9 @@ This tool reads such a log (the cuBLAS names of logs written by the reference
 are accepted too), runs every recorded shape through the library with the
 recorded mode on random inputs, checks the result against an FP64 GEMM with the
 reference's threshold (2^-23 * sqrt(K) for the error-corrected modes, 2^-10 *
-sqrt(K) for the others) and reports throughput -- the counterpart of the
-reference harness's "log" command (test/main.cu:820-1016).
+sqrt(K) for the others) and prints one line per shape in the reference
+harness's CSV format -- the counterpart of its "log" command
+(test/main.cu:820-1016, line format :404-410).
 
     python -m cumpsgemm_amd.replay_log app.log
 """
@@ -76,6 +77,10 @@ def replay(calls, max_elements=1 << 28, out=sys.stdout):
                                         br * bc, 0.0, fc, m, m * n, batch, modes[c["mode"]], cplx=cplx)
         assert run() == 0
         torch.cuda.synchronize()
+        module = 0
+        if c["mode"] not in ("AUTO", "FP16TCEC_SCALING") and batch == 1:
+            _, module = h.gemm(ops[c["op_a"]], ops[c["op_b"]], m, n, k, 1.0, fa, ar, fb, br, 0.0, fc, m,
+                               modes[c["mode"]], cplx=cplx, want_module_id=True)
 
         def logical(t, op):
             x = t.transpose(1, 2).to(torch.complex128 if cplx else torch.float64)
@@ -100,8 +105,12 @@ def replay(calls, max_elements=1 << 28, out=sys.stdout):
         ok = res < bar
         tested += 1
         passed += ok
-        print(f"{c['func']},{c['op_a']},{c['op_b']},{m},{n},{k},{batch},{c['mode']},"
-              f"residual={res:.3e},throughput={tflops:.2f}TFlop/s,{'OK' if ok else 'NG'}", file=out)
+        # the result line of the reference harness (test/main.cu:404-410, batched :522-529):
+        # gemm,MODE,opA,opB,m,n,k[,batch],TFlop/s,residual,OK|NG,module id
+        kind = "cgemm" if cplx else "sgemm"
+        shape = f"{m},{n},{k}" + (f",{batch}" if batch > 1 else "")
+        print(f"{kind},{c['mode']},{c['op_a']},{c['op_b']},{shape},{tflops:e},{res:e},{'OK' if ok else 'NG'},{module}",
+              file=out)
     h.close()
     print(f"{passed} / {tested} passed", file=out)
     return passed, tested

@@ -39,4 +39,6 @@ def test_replay(tmp_path, cg, torch_gpu):
     text = out.getvalue()
     # duplicates collapse, forwarded (CUBLAS_*) calls are not ours to replay
     assert (passed, tested) == (4, 4), text
-    assert "hipblasSgemm,N,N,1280,1280,1280,1,FP16TCEC,residual=" in text and "4 / 4 passed" in text
+    import re
+    assert re.search(r"^sgemm,FP16TCEC,N,N,1280,1280,1280,\d\.\d+e[+-]\d+,\d\.\d+e-\d+,OK,\d+$", text, re.M), text
+    assert re.search(r"^sgemm,FP16TC,T,N,300,200,96,3,", text, re.M) and "4 / 4 passed" in text
