@@ -111,6 +111,14 @@ def _declare(L):
     L.cuMpSGEMM_reset_exp_stats_buffer_id.restype = None
     L.cuMpSGEMM_enable_exp_stats.argtypes = [_ptr]
     L.cuMpSGEMM_disable_exp_stats.argtypes = [_ptr]
+    for name in ("enable", "disable", "reset"):
+        fn = getattr(L, f"cuMpSGEMM_{name}_exp_stats_profiling")
+        fn.argtypes = [_ptr]
+        fn.restype = None
+    L.cuMpSGEMM_print_exp_stats_profiling.argtypes = [_ptr, _u32]
+    L.cuMpSGEMM_print_exp_stats_profiling.restype = None
+    L.cuMpSGEMM_get_exp_stats_profiling_entry.argtypes = [_ptr, ctypes.c_char_p, ctypes.POINTER(ctypes.c_double),
+                                                          ctypes.POINTER(_u64)]
     scale_args = [_ptr, _u32, _u32, _u32, _u32, _ptr, _u32, _u32, _u32]
     for base in ("scale_A", "scale_B", "reset_scale_A", "reset_scale_B"):
         for sfx in ("s", "c"):
@@ -259,6 +267,27 @@ class Handle:
 
     def reset_exp_stats_buffer_id(self):
         self._L.cuMpSGEMM_reset_exp_stats_buffer_id(self._h)
+
+    # ---- wall-clock profiling of stats / scaling / GEMM launches ----
+    def enable_exp_stats_profiling(self):
+        self._L.cuMpSGEMM_enable_exp_stats_profiling(self._h)
+
+    def disable_exp_stats_profiling(self):
+        self._L.cuMpSGEMM_disable_exp_stats_profiling(self._h)
+
+    def reset_exp_stats_profiling(self):
+        self._L.cuMpSGEMM_reset_exp_stats_profiling(self._h)
+
+    def print_exp_stats_profiling(self, csv=False):
+        self._L.cuMpSGEMM_print_exp_stats_profiling(self._h, int(csv))
+
+    def get_exp_stats_profiling_entry(self, name):
+        """(seconds, count) recorded under a label, or None if the label never ran."""
+        t, n = ctypes.c_double(0), _u64(0)
+        if not self._L.cuMpSGEMM_get_exp_stats_profiling_entry(self._h, name.encode(), ctypes.byref(t),
+                                                               ctypes.byref(n)):
+            return None
+        return t.value, n.value
 
     # ---- scaling ----
     def _scale(self, base, cplx, *args):

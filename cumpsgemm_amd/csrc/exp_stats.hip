@@ -458,4 +458,25 @@ void cuMpSGEMM_reset_exp_stats_buffer_id(cuMpSGEMM_handle_t h) {
 }
 void cuMpSGEMM_enable_exp_stats(cuMpSGEMM_handle_t h) { cumpsgemm::enable_exp_stats(h); }
 void cuMpSGEMM_disable_exp_stats(cuMpSGEMM_handle_t h) { cumpsgemm::disable_exp_stats(h); }
+void cuMpSGEMM_enable_exp_stats_profiling(cuMpSGEMM_handle_t h) {
+  cumpsgemm::enable_exp_stats_profiling(h);
+}
+void cuMpSGEMM_disable_exp_stats_profiling(cuMpSGEMM_handle_t h) {
+  cumpsgemm::disable_exp_stats_profiling(h);
+}
+void cuMpSGEMM_reset_exp_stats_profiling(cuMpSGEMM_handle_t h) {
+  cumpsgemm::reset_exp_stats_profiling(h);
+}
+void cuMpSGEMM_print_exp_stats_profiling(cuMpSGEMM_handle_t h, unsigned csv) {
+  cumpsgemm::print_exp_stats_profiling(h, csv);
+}
+int cuMpSGEMM_get_exp_stats_profiling_entry(cuMpSGEMM_handle_t h, const char *name,
+                                            double *time_sum, uint64_t *n) {
+  if (!h || !name) return 0;
+  const auto it = h->profiler.entries.find(name);
+  if (it == h->profiler.entries.end()) return 0;
+  if (time_sum) *time_sum = it->second.sum;
+  if (n) *n = it->second.n;
+  return 1;
+}
 } // extern "C"

@@ -113,6 +113,17 @@ unsigned cuMpSGEMM_get_current_exp_stats_buffer_id(cuMpSGEMM_handle_t h);
 void cuMpSGEMM_reset_exp_stats_buffer_id(cuMpSGEMM_handle_t h);
 void cuMpSGEMM_enable_exp_stats(cuMpSGEMM_handle_t h);
 void cuMpSGEMM_disable_exp_stats(cuMpSGEMM_handle_t h);
+/* wall-clock profiling of the stats / scaling / GEMM launches (cumpsgemm.hpp:116-129).
+ * get_..._entry is debug::get_exp_stats_profiling_result for one label
+ * ("exp_stats_1", "exp_stats_2", "exp_max", "scaling_AB", "scaling_C",
+ * "reset_scaling_AB", a GEMM label): returns 1 and fills seconds / count when
+ * the label has been recorded, else 0. */
+void cuMpSGEMM_enable_exp_stats_profiling(cuMpSGEMM_handle_t h);
+void cuMpSGEMM_disable_exp_stats_profiling(cuMpSGEMM_handle_t h);
+void cuMpSGEMM_reset_exp_stats_profiling(cuMpSGEMM_handle_t h);
+void cuMpSGEMM_print_exp_stats_profiling(cuMpSGEMM_handle_t h, unsigned csv);
+int cuMpSGEMM_get_exp_stats_profiling_entry(cuMpSGEMM_handle_t h, const char *name,
+                                            double *time_sum, uint64_t *n);
 
 /* cumpsgemm::scale_A/B/C, reset_scale_A/B (cumpsgemm.hpp:71-100) */
 void cuMpSGEMM_scale_A_s(cuMpSGEMM_handle_t h, unsigned stats_id, unsigned flag_id, unsigned m,
