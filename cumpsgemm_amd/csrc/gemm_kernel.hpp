@@ -593,6 +593,16 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
       coef_c *= mb / 16384.0f;
     }
   }
+  if constexpr (Cfg::SCALED) {
+    // loaded through vector memory, so the compiler cannot see that they are
+    // uniform: say so, or each costs every lane a register for the whole kernel
+    auto uniform = [](float x) {
+      return __uint_as_float(__builtin_amdgcn_readfirstlane(__float_as_uint(x)));
+    };
+    coef_a = uniform(coef_a);
+    coef_b = uniform(coef_b);
+    coef_c = uniform(coef_c);
+  }
   const float coef_a2048 = coef_a * 2048.0f, coef_b2048 = coef_b * 2048.0f;
   // alpha with the inverse scaling of C folded in (exact: a power of two)
   const float alpha_re = args.alpha_re * coef_c, alpha_im = args.alpha_im * coef_c;
