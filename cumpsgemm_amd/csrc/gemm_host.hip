@@ -172,13 +172,26 @@ Plan make_plan(const cuMpSGEMM_handle *h, Prec p, bool cplx, bool a_kc, bool b_k
 // tile wide and high (edge tiles are computed from an origin moved inwards),
 // every K-chunk a multiple of the 32-wide step and at least four steps long,
 // and every per-thread offset must fit 31 bits.
+constexpr unsigned kPersistentMaxSteps = 32; // K-steps per tile up to which tiles are walked
+
 template <class T>
 bool persistent_ok(const KernelEntry *e, bool a_kc, bool b_kc, uint64_t m, uint64_t n, uint64_t k,
-                   const Plan &plan, uint64_t lda, uint64_t ldb, uint64_t batch) {
+                   const Plan &plan, uint64_t lda, uint64_t ldb, uint64_t batch, bool any_length) {
   constexpr uint64_t ES = sizeof(T) / sizeof(float);
   if (m < (uint64_t)e->bm || n < (uint64_t)e->bn || k % 32 != 0) return false;
   const uint64_t last_chunk = k - (uint64_t)(plan.ksplit - 1) * plan.k_chunk;
   if (plan.k_chunk % 32 != 0 || plan.k_chunk < 128 || last_chunk < 128) return false;
+  // Walking tiles pays while a tile is short: the next tile's first steps load
+  // during the write-out.  Long tiles gain nothing from that and run 1 - 4 %
+  // faster as independent workgroups, which drift apart in time instead of
+  // asking memory for the same K range in lockstep.  (The kernels with fused
+  // scaling are the exception: their one-tile form measures 7 % slower for the
+  // NN layout, so they walk tiles of any length.)
+  static const unsigned max_steps = [] {
+    const char *e = std::getenv("CUMPSGEMM_PERSISTENT_MAX_STEPS");
+    return e != nullptr ? (unsigned)std::atoi(e) : kPersistentMaxSteps;
+  }();
+  if (!any_length && plan.k_chunk / 32 > max_steps) return false;
   auto fits = [&](bool kc, uint64_t rows, uint64_t ld) {
     const uint64_t span = kc ? rows * ld + 32 : 32 * ld + rows;
     return span * ES * 4 < 0x7fffffffull;
@@ -416,7 +429,8 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
       args.scale_flag = h->flag_buffer + h->fused_flag;
     }
     if (launch_walk != nullptr && !no_persist &&
-        persistent_ok<T>(e, a_kc, b_kc, m, n, k, plan, lda, ldb, batch)) {
+        persistent_ok<T>(e, a_kc, b_kc, m, n, k, plan, lda, ldb, batch,
+                         launch_walk == e->launch_scaled_persistent)) {
       const uint64_t slots = (uint64_t)h->num_cus * resident_groups(e);
       const uint64_t total = (uint64_t)plan.tiles_m * plan.tiles_n * batch;
       const dim3 grid((unsigned)std::min(total, slots), 1, plan.ksplit);
