@@ -92,6 +92,8 @@ def _declare(L):
                      ("cuMpSGEMM_sgemm_2xNx2", f32p), ("cuMpSGEMM_cgemm_2xNx2", c2p)):
         getattr(L, name).argtypes = [_ptr, _int, _int, _u64, sp, _ptr, _u64, _u64, _ptr, _u64, _u64,
                                      sp, _ptr, _u64, _u64, _u64]
+    L.cuMpSGEMM_get_workspace_size.argtypes = [_ptr]
+    L.cuMpSGEMM_get_workspace_size.restype = ctypes.c_size_t
     L.cuMpSGEMM_describe_tile_config.argtypes = [_int, _int, _int, _int, _int, ctypes.c_char_p, ctypes.c_size_t]
     stats_args = [_ptr, _u32, _u32, _ptr, _u32, _u32, _u32]
     for name in ("cuMpSGEMM_exp_stats_ext_s", "cuMpSGEMM_exp_stats_ext_c",
@@ -201,6 +203,10 @@ class Handle:
     def set_stream(self, stream):
         s = getattr(stream, "cuda_stream", stream)
         return self._L.cuMpSGEMM_set_stream(self._h, _ptr(int(s) if s else 0))
+
+    def workspace_size(self):
+        """Bytes of device memory held for pre-split operands."""
+        return self._L.cuMpSGEMM_get_workspace_size(self._h)
 
     # ---- GEMM ----
     def gemm(self, op_a, op_b, m, n, k, alpha, a, lda, b, ldb, beta, c, ldc, mode, cplx=False,

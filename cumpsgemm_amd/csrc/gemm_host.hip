@@ -309,7 +309,12 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
     const bool shape_ok = batch == 1 && k >= 128 && (uint64_t)m * n >= (uint64_t)h->num_cus * kPackedBM * kPackedBN;
     const bool pays = !a_kc && !b_kc && k >= 256 &&
                       (double)m * (double)n / ((double)m + (double)n) >= 1800.0;
-    if (mode == CUMPSGEMM_FP16TCEC && !h->fused_scaling && !never && shape_ok && (pays || always) &&
+    // With fused scaling the in-loop split costs one more instruction per pair
+    // and those kernels run 8 - 25 % below the plain ones, so the pre-pass (which
+    // scales as it splits) pays for every layout.
+    const bool pays_scaled = h->fused_scaling && k >= 256 &&
+                             (double)m * (double)n / ((double)m + (double)n) >= 1800.0;
+    if (mode == CUMPSGEMM_FP16TCEC && !never && shape_ok && (pays || pays_scaled || always) &&
         force_cls <= 0 && force_split <= 1) {
       const uint32_t mp = packed_rows(m), np = packed_rows(n);
       const uint64_t a_bytes = packed_bytes(mp, k), b_bytes = packed_bytes(np, k);
@@ -332,11 +337,21 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
         }
         if (h->pack_ws != nullptr) {
           char *pa = static_cast<char *>(h->pack_ws), *pb = pa + a_bytes;
-          launch_pack_split(h->stream, reinterpret_cast<const float *>(a), a_kc, lda, (uint32_t)m,
-                            (uint32_t)k, pa, mp);
-          launch_pack_split(h->stream, reinterpret_cast<const float *>(b), b_kc, ldb, (uint32_t)n,
-                            (uint32_t)k, pb, np);
           GemmArgs pargs = args;
+          const uint32_t *max_a = nullptr, *max_b = nullptr;
+          const int *sflag = nullptr;
+          if (h->fused_scaling) {
+            max_a = &h->stats_slots[h->fused_slot_a].max_exp_bits;
+            max_b = &h->stats_slots[h->fused_slot_b].max_exp_bits;
+            sflag = h->flag_buffer + h->fused_flag;
+            pargs.scale_max_a = max_a; // the kernel derives the inverse scaling of C from them
+            pargs.scale_max_b = max_b;
+            pargs.scale_flag = sflag;
+          }
+          launch_pack_split(h->stream, reinterpret_cast<const float *>(a), a_kc, lda, (uint32_t)m,
+                            (uint32_t)k, pa, mp, max_a, sflag, 0x40);
+          launch_pack_split(h->stream, reinterpret_cast<const float *>(b), b_kc, ldb, (uint32_t)n,
+                            (uint32_t)k, pb, np, max_b, sflag, 0x20);
           pargs.a = pa;
           pargs.b = pb;
           pargs.lda = mp; // padded row counts of the packed operands
@@ -350,7 +365,11 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
           pargs.launch_flag = nullptr;
           const uint64_t total = (uint64_t)pargs.tiles_m * pargs.tiles_n;
           const dim3 grid((unsigned)std::min<uint64_t>(total, h->num_cus), 1, 1);
-          launch_packed_fp16tcec_s(pargs, grid, h->stream);
+          if (h->fused_scaling) {
+            launch_packed_scaled_fp16tcec_s(pargs, grid, h->stream);
+          } else {
+            launch_packed_fp16tcec_s(pargs, grid, h->stream);
+          }
           if (used_id != nullptr) *used_id = 200u; // pre-split path
           const hipError_t perr = hipGetLastError();
           if (perr != hipSuccess) {
@@ -635,6 +654,10 @@ hipblasStatus_t cuMpSGEMM_cgemm_ex(cuMpSGEMM_handle_t handle, hipblasOperation_t
                                    unsigned *used_kernel_module_id) {
   return cumpsgemm::gemm<hipComplex>(handle, op_A, op_B, m, n, k, alpha, a, lda, b, ldb, beta, c,
                                      ldc, mode, used_kernel_module_id);
+}
+
+size_t cuMpSGEMM_get_workspace_size(cuMpSGEMM_handle_t handle) {
+  return handle != nullptr ? (size_t)handle->pack_ws_bytes : 0;
 }
 
 int cuMpSGEMM_describe_tile_config(int compute_mode, int is_complex, int op_A, int op_B,

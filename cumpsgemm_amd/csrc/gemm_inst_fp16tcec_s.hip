@@ -12,5 +12,9 @@ void launch_packed_fp16tcec_s(const GemmArgs &args, dim3 grid, hipStream_t strea
   launch_cfg<GemmCfg<Prec::FP16TCEC, false, true, true, 256, 128, 64, 64, 2, true, true, false, true>>(
       args, grid, stream);
 }
+void launch_packed_scaled_fp16tcec_s(const GemmArgs &args, dim3 grid, hipStream_t stream) {
+  launch_cfg<GemmCfg<Prec::FP16TCEC, false, true, true, 256, 128, 64, 64, 2, true, true, true, true>>(
+      args, grid, stream);
+}
 #undef ROW
 } // namespace cumpsgemm_amd

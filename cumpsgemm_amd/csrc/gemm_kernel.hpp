@@ -232,7 +232,9 @@ template <Prec P_, bool CPLX_, bool A_KC_, bool B_KC_, int BM_, int BN_, int WM_
           int WN_, int OCC_ = 1, bool DEEP_ = false, bool PERSIST_ = false, bool SCALED_ = false,
           bool PACKED_ = false>
 struct GemmCfg {
-  static_assert(!PACKED_ || (PERSIST_ && !CPLX_ && !SCALED_ && P_ == Prec::FP16TCEC), "packed form");
+  // (PACKED + SCALED: the operands were scaled when they were pre-split; the
+  // kernel only folds the inverse scaling of C into alpha)
+  static_assert(!PACKED_ || (PERSIST_ && !CPLX_ && P_ == Prec::FP16TCEC), "packed form");
   static constexpr bool PACKED = PACKED_;
   static_assert(!PERSIST_ || DEEP_, "persistent kernels use the three-buffer pipeline");
   static_assert(!SCALED_ || P_ == Prec::FP16TCEC, "scaling guards the fp16 range only");

@@ -19,10 +19,22 @@ constexpr int kRowsPerBlock = 64;
 
 // KC: the source is K-contiguous (element (row, kk) at src[row * ld + kk]);
 // else row-contiguous (src[kk * ld + row]).
+// scale_max != nullptr: the operand is multiplied by 2^14 / *scale_max (the
+// bits of 2^floor(log2 max|x|) recorded by the statistics pass) while it is
+// split, if that maximum is non-zero and *scale_flag has `flag_bit` set -- the
+// coefficient of the stand-alone scaling kernels, read on the device.
 template <bool KC>
 __global__ __launch_bounds__(256) void pack_split_kernel(const float *__restrict__ src, uint64_t ld,
                                                          uint32_t rows, uint32_t k,
-                                                         char *__restrict__ dst, uint32_t rows_pad) {
+                                                         char *__restrict__ dst, uint32_t rows_pad,
+                                                         const uint32_t *scale_max,
+                                                         const int *scale_flag, int flag_bit) {
+  float coef = 1.0f;
+  if (scale_max != nullptr) {
+    const float mx = __uint_as_float(*scale_max);
+    if ((*scale_flag & flag_bit) && mx != 0.0f) coef = 16384.0f / mx;
+    coef = __uint_as_float(__builtin_amdgcn_readfirstlane(__float_as_uint(coef)));
+  }
   const uint32_t kb = blockIdx.y;
   const uint32_t t = threadIdx.x;
   // lanes run along the contiguous direction of the source
@@ -38,7 +50,11 @@ __global__ __launch_bounds__(256) void pack_split_kernel(const float *__restrict
     x[j] = v;
   }
   u4_t out[2];
-  splitter<Prec::FP16TCEC>::run(x, out);
+  if (scale_max != nullptr) {
+    splitter<Prec::FP16TCEC>::run_scaled(x, out, coef, coef * 2048.0f);
+  } else {
+    splitter<Prec::FP16TCEC>::run(x, out);
+  }
   char *p = dst + ((uint64_t)kb * 2 * rows_pad + row) * 64 + ((chunk ^ (uint32_t)lds_swizzle((int)row)) << 4);
   *reinterpret_cast<u4_t *>(p) = out[0];
   *reinterpret_cast<u4_t *>(p + (uint64_t)rows_pad * 64) = out[1];
@@ -46,14 +62,15 @@ __global__ __launch_bounds__(256) void pack_split_kernel(const float *__restrict
 } // namespace
 
 void launch_pack_split(hipStream_t stream, const float *src, bool k_contiguous, uint64_t ld,
-                       uint32_t rows, uint32_t k, void *dst, uint32_t rows_pad) {
+                       uint32_t rows, uint32_t k, void *dst, uint32_t rows_pad,
+                       const uint32_t *scale_max, const int *scale_flag, int flag_bit) {
   const dim3 grid(rows_pad / kRowsPerBlock, (k + 31) / 32);
   if (k_contiguous) {
     hipLaunchKernelGGL(pack_split_kernel<true>, grid, dim3(256), 0, stream, src, ld, rows, k,
-                       static_cast<char *>(dst), rows_pad);
+                       static_cast<char *>(dst), rows_pad, scale_max, scale_flag, flag_bit);
   } else {
     hipLaunchKernelGGL(pack_split_kernel<false>, grid, dim3(256), 0, stream, src, ld, rows, k,
-                       static_cast<char *>(dst), rows_pad);
+                       static_cast<char *>(dst), rows_pad, scale_max, scale_flag, flag_bit);
   }
 }
 } // namespace cumpsgemm_amd

@@ -33,6 +33,12 @@ hipblasStatus_t cuMpSGEMM_cgemm_ex(cuMpSGEMM_handle_t handle, hipblasOperation_t
 int cuMpSGEMM_describe_tile_config(int compute_mode, int is_complex, int op_A, int op_B,
                                    int tile_class, char *buf, size_t buf_len);
 
+/* Bytes of device memory the handle currently holds as workspace for
+ * pre-split operands (0 until a call takes that path; grows on demand; freed
+ * by cuMpSGEMM_destroy).  No counterpart in the reference, whose kernels need
+ * no workspace beyond the fixed scratch of its handle. */
+size_t cuMpSGEMM_get_workspace_size(cuMpSGEMM_handle_t handle);
+
 /* The whole mode pipeline of an intercepted call, callable directly:
  *   FP16TCEC_SCALING: exp_max(A), exp_max(B) -> scale A, B in place -> FP16TCEC
  *                     GEMM -> scale C -> (optionally) undo the scaling of A, B

@@ -143,3 +143,45 @@ def test_fused_scaling_matches_in_place_scaling(O, handle, dev, monkeypatch, mod
                      np.zeros(m * n, a.dtype), m)
     for c in outs:
         assert O.residual(ref, c, m, n, m) <= 2.0 * O.residual(ref, cf, m, n, m)
+
+
+# Large real problems in FP16TCEC_SCALING take the pre-split path: A and B are
+# scaled and split once into fp16 planes (workspace of the handle) and the GEMM
+# kernel only folds the inverse scaling of C into alpha.  Same scaling, same
+# split, same order of accumulation as the two other forms -> same bits.
+@pytest.mark.parametrize("opa,opb,m,n,k", [
+    (N, N, 4096, 4096, 256),      # (the path is taken from m*n/(m+n) >= 1800 on)
+    (T, N, 4000, 3700, 300),      # ragged M, N and K
+    (N, T, 3800, 4100, 288),
+    (T, T, 3712, 4096, 256),
+])
+def test_scaled_pre_split_path_matches_the_other_forms(O, cg, torch_gpu, dev, monkeypatch, opa, opb, m, n, k):
+    a = (inputs.uniform(71, m * k) * np.float32(2.0 ** -22)).astype(np.float32)
+    b = (inputs.uniform(72, k * n) * np.float32(2.0 ** 5)).astype(np.float32)
+    h = cg.Handle()                      # a fresh handle owns no workspace yet
+    h.set_stream(torch_gpu.cuda.current_stream())
+    try:
+        outs = {}
+        for form in ("in_loop", "in_place", "pre_split"):
+            monkeypatch.delenv("CUMPSGEMM_NO_FUSED_SCALING", raising=False)
+            monkeypatch.delenv("CUMPSGEMM_PACKED", raising=False)
+            if form == "in_loop":
+                monkeypatch.setenv("CUMPSGEMM_PACKED", "0")
+            elif form == "in_place":
+                monkeypatch.setenv("CUMPSGEMM_NO_FUSED_SCALING", "1")
+                monkeypatch.setenv("CUMPSGEMM_PACKED", "0")   # (the unscaled pre-split path serves NT layouts)
+            c, a_after, b_after, _ = _pipeline(h, dev, SCALING, opa, opb, m, n, k, a, b)
+            # only the pre-split form holds a workspace: fp16 hi + lo planes of A and B
+            assert (h.workspace_size() >= (m + n) * k * 4) == (form == "pre_split")
+            assert np.array_equal(a_after.view(np.uint32), a.view(np.uint32))
+            assert np.array_equal(b_after.view(np.uint32), b.view(np.uint32))
+            outs[form] = c
+        assert np.array_equal(outs["pre_split"].view(np.uint32), outs["in_loop"].view(np.uint32))
+        assert np.array_equal(outs["pre_split"].view(np.uint32), outs["in_place"].view(np.uint32))
+    finally:
+        torch_gpu.cuda.synchronize()
+        h.close()
+    if opa == T and opb == N:            # the other forms are checked against FP64 elsewhere; once here
+        ref = O.gemm_fp64(opa, opb, m, n, k, 1.0, a, k, b, k)
+        cf = oracle_gemm(O, FP32, opa, opb, m, n, k, 1.0, a, k, b, k, 0.0, np.zeros(m * n, np.float32), m)
+        assert O.residual(ref, outs["pre_split"], m, n, m) <= 2.0 * O.residual(ref, cf, m, n, m)
