@@ -303,6 +303,7 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
   // the slow kind for both operands (A and B both M/N-contiguous, "NT": +15 % at
   // 8192^3); everywhere else the in-loop kernels are as fast and need no
   // workspace.  CUMPSGEMM_PACKED=1 / 0 forces / forbids the path.
+  bool fp16_served = false;
   if constexpr (!CPLX) {
     const char *fp = std::getenv("CUMPSGEMM_PACKED"); // "0" never, "1" whenever possible
     const bool never = fp != nullptr && fp[0] == '0', always = fp != nullptr && fp[0] == '1';
@@ -314,8 +315,16 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
     // scales as it splits) pays for every layout.
     const bool pays_scaled = h->fused_scaling && k >= 256 &&
                              (double)m * (double)n / ((double)m + (double)n) >= 1800.0;
-    if (mode == CUMPSGEMM_FP16TCEC && !never && shape_ok && (pays || pays_scaled || always) &&
-        force_cls <= 0 && force_split <= 1) {
+    // AUTO: the FP16TCEC candidate may take the path as well, gated by the
+    // launch flag like every AUTO kernel (pre-pass included); the bf16x3
+    // candidate then goes through the ordinary launch below, alone.  Both
+    // write C directly, which needs the bf16x3 plan to be free of split-K.
+    bool auto_ok = false;
+    if (mode == CUMPSGEMM_AUTO && pays_scaled && depth == 0) {
+      auto_ok = make_plan(h, launches[0].p, CPLX, a_kc, b_kc, m, n, k, batch, force_cls, force_split).ksplit == 1;
+    }
+    if ((mode == CUMPSGEMM_FP16TCEC || auto_ok) && !never && shape_ok &&
+        (pays || pays_scaled || always) && force_cls <= 0 && force_split <= 1) {
       const uint32_t mp = packed_rows(m), np = packed_rows(n);
       const uint64_t a_bytes = packed_bytes(mp, k), b_bytes = packed_bytes(np, k);
       if (a_bytes + b_bytes <= (16ull << 30) && mp * 64ull < 0xffffffffull && np * 64ull < 0xffffffffull) {
@@ -348,10 +357,12 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
             pargs.scale_max_b = max_b;
             pargs.scale_flag = sflag;
           }
+          const int *gate = auto_ok ? args.launch_flag : nullptr;
+          const uint32_t accept = auto_ok ? launches[1].accept : 0u;
           launch_pack_split(h->stream, reinterpret_cast<const float *>(a), a_kc, lda, (uint32_t)m,
-                            (uint32_t)k, pa, mp, max_a, sflag, 0x40);
+                            (uint32_t)k, pa, mp, max_a, sflag, 0x40, gate, accept);
           launch_pack_split(h->stream, reinterpret_cast<const float *>(b), b_kc, ldb, (uint32_t)n,
-                            (uint32_t)k, pb, np, max_b, sflag, 0x20);
+                            (uint32_t)k, pb, np, max_b, sflag, 0x20, gate, accept);
           pargs.a = pa;
           pargs.b = pb;
           pargs.lda = mp; // padded row counts of the packed operands
@@ -362,7 +373,8 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
           pargs.tiles_n = (uint32_t)((n + kPackedBN - 1) / kPackedBN);
           pargs.batch = 1;
           pargs.atomic_out = 0;
-          pargs.launch_flag = nullptr;
+          pargs.launch_flag = gate;
+          pargs.flag_accept_mask = accept;
           const uint64_t total = (uint64_t)pargs.tiles_m * pargs.tiles_n;
           const dim3 grid((unsigned)std::min<uint64_t>(total, h->num_cus), 1, 1);
           if (h->fused_scaling) {
@@ -376,7 +388,9 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
             log_error(std::string("packed GEMM launch failed: ") + hipGetErrorString(perr));
             return HIPBLAS_STATUS_EXECUTION_FAILED;
           }
-          return HIPBLAS_STATUS_SUCCESS;
+          if (!auto_ok) return HIPBLAS_STATUS_SUCCESS;
+          nlaunch = 1;        // the FP16TCEC candidate is served; bf16x3 remains
+          fp16_served = true; // (and is not cut into column blocks: they would come back here)
         }
       }
     }
@@ -391,7 +405,8 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
   // idle for the last round.  C's columns are independent, so such a problem is
   // cut in two: a first part whose tiles fill whole rounds, and the remaining
   // columns, planned on their own (typically with K split to fill the chip).
-  if (!split && batch == 1 && depth == 0 && k >= 256 && std::getenv("CUMPSGEMM_NO_COLUMN_SPLIT") == nullptr) {
+  if (!split && batch == 1 && depth == 0 && !fp16_served && k >= 256 &&
+      std::getenv("CUMPSGEMM_NO_COLUMN_SPLIT") == nullptr) {
     const KernelEntry *e0 = plan0.entry;
     const uint64_t slots = (uint64_t)h->num_cus * resident_groups(e0);
     const uint64_t tiles = (uint64_t)plan0.tiles_m * plan0.tiles_n;

@@ -28,7 +28,11 @@ __global__ __launch_bounds__(256) void pack_split_kernel(const float *__restrict
                                                          uint32_t rows, uint32_t k,
                                                          char *__restrict__ dst, uint32_t rows_pad,
                                                          const uint32_t *scale_max,
-                                                         const int *scale_flag, int flag_bit) {
+                                                         const int *scale_flag, int flag_bit,
+                                                         const int *launch_flag,
+                                                         uint32_t flag_accept_mask) {
+  // AUTO mode: nothing to do unless the launch flag names a mode this pass serves
+  if (launch_flag != nullptr && ((1u << (*launch_flag & 31)) & flag_accept_mask) == 0) return;
   float coef = 1.0f;
   if (scale_max != nullptr) {
     const float mx = __uint_as_float(*scale_max);
@@ -63,14 +67,17 @@ __global__ __launch_bounds__(256) void pack_split_kernel(const float *__restrict
 
 void launch_pack_split(hipStream_t stream, const float *src, bool k_contiguous, uint64_t ld,
                        uint32_t rows, uint32_t k, void *dst, uint32_t rows_pad,
-                       const uint32_t *scale_max, const int *scale_flag, int flag_bit) {
+                       const uint32_t *scale_max, const int *scale_flag, int flag_bit,
+                       const int *launch_flag, uint32_t flag_accept_mask) {
   const dim3 grid(rows_pad / kRowsPerBlock, (k + 31) / 32);
   if (k_contiguous) {
     hipLaunchKernelGGL(pack_split_kernel<true>, grid, dim3(256), 0, stream, src, ld, rows, k,
-                       static_cast<char *>(dst), rows_pad, scale_max, scale_flag, flag_bit);
+                       static_cast<char *>(dst), rows_pad, scale_max, scale_flag, flag_bit, launch_flag,
+                       flag_accept_mask);
   } else {
     hipLaunchKernelGGL(pack_split_kernel<false>, grid, dim3(256), 0, stream, src, ld, rows, k,
-                       static_cast<char *>(dst), rows_pad, scale_max, scale_flag, flag_bit);
+                       static_cast<char *>(dst), rows_pad, scale_max, scale_flag, flag_bit, launch_flag,
+                       flag_accept_mask);
   }
 }
 } // namespace cumpsgemm_amd

@@ -155,11 +155,15 @@ def test_fused_scaling_matches_in_place_scaling(O, handle, dev, monkeypatch, mod
     (N, T, 3800, 4100, 288),
     (T, T, 3712, 4096, 256),
 ])
-def test_scaled_pre_split_path_matches_the_other_forms(O, cg, torch_gpu, dev, monkeypatch, opa, opb, m, n, k):
+@pytest.mark.parametrize("mode", [SCALING, AUTO])
+def test_scaled_pre_split_path_matches_the_other_forms(O, cg, torch_gpu, dev, monkeypatch, mode, opa, opb, m, n, k):
     a = (inputs.uniform(71, m * k) * np.float32(2.0 ** -22)).astype(np.float32)
     b = (inputs.uniform(72, k * n) * np.float32(2.0 ** 5)).astype(np.float32)
     h = cg.Handle()                      # a fresh handle owns no workspace yet
     h.set_stream(torch_gpu.cuda.current_stream())
+    # AUTO: with a tenth of the elements allowed below the threshold A is found to need scaling
+    # and B to be fine as it is, so the FP16TCEC candidate runs, scaling A only
+    h.set_exp_stats_params(0.0, 2.0 ** -15, 0.1)
     try:
         outs = {}
         for form in ("in_loop", "in_place", "pre_split"):
@@ -170,7 +174,9 @@ def test_scaled_pre_split_path_matches_the_other_forms(O, cg, torch_gpu, dev, mo
             elif form == "in_place":
                 monkeypatch.setenv("CUMPSGEMM_NO_FUSED_SCALING", "1")
                 monkeypatch.setenv("CUMPSGEMM_PACKED", "0")   # (the unscaled pre-split path serves NT layouts)
-            c, a_after, b_after, _ = _pipeline(h, dev, SCALING, opa, opb, m, n, k, a, b)
+            c, a_after, b_after, ids = _pipeline(h, dev, mode, opa, opb, m, n, k, a, b)
+            if mode == AUTO:
+                assert h.get_dynamic_launch_flag(ids[2]) == (FP16TCEC | 0x40)
             # only the pre-split form holds a workspace: fp16 hi + lo planes of A and B
             assert (h.workspace_size() >= (m + n) * k * 4) == (form == "pre_split")
             assert np.array_equal(a_after.view(np.uint32), a.view(np.uint32))
@@ -185,3 +191,31 @@ def test_scaled_pre_split_path_matches_the_other_forms(O, cg, torch_gpu, dev, mo
         ref = O.gemm_fp64(opa, opb, m, n, k, 1.0, a, k, b, k)
         cf = oracle_gemm(O, FP32, opa, opb, m, n, k, 1.0, a, k, b, k, 0.0, np.zeros(m * n, np.float32), m)
         assert O.residual(ref, outs["pre_split"], m, n, m) <= 2.0 * O.residual(ref, cf, m, n, m)
+
+
+def test_auto_pre_split_path_steps_aside_for_bf16x3(O, cg, torch_gpu, dev, monkeypatch):
+    """Same shape class, but AUTO decides for TF32TCEC (no underflow tolerated):
+    the gated pre-pass and the gated FP16TCEC kernel do nothing, the bf16x3
+    kernel produces C -- the same bits as with the pre-split path forbidden."""
+    m, n, k = 4096, 4096, 256
+    a = (inputs.uniform(81, m * k) * np.float32(2.0 ** -22)).astype(np.float32)
+    b = (inputs.uniform(82, k * n) * np.float32(2.0 ** 5)).astype(np.float32)
+    h = cg.Handle()
+    h.set_stream(torch_gpu.cuda.current_stream())
+    try:
+        outs = []
+        for packed in ("0", None):
+            if packed is None:
+                monkeypatch.delenv("CUMPSGEMM_PACKED", raising=False)
+            else:
+                monkeypatch.setenv("CUMPSGEMM_PACKED", packed)
+            c, _, _, ids = _pipeline(h, dev, AUTO, N, N, m, n, k, a, b)
+            assert h.get_dynamic_launch_flag(ids[2]) & 0x1f == TF32TCEC
+            outs.append(c)
+        assert np.array_equal(outs[0].view(np.uint32), outs[1].view(np.uint32))
+    finally:
+        torch_gpu.cuda.synchronize()
+        h.close()
+    ref = O.gemm_fp64(N, N, m, n, k, 1.0, a, m, b, k)
+    cf = oracle_gemm(O, FP32, N, N, m, n, k, 1.0, a, m, b, k, 0.0, np.zeros(m * n, np.float32), m)
+    assert O.residual(ref, outs[1], m, n, m) <= 2.0 * O.residual(ref, cf, m, n, m)
