@@ -109,10 +109,13 @@ unsigned resident_groups(const KernelEntry *e) {
 // measurements on MI355X, and the cheapest wins:
 //   cost = rounds * (K-steps per chunk + 4) * tile area * resident groups / efficiency
 //          [+ a fixed charge when K is split]
-// rounds     = how many times the chip's CU slots must be refilled,
+// rounds     = how many times the chip's CU slots must be refilled (a problem
+//              smaller than one round is charged for the workgroups a CU
+//              really holds),
 // + 4        = a tile's fixed cost (pipeline fill, write-out) in K-steps,
 // efficiency = sustained MFMA rate relative to the 64x64 wave tile, which has
-//              the fewest LDS fragment reads per MFMA (64x32: 0.83, 32x32: 0.55),
+//              the fewest LDS fragment reads per MFMA (64x32: 0.83, 32x32: 0.55,
+//              less when a CU holds under two waves per SIMD),
 // split charge = the extra launch that prepares C (about four K-steps of the
 //              largest tile) plus the atomic write-out, which grows with the
 //              number of chunks adding into the same C.
@@ -137,14 +140,33 @@ Plan make_plan(const cuMpSGEMM_handle *h, Prec p, bool cplx, bool a_kc, bool b_k
     const unsigned res = resident_groups(e);
     const uint64_t slots = (uint64_t)h->num_cus * res;
     const int wave_area = e->wm * e->wn;
-    const double eff = wave_area >= 4096 ? 1.0 : (wave_area >= 2048 ? 0.83 : 0.55);
-    const double unit = (double)e->bm * e->bn * res / eff;
+    // efficiency with `groups` workgroups on a CU: the 32x32 wave tiles need
+    // two waves per SIMD to hide their own latencies (0.52 us per K-step for a
+    // lone 4-wave 64x64 workgroup, 0.65 us for two of them side by side)
+    auto eff_of = [&](double groups) {
+      if (wave_area >= 4096) return 1.0;
+      if (wave_area >= 2048) return 0.83;
+      const double waves_per_simd = (double)e->threads * groups / 256.0;
+      return waves_per_simd >= 2.0 ? 0.55 : (waves_per_simd >= 1.0 ? 0.375 : 0.19);
+    };
+    // (a tile's operand traffic per flop grows with 1/bm + 1/bn: charged lightly,
+    // which also settles ties in favour of the larger tile)
+    const double area = (double)e->bm * e->bn * (1.0 + 2.0 / e->bm + 2.0 / e->bn);
+    const double unit = area * res / eff_of((double)res);
     const double atomics = (double)m * (double)n * (double)batch * (cplx ? 2.0 : 1.0);
     for (uint64_t sp = 1; sp <= max_split; sp *= 2) {
       if (forced_split != 0 && sp != forced_split) continue;
-      const double rounds = (double)((tiles * sp + slots - 1) / slots);
+      // a problem that does not fill the CU slots once keeps fewer workgroups on
+      // a CU than could live there; otherwise whole rounds are charged
+      const uint64_t groups = tiles * sp;
       const double steps = (double)((nk + sp - 1) / sp) + 4.0;
-      double cost = rounds * steps * unit;
+      double cost;
+      if (groups < slots) {
+        const double per_cu = (double)((groups + h->num_cus - 1) / h->num_cus);
+        cost = steps * per_cu * area / eff_of(per_cu);
+      } else {
+        cost = steps * (double)((groups + slots - 1) / slots) * unit;
+      }
       if (sp > 1) cost += 4.0 * 256.0 * 128.0 + 0.1 * atomics * (double)sp;
       if (best < 0.0 || cost < best) {
         best = cost;
