@@ -316,8 +316,8 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
     return HIPBLAS_STATUS_SUCCESS;
   }
 
-  // Pre-split path (real FP16TCEC): split A and B once, up front, into fp16
-  // planes held in the handle's workspace, and run the kernel that only copies
+  // Pre-split path (real FP16TCEC and bf16x3): split A and B once, up front, into
+  // fp16 / bf16 planes held in the handle's workspace, and run the kernel that only copies
   // them into LDS.  Results are bit-identical to the in-loop split (same split,
   // same order of accumulation).  Measured on MI355X the K loop is limited by
   // the power the MFMAs draw on real data, not by the split arithmetic, so the
@@ -329,7 +329,12 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
   if constexpr (!CPLX) {
     const char *fp = std::getenv("CUMPSGEMM_PACKED"); // "0" never, "1" whenever possible
     const bool never = fp != nullptr && fp[0] == '0', always = fp != nullptr && fp[0] == '1';
-    const bool shape_ok = batch == 1 && k >= 128 && (uint64_t)m * n >= (uint64_t)h->num_cus * kPackedBM * kPackedBN;
+    // bf16x3 (explicit TF32TCEC mode): its in-loop three-way split costs 5.4
+    // vector instructions per MFMA, so the pre-pass pays for every layout
+    const bool bf16 = (mode == CUMPSGEMM_TF32TCEC);
+    const int pbm = bf16 ? kPackedBf16BM : kPackedBM, pbn = bf16 ? kPackedBf16BN : kPackedBN;
+    const unsigned planes = bf16 ? 3u : 2u;
+    const bool shape_ok = batch == 1 && k >= 128 && (uint64_t)m * n >= (uint64_t)h->num_cus * pbm * pbn;
     const bool pays = !a_kc && !b_kc && k >= 256 &&
                       (double)m * (double)n / ((double)m + (double)n) >= 1800.0;
     // With fused scaling the in-loop split costs one more instruction per pair
@@ -345,10 +350,13 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
     if (mode == CUMPSGEMM_AUTO && pays_scaled && depth == 0) {
       auto_ok = make_plan(h, launches[0].p, CPLX, a_kc, b_kc, m, n, k, batch, force_cls, force_split).ksplit == 1;
     }
-    if ((mode == CUMPSGEMM_FP16TCEC || auto_ok) && !never && shape_ok &&
-        (pays || pays_scaled || always) && force_cls <= 0 && force_split <= 1) {
+    // (measured break-even at 4096^2; + 5 % at 6144^3, + 7 - 10 % from 8192^2 on)
+    const bool pays_bf16 = bf16 && k >= 256 && (double)m * (double)n / ((double)m + (double)n) >= 2600.0;
+    if ((mode == CUMPSGEMM_FP16TCEC || bf16 || auto_ok) && !never && shape_ok &&
+        (bf16 ? (pays_bf16 || always) : (pays || pays_scaled || always)) && force_cls <= 0 &&
+        force_split <= 1) {
       const uint32_t mp = packed_rows(m), np = packed_rows(n);
-      const uint64_t a_bytes = packed_bytes(mp, k), b_bytes = packed_bytes(np, k);
+      const uint64_t a_bytes = packed_bytes(mp, k, planes), b_bytes = packed_bytes(np, k, planes);
       if (a_bytes + b_bytes <= (16ull << 30) && mp * 64ull < 0xffffffffull && np * 64ull < 0xffffffffull) {
         if (h->pack_ws_bytes < a_bytes + b_bytes) {
           // the previous workspace may still be in use by work queued on the stream
@@ -371,7 +379,7 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
           GemmArgs pargs = args;
           const uint32_t *max_a = nullptr, *max_b = nullptr;
           const int *sflag = nullptr;
-          if (h->fused_scaling) {
+          if (h->fused_scaling && !bf16) {
             max_a = &h->stats_slots[h->fused_slot_a].max_exp_bits;
             max_b = &h->stats_slots[h->fused_slot_b].max_exp_bits;
             sflag = h->flag_buffer + h->fused_flag;
@@ -382,24 +390,26 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
           const int *gate = auto_ok ? args.launch_flag : nullptr;
           const uint32_t accept = auto_ok ? launches[1].accept : 0u;
           launch_pack_split(h->stream, reinterpret_cast<const float *>(a), a_kc, lda, (uint32_t)m,
-                            (uint32_t)k, pa, mp, max_a, sflag, 0x40, gate, accept);
+                            (uint32_t)k, pa, mp, bf16, max_a, sflag, 0x40, gate, accept);
           launch_pack_split(h->stream, reinterpret_cast<const float *>(b), b_kc, ldb, (uint32_t)n,
-                            (uint32_t)k, pb, np, max_b, sflag, 0x20, gate, accept);
+                            (uint32_t)k, pb, np, bf16, max_b, sflag, 0x20, gate, accept);
           pargs.a = pa;
           pargs.b = pb;
           pargs.lda = mp; // padded row counts of the packed operands
           pargs.ldb = np;
           pargs.k = (uint32_t)((k + 31) / 32 * 32); // zero-padded to whole K-steps
           pargs.k_chunk = pargs.k;
-          pargs.tiles_m = (uint32_t)((m + kPackedBM - 1) / kPackedBM);
-          pargs.tiles_n = (uint32_t)((n + kPackedBN - 1) / kPackedBN);
+          pargs.tiles_m = (uint32_t)((m + pbm - 1) / pbm);
+          pargs.tiles_n = (uint32_t)((n + pbn - 1) / pbn);
           pargs.batch = 1;
           pargs.atomic_out = 0;
           pargs.launch_flag = gate;
           pargs.flag_accept_mask = accept;
           const uint64_t total = (uint64_t)pargs.tiles_m * pargs.tiles_n;
           const dim3 grid((unsigned)std::min<uint64_t>(total, h->num_cus), 1, 1);
-          if (h->fused_scaling) {
+          if (bf16) {
+            launch_packed_bf16x3_s(pargs, grid, h->stream);
+          } else if (h->fused_scaling) {
             launch_packed_scaled_fp16tcec_s(pargs, grid, h->stream);
           } else {
             launch_packed_fp16tcec_s(pargs, grid, h->stream);

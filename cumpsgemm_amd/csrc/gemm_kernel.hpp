@@ -234,7 +234,8 @@ template <Prec P_, bool CPLX_, bool A_KC_, bool B_KC_, int BM_, int BN_, int WM_
 struct GemmCfg {
   // (PACKED + SCALED: the operands were scaled when they were pre-split; the
   // kernel only folds the inverse scaling of C into alpha)
-  static_assert(!PACKED_ || (PERSIST_ && !CPLX_ && P_ == Prec::FP16TCEC), "packed form");
+  static_assert(!PACKED_ || (PERSIST_ && !CPLX_ && (P_ == Prec::FP16TCEC || P_ == Prec::BF16X3)),
+                "packed form");
   static constexpr bool PACKED = PACKED_;
   static_assert(!PERSIST_ || DEEP_, "persistent kernels use the three-buffer pipeline");
   static_assert(!SCALED_ || P_ == Prec::FP16TCEC, "scaling guards the fp16 range only");
@@ -407,6 +408,7 @@ struct tile_loader {
   // Staging registers of one thread: the 8 K-values (re, im) of each unit.
   struct Regs {
     f8_t v[U][NC];
+    u4_t third[U]; // pre-split operands with three planes: the third chunk
   };
 
   // interior tile: base points at element (row 0 of the tile, k 0 of the K-step).
@@ -471,8 +473,10 @@ struct tile_loader {
   // image, ROWS * 64 bytes each, `plane_bytes` apart.  Unit u of thread t is the
   // 16-byte chunk number t + u * NT of every plane; the two chunks (hi, lo)
   // travel in the unit's staging registers.
+  template <int NPL>
   __device__ static inline void load_packed(Regs &reg, const float *__restrict__ base,
                                             uint32_t plane_bytes) {
+    static_assert(NPL == 2 || NPL == 3, "two or three planes");
     if (!active(threadIdx.x)) return;
     const char *p = reinterpret_cast<const char *>(base);
 #pragma unroll
@@ -482,8 +486,11 @@ struct tile_loader {
       const float4 lo = *reinterpret_cast<const float4 *>(p + plane_bytes + off);
       reg.v[u][0][0] = hi.x; reg.v[u][0][1] = hi.y; reg.v[u][0][2] = hi.z; reg.v[u][0][3] = hi.w;
       reg.v[u][0][4] = lo.x; reg.v[u][0][5] = lo.y; reg.v[u][0][6] = lo.z; reg.v[u][0][7] = lo.w;
+      if constexpr (NPL == 3)
+        reg.third[u] = *reinterpret_cast<const u4_t *>(p + 2u * plane_bytes + off);
     }
   }
+  template <int NPL>
   __device__ static inline void store_packed(Regs &reg, char *lds_op, int tid) {
     constexpr int PLANE = ROWS * 64;
     if (!active(tid)) return;
@@ -493,6 +500,7 @@ struct tile_loader {
       const f8_t v = reg.v[u][0];
       *reinterpret_cast<float4 *>(lds_op + off) = make_float4(v[0], v[1], v[2], v[3]);
       *reinterpret_cast<float4 *>(lds_op + PLANE + off) = make_float4(v[4], v[5], v[6], v[7]);
+      if constexpr (NPL == 3) *reinterpret_cast<u4_t *>(lds_op + 2 * PLANE + off) = reg.third[u];
     }
   }
 
@@ -714,8 +722,8 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
     const float *ap = a_tile + (uint64_t)kt * a_kstep;
     const float *bp = b_tile + (uint64_t)kt * b_kstep;
     if constexpr (Cfg::PACKED) {
-      LA::load_packed(ra, ap, (uint32_t)args.lda * 64u);
-      LB::load_packed(rb, bp, (uint32_t)args.ldb * 64u);
+      LA::template load_packed<NP>(ra, ap, (uint32_t)args.lda * 64u);
+      LB::template load_packed<NP>(rb, bp, (uint32_t)args.ldb * 64u);
     } else if constexpr (FAST) {
       LA::load_fast(ra, ap, args.lda, offa);
       LB::load_fast(rb, bp, args.ldb, offb);
@@ -729,8 +737,8 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
     char *sa = lds + stage * Cfg::STAGE_BYTES;
     char *sb = sa + Cfg::A_STAGE_BYTES;
     if constexpr (Cfg::PACKED) {
-      LA::store_packed(ra, sa, tid);
-      LB::store_packed(rb, sb, tid);
+      LA::template store_packed<NP>(ra, sa, tid);
+      LB::template store_packed<NP>(rb, sb, tid);
     } else {
       LA::template store<P, Cfg::SCALED>(ra, sa, tid, coef_a, coef_a2048);
       LB::template store<P, Cfg::SCALED>(rb, sb, tid, coef_b, coef_b2048);

@@ -1,17 +1,19 @@
-// Pre-split of an FP32 operand into fp16 planes (see pack_split.hip).
+// Pre-split of an FP32 operand into fp16 or bf16 planes (see pack_split.hip).
 #pragma once
 #include <hip/hip_runtime.h>
 #include <cstdint>
 
 namespace cumpsgemm_amd {
 // bytes of the packed form of a (rows x k) operand
-inline uint64_t packed_bytes(uint64_t rows_pad, uint64_t k) { return ((k + 31) / 32) * 2 * rows_pad * 64; }
+inline uint64_t packed_bytes(uint64_t rows_pad, uint64_t k, unsigned planes = 2) {
+  return ((k + 31) / 32) * planes * rows_pad * 64;
+}
 inline uint32_t packed_rows(uint64_t rows) { return (uint32_t)((rows + 255) / 256 * 256); }
 // scale_max / scale_flag / flag_bit: optional power-of-two scaling fused into
 // the split (nullptr: none); launch_flag / flag_accept_mask: optional AUTO-mode
 // gate, as in GemmArgs
 void launch_pack_split(hipStream_t stream, const float *src, bool k_contiguous, uint64_t ld,
-                       uint32_t rows, uint32_t k, void *dst, uint32_t rows_pad,
+                       uint32_t rows, uint32_t k, void *dst, uint32_t rows_pad, bool bf16x3,
                        const uint32_t *scale_max = nullptr, const int *scale_flag = nullptr,
                        int flag_bit = 0, const int *launch_flag = nullptr,
                        uint32_t flag_accept_mask = 0);

@@ -285,7 +285,7 @@ def test_edge_tiles_split_k(O, handle, dev, monkeypatch, cls):
 
 
 # ---- pre-split (packed) path ------------------------------------------------------
-# Large real FP16TCEC problems split A and B once into fp16 planes (workspace of the
+# Large real FP16TCEC / bf16x3 problems split A and B once into fp16 / bf16 planes (workspace of the
 # handle) and run a kernel that only copies them into LDS.  Same split, same order of
 # accumulation: the result must equal the in-loop kernels' bit for bit.
 @pytest.mark.parametrize("opa,opb,m,n,k,pads,alpha,beta", [
@@ -294,7 +294,8 @@ def test_edge_tiles_split_k(O, handle, dev, monkeypatch, cls):
     (N, T, 2304, 4100, 1000, (0, 5, 0), 1.0, 1.0),
     (T, T, 3333, 2777, 129, (2, 0, 1), -1.0, 0.25),
 ])
-def test_packed_path_matches_in_loop_split(O, handle, dev, monkeypatch, opa, opb, m, n, k, pads, alpha, beta):
+@pytest.mark.parametrize("mode", [FP16TCEC, TF32TCEC])
+def test_packed_path_matches_in_loop_split(O, handle, dev, monkeypatch, mode, opa, opb, m, n, k, pads, alpha, beta):
     a, lda = make_operand(inputs.uniform, 61, opa, m, k, pads[0])
     b, ldb = make_operand(inputs.uniform, 62, opb, k, n, pads[1])
     ldc = m + pads[2]
@@ -302,7 +303,7 @@ def test_packed_path_matches_in_loop_split(O, handle, dev, monkeypatch, opa, opb
     outs = []
     for packed in ("1", "0"):
         monkeypatch.setenv("CUMPSGEMM_PACKED", packed)
-        c, st, mid = run_gemm(handle, dev, FP16TCEC, opa, opb, m, n, k, alpha, a, lda, b, ldb, beta, c0, ldc, False,
+        c, st, mid = run_gemm(handle, dev, mode, opa, opb, m, n, k, alpha, a, lda, b, ldb, beta, c0, ldc, False,
                               want_module_id=True)
         assert st == 0 and (mid == 200) == (packed == "1")
         outs.append(c)
