@@ -334,7 +334,9 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
     const bool bf16 = (mode == CUMPSGEMM_TF32TCEC);
     const int pbm = bf16 ? kPackedBf16BM : kPackedBM, pbn = bf16 ? kPackedBf16BN : kPackedBN;
     const unsigned planes = bf16 ? 3u : 2u;
-    const bool shape_ok = batch == 1 && k >= 128 && (uint64_t)m * n >= (uint64_t)h->num_cus * pbm * pbn;
+    // (the pre-pass launches workgroups of 64 rows x 32 .. 256 K-values on a 2-D grid)
+    const bool shape_ok = batch == 1 && k >= 128 && (uint64_t)m * n >= (uint64_t)h->num_cus * pbm * pbn &&
+                          k / 32 < 65535;
     const bool pays = !a_kc && !b_kc && k >= 256 &&
                       (double)m * (double)n / ((double)m + (double)n) >= 1800.0;
     // With fused scaling the in-loop split costs one more instruction per pair
@@ -350,8 +352,8 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
     if (mode == CUMPSGEMM_AUTO && pays_scaled && depth == 0) {
       auto_ok = make_plan(h, launches[0].p, CPLX, a_kc, b_kc, m, n, k, batch, force_cls, force_split).ksplit == 1;
     }
-    // (measured break-even at 4096^2; + 5 % at 6144^3, + 7 - 10 % from 8192^2 on)
-    const bool pays_bf16 = bf16 && k >= 256 && (double)m * (double)n / ((double)m + (double)n) >= 2600.0;
+    // (measured: - 4 % at 3072^3, + 5 % at 4096^3, + 8 % at 6144^3, + 10 % from 8192^2 on)
+    const bool pays_bf16 = bf16 && k >= 512 && (double)m * (double)n / ((double)m + (double)n) >= 2000.0;
     if ((mode == CUMPSGEMM_FP16TCEC || bf16 || auto_ok) && !never && shape_ok &&
         (bf16 ? (pays_bf16 || always) : (pays || pays_scaled || always)) && force_cls <= 0 &&
         force_split <= 1) {

@@ -12,11 +12,12 @@
 //   c ^ lds_swizzle(row).
 // HBM-bound: reads 4 bytes and writes 4 (6) bytes per element.
 #include "gemm_kernel.hpp"
+#include <algorithm>
 #include "pack_split.hpp"
 
 namespace cumpsgemm_amd {
 namespace {
-constexpr int kRowsPerBlock = 64;
+constexpr uint32_t kRowsPerBlock = 64;
 
 // KC: the source is K-contiguous (element (row, kk) at src[row * ld + kk]);
 // else row-contiguous (src[kk * ld + row]).
@@ -31,7 +32,8 @@ __global__ __launch_bounds__(256) void pack_split_kernel(const float *__restrict
                                                          const uint32_t *scale_max,
                                                          const int *scale_flag, int flag_bit,
                                                          const int *launch_flag,
-                                                         uint32_t flag_accept_mask) {
+                                                         uint32_t flag_accept_mask,
+                                                         uint32_t steps_per_block) {
   // AUTO mode: nothing to do unless the launch flag names a mode this pass serves
   if (launch_flag != nullptr && ((1u << (*launch_flag & 31)) & flag_accept_mask) == 0) return;
   float coef = 1.0f;
@@ -40,34 +42,96 @@ __global__ __launch_bounds__(256) void pack_split_kernel(const float *__restrict
     if ((*scale_flag & flag_bit) && mx != 0.0f) coef = 16384.0f / mx;
     coef = __uint_as_float(__builtin_amdgcn_readfirstlane(__float_as_uint(coef)));
   }
-  const uint32_t kb = blockIdx.y;
+  // One workgroup converts `steps_per_block` K-steps of 64 rows, thread = (row,
+  // 16-byte chunk), two steps in flight.  Lanes run along the contiguous
+  // direction of the source:
+  //   KC:  4 lanes per row -> steps_per_block * 128 contiguous bytes of every
+  //        row; the 4 lanes of a row write its whole 64-byte plane rows;
+  //   !KC: 64 lanes along the rows -> 256 contiguous bytes of each K-line; a
+  //        lane's chunks are 16 bytes out of every 64 of the destination, so
+  //        they are gathered in LDS -- which then holds the destination image
+  //        of the block, 4 KiB per plane -- and written out as a linear copy.
+  const uint32_t k_steps = (k + 31) / 32;
+  const uint32_t kb0 = blockIdx.y * steps_per_block;
   const uint32_t t = threadIdx.x;
-  // lanes run along the contiguous direction of the source
-  const uint32_t row = blockIdx.x * kRowsPerBlock + (KC ? t / 4 : t % kRowsPerBlock);
+  const uint32_t lrow = KC ? t / 4 : t % kRowsPerBlock; // row within the block
+  const uint32_t row = blockIdx.x * kRowsPerBlock + lrow;
   const uint32_t chunk = KC ? t % 4 : t / kRowsPerBlock;
-  const uint32_t k0 = kb * 32 + chunk * 8;
-  f8_t x;
-#pragma unroll
-  for (int j = 0; j < 8; j++) {
-    const uint32_t kk = k0 + j;
-    float v = 0.0f;
-    if (row < rows && kk < k) v = KC ? src[(uint64_t)row * ld + kk] : src[(uint64_t)kk * ld + row];
-    x[j] = v;
-  }
+  const bool row_in = row < rows;
   constexpr int NP = prec_traits<P>::NP;
-  u4_t out[NP];
-  if constexpr (P == Prec::FP16TCEC) {
-    if (scale_max != nullptr) {
-      splitter<P>::run_scaled(x, out, coef, coef * 2048.0f);
-    } else {
-      splitter<P>::run(x, out);
-    }
-  } else {
-    splitter<P>::run(x, out); // (bf16 has FP32's exponent range: never scaled)
-  }
-  char *p = dst + ((uint64_t)kb * NP * rows_pad + row) * 64 + ((chunk ^ (uint32_t)lds_swizzle((int)row)) << 4);
+  typedef float f4u_t __attribute__((ext_vector_type(4), aligned(4)));
+  __shared__ __attribute__((aligned(16))) char stage[KC ? 1 : 2][NP][KC ? 16 : kRowsPerBlock * 64];
+
+  auto load = [&](uint32_t kb, f8_t &x) {
+    const uint32_t k0 = kb * 32 + chunk * 8;
+    if (row_in && k0 + 8 <= k) {
+      if constexpr (KC) {
+        const float *p = src + (uint64_t)row * ld + k0;
+        const f4u_t lo = *reinterpret_cast<const f4u_t *>(p), hi = *reinterpret_cast<const f4u_t *>(p + 4);
+        x = f8_t{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      } else {
+        const float *p = src + (uint64_t)k0 * ld + row;
 #pragma unroll
-  for (int pl = 0; pl < NP; pl++) *reinterpret_cast<u4_t *>(p + (uint64_t)pl * rows_pad * 64) = out[pl];
+        for (int j = 0; j < 8; j++) x[j] = p[(uint64_t)j * ld];
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; j++) {
+        const uint32_t kk = k0 + j;
+        float v = 0.0f;
+        if (row_in && kk < k) v = KC ? src[(uint64_t)row * ld + kk] : src[(uint64_t)kk * ld + row];
+        x[j] = v;
+      }
+    }
+  };
+  // position of the thread's chunk inside the 64-row block image of one plane
+  const uint32_t pos = lrow * 64 + ((chunk ^ (uint32_t)lds_swizzle((int)row)) << 4);
+  auto split_to = [&](const f8_t &x, uint32_t kb, int buf) {
+    u4_t out[NP];
+    if constexpr (P == Prec::FP16TCEC) {
+      if (scale_max != nullptr) {
+        splitter<P>::run_scaled(x, out, coef, coef * 2048.0f);
+      } else {
+        splitter<P>::run(x, out);
+      }
+    } else {
+      splitter<P>::run(x, out); // (bf16 has FP32's exponent range: never scaled)
+    }
+#pragma unroll
+    for (int pl = 0; pl < NP; pl++) {
+      if constexpr (KC) {
+        char *p = dst + (((uint64_t)kb * NP + pl) * rows_pad + (uint64_t)blockIdx.x * kRowsPerBlock) * 64;
+        *reinterpret_cast<u4_t *>(p + pos) = out[pl];
+      } else {
+        *reinterpret_cast<u4_t *>(&stage[buf][pl][pos]) = out[pl];
+      }
+    }
+  };
+  auto copy_out = [&](uint32_t kb, int buf) { // !KC: 256 threads x 16 bytes = one plane of the block
+#pragma unroll
+    for (int pl = 0; pl < NP; pl++) {
+      char *p = dst + (((uint64_t)kb * NP + pl) * rows_pad + (uint64_t)blockIdx.x * kRowsPerBlock) * 64;
+      *reinterpret_cast<u4_t *>(p + t * 16) = *reinterpret_cast<const u4_t *>(&stage[buf][pl][t * 16]);
+    }
+  };
+  for (uint32_t s = 0; s < steps_per_block; s += 2) {
+    const uint32_t ka = kb0 + s, kb = ka + 1;
+    if (ka >= k_steps) break; // uniform
+    const bool two = (s + 1 < steps_per_block) && (kb < k_steps);
+    f8_t xa, xb;
+    load(ka, xa);
+    if (two) load(kb, xb);
+    if constexpr (!KC) {
+      if (s > 0) __syncthreads(); // the previous pair's copies have read the stage
+    }
+    split_to(xa, ka, 0);
+    if (two) split_to(xb, kb, 1);
+    if constexpr (!KC) {
+      __syncthreads();
+      copy_out(ka, 0);
+      if (two) copy_out(kb, 1);
+    }
+  }
 }
 } // namespace
 
@@ -75,10 +139,13 @@ void launch_pack_split(hipStream_t stream, const float *src, bool k_contiguous, 
                        uint32_t rows, uint32_t k, void *dst, uint32_t rows_pad, bool bf16x3,
                        const uint32_t *scale_max, const int *scale_flag, int flag_bit,
                        const int *launch_flag, uint32_t flag_accept_mask) {
-  const dim3 grid(rows_pad / kRowsPerBlock, (k + 31) / 32);
+  // up to 8 K-steps per workgroup, fewer while that would leave under ~2048 workgroups
+  const unsigned k_steps = (k + 31) / 32, row_blocks = rows_pad / kRowsPerBlock;
+  const unsigned spb = (unsigned)std::max<uint64_t>(1, std::min<uint64_t>(8, (uint64_t)k_steps * row_blocks / 2048));
+  const dim3 grid(row_blocks, (k_steps + spb - 1) / spb);
   auto launch = [&](auto kernel) {
     hipLaunchKernelGGL(kernel, grid, dim3(256), 0, stream, src, ld, rows, k, static_cast<char *>(dst),
-                       rows_pad, scale_max, scale_flag, flag_bit, launch_flag, flag_accept_mask);
+                       rows_pad, scale_max, scale_flag, flag_bit, launch_flag, flag_accept_mask, spb);
   };
   if (bf16x3) {
     if (k_contiguous) launch(pack_split_kernel<true, Prec::BF16X3>);
