@@ -1,0 +1,64 @@
+"""The GEMM entry points and the FP16TCEC_SCALING / AUTO pipelines only launch
+kernels on the handle's stream (no allocation, memset, copy or synchronisation
+once the handle exists), so a caller can capture them into a HIP graph.  Each
+replay is checked against an eager call on the same inputs, with the inputs
+changed and eager work run between replays."""
+import numpy as np
+import pytest
+
+from cumpsgemm_amd import inputs
+
+pytestmark = pytest.mark.gpu
+N_OP = 111
+FP16TCEC, TF32TCEC, AUTO, SCALING = 1, 2, 9, 11
+
+
+@pytest.mark.parametrize("mode,cplx", [(FP16TCEC, False), (TF32TCEC, False), (FP16TCEC, True),
+                                       (SCALING, False), (AUTO, False)])
+def test_captured_calls_replay_like_eager_calls(cg, torch_gpu, mode, cplx):
+    torch = torch_gpu
+    m, n, k = 640, 384, 512
+    es = 2 if cplx else 1
+    dev = torch.device("cuda:0")
+    h = cg.Handle()
+    side = torch.cuda.Stream()
+    a = torch.empty(m * k * es, device=dev)
+    b = torch.empty(k * n * es, device=dev)
+    c_graph = torch.zeros(m * n * es, device=dev)
+    c_eager = torch.zeros(m * n * es, device=dev)
+
+    def call(c_out):
+        if mode in (SCALING, AUTO):
+            st, _ = h.gemm_pipeline(N_OP, N_OP, m, n, k, 1.0, a, m, b, k, 0.0, c_out, m, mode, cplx=cplx)
+        else:
+            st = h.gemm(N_OP, N_OP, m, n, k, 1.0, a, m, b, k, 0.0, c_out, m, mode, cplx=cplx)
+        assert st == 0
+
+    def fill(seed, scale):
+        a.copy_(torch.from_numpy(inputs.uniform(seed, m * k * es) * np.float32(scale)).to(dev))
+        b.copy_(torch.from_numpy(inputs.uniform(seed + 1, k * n * es)).to(dev))
+
+    try:
+        fill(1, 1.0)
+        h.set_stream(side)
+        with torch.cuda.stream(side):
+            call(c_graph)                       # warm-up outside the capture (lazy kernel loading)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=side):
+            h.set_stream(torch.cuda.current_stream())
+            call(c_graph)
+        for rep, scale in enumerate((1.0, 2.0 ** -18, 3.0)):
+            fill(10 + 2 * rep, scale)
+            c_graph.zero_()
+            torch.cuda.synchronize()
+            g.replay()
+            torch.cuda.synchronize()
+            h.set_stream(torch.cuda.current_stream())
+            call(c_eager)                       # eager work between the replays
+            torch.cuda.synchronize()
+            assert torch.equal(c_graph, c_eager), (mode, cplx, rep)
+            assert float(c_eager.abs().max()) > 0
+    finally:
+        torch.cuda.synchronize()
+        h.close()
