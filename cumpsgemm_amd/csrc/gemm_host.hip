@@ -195,6 +195,13 @@ Plan make_plan(const cuMpSGEMM_handle *h, Prec p, bool cplx, bool a_kc, bool b_k
 // every K-chunk a multiple of the 32-wide step and at least four steps long,
 // and every per-thread offset must fit 31 bits.
 constexpr unsigned kPersistentMaxSteps = 32; // K-steps per tile up to which tiles are walked
+unsigned persistent_max_steps() {
+  static const unsigned max_steps = [] {
+    const char *e = std::getenv("CUMPSGEMM_PERSISTENT_MAX_STEPS");
+    return e != nullptr ? (unsigned)std::atoi(e) : kPersistentMaxSteps;
+  }();
+  return max_steps;
+}
 
 template <class T>
 bool persistent_ok(const KernelEntry *e, bool a_kc, bool b_kc, uint64_t m, uint64_t n, uint64_t k,
@@ -209,11 +216,7 @@ bool persistent_ok(const KernelEntry *e, bool a_kc, bool b_kc, uint64_t m, uint6
   // asking memory for the same K range in lockstep.  (The kernels with fused
   // scaling are the exception: their one-tile form measures 7 % slower for the
   // NN layout, so they walk tiles of any length.)
-  static const unsigned max_steps = [] {
-    const char *e = std::getenv("CUMPSGEMM_PERSISTENT_MAX_STEPS");
-    return e != nullptr ? (unsigned)std::atoi(e) : kPersistentMaxSteps;
-  }();
-  if (!any_length && plan.k_chunk / 32 > max_steps) return false;
+  if (!any_length && plan.k_chunk / 32 > persistent_max_steps()) return false;
   auto fits = [&](bool kc, uint64_t rows, uint64_t ld) {
     const uint64_t span = kc ? rows * ld + 32 : 32 * ld + rows;
     return span * ES * 4 < 0x7fffffffull;
@@ -317,14 +320,13 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
   }
 
   // Pre-split path (real FP16TCEC and bf16x3): split A and B once, up front, into
-  // fp16 / bf16 planes held in the handle's workspace, and run the kernel that only copies
-  // them into LDS.  Results are bit-identical to the in-loop split (same split,
-  // same order of accumulation).  Measured on MI355X the K loop is limited by
-  // the power the MFMAs draw on real data, not by the split arithmetic, so the
-  // pre-pass (one read + write of A and B) only pays where the in-loop loads are
-  // the slow kind for both operands (A and B both M/N-contiguous, "NT": +15 % at
-  // 8192^3); everywhere else the in-loop kernels are as fast and need no
-  // workspace.  CUMPSGEMM_PACKED=1 / 0 forces / forbids the path.
+  // fp16 / bf16 planes held in the handle's workspace, and run the kernel that
+  // only copies them into LDS.  Results are bit-identical to the in-loop split
+  // (same split, same order of accumulation).  The pre-pass is one read + write
+  // of A and B at 5 - 6 TB/s; what it buys is a K loop without split arithmetic,
+  // which runs at a higher clock under the power limit.  It pays for large
+  // problems (rules below, per mode and layout); the in-loop kernels serve the
+  // rest and need no workspace.  CUMPSGEMM_PACKED=1 / 0 forces / forbids the path.
   bool fp16_served = false;
   if constexpr (!CPLX) {
     const char *fp = std::getenv("CUMPSGEMM_PACKED"); // "0" never, "1" whenever possible
@@ -337,13 +339,20 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
     // (the pre-pass launches workgroups of 64 rows x 32 .. 256 K-values on a 2-D grid)
     const bool shape_ok = batch == 1 && k >= 128 && (uint64_t)m * n >= (uint64_t)h->num_cus * pbm * pbn &&
                           k / 32 < 65535;
-    const bool pays = !a_kc && !b_kc && k >= 256 &&
-                      (double)m * (double)n / ((double)m + (double)n) >= 1800.0;
+    const double mn_ratio = (double)m * (double)n / ((double)m + (double)n);
+    const bool pays_nt = !a_kc && !b_kc && k >= 256 && mn_ratio >= 1800.0;
+    // Every other layout: the pre-split kernel, freed of the split arithmetic,
+    // outruns the in-loop one by more than the pre-pass costs once the problem
+    // is large (8192^3: 381 vs 361 - 372 TFLOP/s; 8192^2 x 1024: 351 vs 318 -
+    // 343) -- provided the tiles fill the CU slots in whole rounds or in many:
+    // the path has no column split for a mostly empty last round.
+    const uint64_t ptiles = ((m + pbm - 1) / pbm) * ((n + pbn - 1) / pbn);
+    const bool rounds_ok = ptiles % h->num_cus == 0 || ptiles >= 6ull * h->num_cus;
+    const bool pays = pays_nt || (k >= 1024 && mn_ratio >= 3000.0 && rounds_ok);
     // With fused scaling the in-loop split costs one more instruction per pair
     // and those kernels run 8 - 25 % below the plain ones, so the pre-pass (which
     // scales as it splits) pays for every layout.
-    const bool pays_scaled = h->fused_scaling && k >= 256 &&
-                             (double)m * (double)n / ((double)m + (double)n) >= 1800.0;
+    const bool pays_scaled = h->fused_scaling && k >= 256 && mn_ratio >= 1800.0;
     // AUTO: the FP16TCEC candidate may take the path as well, gated by the
     // launch flag like every AUTO kernel (pre-pass included); the bf16x3
     // candidate then goes through the ordinary launch below, alone.  Both
@@ -353,7 +362,7 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
       auto_ok = make_plan(h, launches[0].p, CPLX, a_kc, b_kc, m, n, k, batch, force_cls, force_split).ksplit == 1;
     }
     // (measured: - 4 % at 3072^3, + 5 % at 4096^3, + 8 % at 6144^3, + 10 % from 8192^2 on)
-    const bool pays_bf16 = bf16 && k >= 512 && (double)m * (double)n / ((double)m + (double)n) >= 2000.0;
+    const bool pays_bf16 = bf16 && k >= 512 && mn_ratio >= 2000.0;
     if ((mode == CUMPSGEMM_FP16TCEC || bf16 || auto_ok) && !never && shape_ok &&
         (bf16 ? (pays_bf16 || always) : (pays || pays_scaled || always)) && force_cls <= 0 &&
         force_split <= 1) {
@@ -408,13 +417,19 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
           pargs.launch_flag = gate;
           pargs.flag_accept_mask = accept;
           const uint64_t total = (uint64_t)pargs.tiles_m * pargs.tiles_n;
-          const dim3 grid((unsigned)std::min<uint64_t>(total, h->num_cus), 1, 1);
+          // short tiles are walked by persistent workgroups, long ones get a workgroup each
+          // (measured cross-over: 16 K-steps for the fp16 kernel, which gains 6 - 8 % from
+          // the one-tile form at 8192^3, the usual 32 for bf16x3, which gains nothing)
+          bool walk = bf16 ? pargs.k / 32 <= persistent_max_steps() : pargs.k / 32 < 16;
+          if (const char *w = std::getenv("CUMPSGEMM_PACKED_WALK")) walk = w[0] == '1';
+          const dim3 grid = walk ? dim3((unsigned)std::min<uint64_t>(total, h->num_cus), 1, 1)
+                                 : dim3((unsigned)total, 1, 1);
           if (bf16) {
-            launch_packed_bf16x3_s(pargs, grid, h->stream);
+            launch_packed_bf16x3_s(pargs, grid, h->stream, walk);
           } else if (h->fused_scaling) {
-            launch_packed_scaled_fp16tcec_s(pargs, grid, h->stream);
+            launch_packed_scaled_fp16tcec_s(pargs, grid, h->stream, walk);
           } else {
-            launch_packed_fp16tcec_s(pargs, grid, h->stream);
+            launch_packed_fp16tcec_s(pargs, grid, h->stream, walk);
           }
           if (used_id != nullptr) *used_id = 200u; // pre-split path
           const hipError_t perr = hipGetLastError();

@@ -7,10 +7,16 @@ namespace cumpsgemm_amd {
     CUMPSGEMM_ENTRY(Prec::BF16X3, false, AKC, BKC, 128, 128, 64, 32, 2, true, "128x128x32_w64x32_deep"), \
     CUMPSGEMM_ENTRY(Prec::BF16X3, false, AKC, BKC, 64, 64, 32, 32, 2, false, "64x64x32_w32x32") }
 CUMPSGEMM_DEFINE_TABLE(g_tab_bf16x3_s, ROW)
-// the large tile over pre-split operands (three bf16 planes, K-contiguous)
-void launch_packed_bf16x3_s(const GemmArgs &args, dim3 grid, hipStream_t stream) {
-  launch_cfg<GemmCfg<Prec::BF16X3, false, true, true, 128, 128, 64, 32, 2, true, true, false, true>>(
-      args, grid, stream);
+// the large tile over pre-split operands (three bf16 planes, K-contiguous);
+// `walk`: persistent form (short tiles) or one tile per workgroup
+void launch_packed_bf16x3_s(const GemmArgs &args, dim3 grid, hipStream_t stream, bool walk) {
+  if (walk) {
+    launch_cfg<GemmCfg<Prec::BF16X3, false, true, true, 128, 128, 64, 32, 2, true, true, false, true>>(
+        args, grid, stream);
+  } else {
+    launch_cfg<GemmCfg<Prec::BF16X3, false, true, true, 128, 128, 64, 32, 2, true, false, false, true>>(
+        args, grid, stream);
+  }
 }
 #undef ROW
 } // namespace cumpsgemm_amd

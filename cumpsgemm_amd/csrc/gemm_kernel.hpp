@@ -225,7 +225,7 @@ __device__ inline f16v_t mfma32(const u4_t a, const u4_t b, const f16v_t c) {
 //   SCALED (FP16TCEC only): op(A), op(B) are multiplied by powers of two read
 //         from device memory while they are split, and the result by the
 //         inverse product when it is written out (see GemmArgs).
-//   PACKED (persistent, real FP16TCEC): A and B were split beforehand into
+//   PACKED (three-buffer kernels, real FP16TCEC / bf16x3): A and B were split beforehand into
 //         fp16 planes laid out as the LDS image of every (tile, K-step), see
 //         pack_split_kernel; staging is a plain 16-byte copy, no arithmetic.
 template <Prec P_, bool CPLX_, bool A_KC_, bool B_KC_, int BM_, int BN_, int WM_,
@@ -234,7 +234,7 @@ template <Prec P_, bool CPLX_, bool A_KC_, bool B_KC_, int BM_, int BN_, int WM_
 struct GemmCfg {
   // (PACKED + SCALED: the operands were scaled when they were pre-split; the
   // kernel only folds the inverse scaling of C into alpha)
-  static_assert(!PACKED_ || (PERSIST_ && !CPLX_ && (P_ == Prec::FP16TCEC || P_ == Prec::BF16X3)),
+  static_assert(!PACKED_ || (DEEP_ && !CPLX_ && (P_ == Prec::FP16TCEC || P_ == Prec::BF16X3)),
                 "packed form");
   static constexpr bool PACKED = PACKED_;
   static_assert(!PERSIST_ || DEEP_, "persistent kernels use the three-buffer pipeline");
@@ -681,8 +681,9 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
   const int rows_b = (int)((args.n - nl0 < (uint32_t)BN) ? args.n - nl0 : BN);
   // unguarded loads: the (moved) tile lies inside the matrix and every
   // per-thread offset fits 31 bits
-  const bool a_full = (rows_a == BM) && LA::offsets_fit(args.lda);
-  const bool b_full = (rows_b == BN) && LB::offsets_fit(args.ldb);
+  // (pre-split operands are padded to whole tiles and K-steps: always unguarded)
+  const bool a_full = Cfg::PACKED || ((rows_a == BM) && LA::offsets_fit(args.lda));
+  const bool b_full = Cfg::PACKED || ((rows_b == BN) && LB::offsets_fit(args.ldb));
 
   uint32_t offa[Cfg::UA], offb[Cfg::UB];
 #pragma unroll

@@ -81,9 +81,9 @@ CUMPSGEMM_DECLARE_TABLE(g_tab_bf16x2_c)
 #undef CUMPSGEMM_DECLARE_TABLE
 
 // Real FP16TCEC, 256x128 tile, persistent, operands pre-split by launch_pack_split.
-void launch_packed_fp16tcec_s(const GemmArgs &args, dim3 grid, hipStream_t stream);
-void launch_packed_scaled_fp16tcec_s(const GemmArgs &args, dim3 grid, hipStream_t stream);
-void launch_packed_bf16x3_s(const GemmArgs &args, dim3 grid, hipStream_t stream);
+void launch_packed_fp16tcec_s(const GemmArgs &args, dim3 grid, hipStream_t stream, bool walk);
+void launch_packed_scaled_fp16tcec_s(const GemmArgs &args, dim3 grid, hipStream_t stream, bool walk);
+void launch_packed_bf16x3_s(const GemmArgs &args, dim3 grid, hipStream_t stream, bool walk);
 constexpr int kPackedBM = 256, kPackedBN = 128;             // FP16TCEC
 constexpr int kPackedBf16BM = 128, kPackedBf16BN = 128;     // bf16x3
 
