@@ -25,11 +25,12 @@ sys.path.insert(0, ROOT)
 
 FP16_MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per 8192^3 FP16TCEC launch from the rocprofv3 FETCH_SIZE + WRITE_SIZE
-# counters, scaled by what the same counters read for a plain copy of known size
-# (profiles/gemm_fp16tcec_8192_nn.md).  This is L2-miss traffic on the fabric
-# (Infinity Cache or HBM); the algorithmic minimum is 3 * 8192^2 * 4 B = 0.805e9.
-GEMM_TRAFFIC_BYTES = 5.70e9
+# HBM bytes per 8192^3 FP16TCEC launch of the GEMM kernel from the rocprofv3
+# FETCH_SIZE + WRITE_SIZE counters, scaled by what the same counters read for a
+# plain copy of known size (profiles/gemm_fp16tcec_8192_nn.md).  This is L2-miss
+# traffic on the fabric (Infinity Cache or HBM); the algorithmic minimum is
+# 3 * 8192^2 * 4 B = 0.805e9.  The call's two pre-split passes add 1.07e9.
+GEMM_TRAFFIC_BYTES = 5.64e9
 
 
 def log(*a):
@@ -229,7 +230,10 @@ def main():
             "unit": "TFLOP/s",
             "frac": round(kernel_tflops / FP16_MFMA_PEAK_TFLOPS, 4),
             "traffic": GEMM_TRAFFIC_BYTES if n == 8192 else None,
+            # one call = two pre-split passes (about 0.2 ms) + the GEMM kernel: all inside
             "kernel_ms": round(ev_ms, 4),
+            "kernels_per_step": "2 x pack_split_kernel + gemm_tcec_kernel (packed)" if n >= 6144 else
+                                "gemm_tcec_kernel",
             # the split-and-correct algorithm issues 3 MFMA products per logical product
             "mfma_products_per_flop": 3,
             "mfma_issued_tflops": round(3.0 * kernel_tflops, 1),
