@@ -127,6 +127,8 @@ def main():
         h.close()
         return
     wall_ms, ev_ms = timed(tcec(cg.FP16TCEC), args.steps, args.warmup)
+    # which path served the call: 200 = pre-split operands, else the tile class of the in-loop kernel
+    _, module_id = h.gemm(cg.OP_N, cg.OP_N, m, n, k, 1.0, a, n, b, n, 0.0, c, n, cg.FP16TCEC, want_module_id=True)
     value = flops / (wall_ms * 1e-3) / 1e12
     kernel_tflops = flops / (ev_ms * 1e-3) / 1e12
 
@@ -232,7 +234,7 @@ def main():
             "traffic": GEMM_TRAFFIC_BYTES if n == 8192 else None,
             # one call = two pre-split passes (about 0.2 ms) + the GEMM kernel: all inside
             "kernel_ms": round(ev_ms, 4),
-            "kernels_per_step": "2 x pack_split_kernel + gemm_tcec_kernel (packed)" if n >= 6144 else
+            "kernels_per_step": "2 x pack_split_kernel + gemm_tcec_kernel (packed)" if module_id == 200 else
                                 "gemm_tcec_kernel",
             # the split-and-correct algorithm issues 3 MFMA products per logical product
             "mfma_products_per_flop": 3,
