@@ -344,10 +344,11 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
     // Every other layout: the pre-split kernel, freed of the split arithmetic,
     // outruns the in-loop one by more than the pre-pass costs once the problem
     // is large (8192^3: 381 vs 361 - 372 TFLOP/s; 8192^2 x 1024: 351 vs 318 -
-    // 343) -- provided the tiles fill the CU slots in whole rounds or in many:
-    // the path has no column split for a mostly empty last round.
+    // 343) -- provided the last round of CU slots is at least half full or one
+    // of many: the path has no column split for a mostly empty last round.
     const uint64_t ptiles = ((m + pbm - 1) / pbm) * ((n + pbn - 1) / pbn);
-    const bool rounds_ok = ptiles % h->num_cus == 0 || ptiles >= 6ull * h->num_cus;
+    const uint64_t last_round = ptiles % h->num_cus;
+    const bool rounds_ok = last_round == 0 || 2 * last_round >= h->num_cus || ptiles >= 6ull * h->num_cus;
     const bool pays = pays_nt || (k >= 1024 && mn_ratio >= 3000.0 && rounds_ok);
     // With fused scaling the in-loop split costs one more instruction per pair
     // and those kernels run 8 - 25 % below the plain ones, so the pre-pass (which
