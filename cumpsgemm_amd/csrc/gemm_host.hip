@@ -328,14 +328,15 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
   // problems (rules below, per mode and layout); the in-loop kernels serve the
   // rest and need no workspace.  CUMPSGEMM_PACKED=1 / 0 forces / forbids the path.
   bool fp16_served = false;
-  if constexpr (!CPLX) {
+  if (!CPLX || mode == CUMPSGEMM_FP16TCEC) { // (complex: FP16TCEC only, also under FP16TCEC_SCALING)
     const char *fp = std::getenv("CUMPSGEMM_PACKED"); // "0" never, "1" whenever possible
     const bool never = fp != nullptr && fp[0] == '0', always = fp != nullptr && fp[0] == '1';
     // bf16x3 (explicit TF32TCEC mode): its in-loop three-way split costs 5.4
     // vector instructions per MFMA, so the pre-pass pays for every layout
     const bool bf16 = (mode == CUMPSGEMM_TF32TCEC);
-    const int pbm = bf16 ? kPackedBf16BM : kPackedBM, pbn = bf16 ? kPackedBf16BN : kPackedBN;
-    const unsigned planes = bf16 ? 3u : 2u;
+    const int pbm = CPLX ? kPackedCplxBM : (bf16 ? kPackedBf16BM : kPackedBM);
+    const int pbn = CPLX ? kPackedCplxBN : (bf16 ? kPackedBf16BN : kPackedBN);
+    const unsigned planes = CPLX ? 4u : (bf16 ? 3u : 2u);
     // (the pre-pass launches workgroups of 64 rows x 32 .. 256 K-values on a 2-D grid)
     const bool shape_ok = batch == 1 && k >= 128 && (uint64_t)m * n >= (uint64_t)h->num_cus * pbm * pbn &&
                           k / 32 < 65535;
@@ -349,7 +350,8 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
     const uint64_t ptiles = ((m + pbm - 1) / pbm) * ((n + pbn - 1) / pbn);
     const uint64_t last_round = ptiles % h->num_cus;
     const bool rounds_ok = last_round == 0 || 2 * last_round >= h->num_cus || ptiles >= 6ull * h->num_cus;
-    const bool pays = pays_nt || (k >= 1024 && mn_ratio >= 3000.0 && rounds_ok);
+    // (complex: four times the MFMA work per element split, so the pre-pass weighs less)
+    const bool pays = pays_nt || (k >= 1024 && mn_ratio >= (CPLX ? 1500.0 : 3000.0) && rounds_ok);
     // With fused scaling the in-loop split costs one more instruction per pair
     // and those kernels run 8 - 25 % below the plain ones, so the pre-pass (which
     // scales as it splits) pays for every layout.
@@ -359,7 +361,7 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
     // candidate then goes through the ordinary launch below, alone.  Both
     // write C directly, which needs the bf16x3 plan to be free of split-K.
     bool auto_ok = false;
-    if (mode == CUMPSGEMM_AUTO && pays_scaled && depth == 0) {
+    if (!CPLX && mode == CUMPSGEMM_AUTO && pays_scaled && depth == 0) {
       auto_ok = make_plan(h, launches[0].p, CPLX, a_kc, b_kc, m, n, k, batch, force_cls, force_split).ksplit == 1;
     }
     // (measured: - 4 % at 3072^3, + 5 % at 4096^3, + 8 % at 6144^3, + 10 % from 8192^2 on)
@@ -399,12 +401,13 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
             pargs.scale_max_b = max_b;
             pargs.scale_flag = sflag;
           }
+          const PackKind kind = CPLX ? PackKind::FP16_COMPLEX : (bf16 ? PackKind::BF16X3_REAL : PackKind::FP16_REAL);
           const int *gate = auto_ok ? args.launch_flag : nullptr;
           const uint32_t accept = auto_ok ? launches[1].accept : 0u;
           launch_pack_split(h->stream, reinterpret_cast<const float *>(a), a_kc, lda, (uint32_t)m,
-                            (uint32_t)k, pa, mp, bf16, max_a, sflag, 0x40, gate, accept);
+                            (uint32_t)k, pa, mp, kind, max_a, sflag, 0x40, gate, accept);
           launch_pack_split(h->stream, reinterpret_cast<const float *>(b), b_kc, ldb, (uint32_t)n,
-                            (uint32_t)k, pb, np, bf16, max_b, sflag, 0x20, gate, accept);
+                            (uint32_t)k, pb, np, kind, max_b, sflag, 0x20, gate, accept);
           pargs.a = pa;
           pargs.b = pb;
           pargs.lda = mp; // padded row counts of the packed operands
@@ -421,11 +424,13 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
           // short tiles are walked by persistent workgroups, long ones get a workgroup each
           // (measured cross-over: 16 K-steps for the fp16 kernel, which gains 6 - 8 % from
           // the one-tile form at 8192^3, the usual 32 for bf16x3, which gains nothing)
-          bool walk = bf16 ? pargs.k / 32 <= persistent_max_steps() : pargs.k / 32 < 16;
+          bool walk = (bf16 || CPLX) ? pargs.k / 32 <= persistent_max_steps() : pargs.k / 32 < 16;
           if (const char *w = std::getenv("CUMPSGEMM_PACKED_WALK")) walk = w[0] == '1';
           const dim3 grid = walk ? dim3((unsigned)std::min<uint64_t>(total, h->num_cus), 1, 1)
                                  : dim3((unsigned)total, 1, 1);
-          if (bf16) {
+          if constexpr (CPLX) {
+            launch_packed_fp16tcec_c(pargs, grid, h->stream, walk, h->fused_scaling);
+          } else if (bf16) {
             launch_packed_bf16x3_s(pargs, grid, h->stream, walk);
           } else if (h->fused_scaling) {
             launch_packed_scaled_fp16tcec_s(pargs, grid, h->stream, walk);

@@ -234,7 +234,7 @@ template <Prec P_, bool CPLX_, bool A_KC_, bool B_KC_, int BM_, int BN_, int WM_
 struct GemmCfg {
   // (PACKED + SCALED: the operands were scaled when they were pre-split; the
   // kernel only folds the inverse scaling of C into alpha)
-  static_assert(!PACKED_ || (DEEP_ && !CPLX_ && (P_ == Prec::FP16TCEC || P_ == Prec::BF16X3)),
+  static_assert(!PACKED_ || (DEEP_ && (P_ == Prec::FP16TCEC || (P_ == Prec::BF16X3 && !CPLX_))),
                 "packed form");
   static constexpr bool PACKED = PACKED_;
   static_assert(!PERSIST_ || DEEP_, "persistent kernels use the three-buffer pipeline");
@@ -476,16 +476,19 @@ struct tile_loader {
   template <int NPL>
   __device__ static inline void load_packed(Regs &reg, const float *__restrict__ base,
                                             uint32_t plane_bytes) {
-    static_assert(NPL == 2 || NPL == 3, "two or three planes");
+    static_assert(NPL == 2 || NPL == 3 || (NPL == 4 && NC == 2), "2, 3 or (complex) 2 x 2 planes");
     if (!active(threadIdx.x)) return;
     const char *p = reinterpret_cast<const char *>(base);
 #pragma unroll
     for (int u = 0; u < U; u++) {
       const uint32_t off = (uint32_t)(threadIdx.x + u * NT) * 16u;
-      const float4 hi = *reinterpret_cast<const float4 *>(p + off);
-      const float4 lo = *reinterpret_cast<const float4 *>(p + plane_bytes + off);
-      reg.v[u][0][0] = hi.x; reg.v[u][0][1] = hi.y; reg.v[u][0][2] = hi.z; reg.v[u][0][3] = hi.w;
-      reg.v[u][0][4] = lo.x; reg.v[u][0][5] = lo.y; reg.v[u][0][6] = lo.z; reg.v[u][0][7] = lo.w;
+#pragma unroll
+      for (int q = 0; q < (NPL == 4 ? 2 : 1); q++) { // complex: (re hi, re lo), (im hi, im lo)
+        const float4 hi = *reinterpret_cast<const float4 *>(p + (2u * q) * plane_bytes + off);
+        const float4 lo = *reinterpret_cast<const float4 *>(p + (2u * q + 1u) * plane_bytes + off);
+        reg.v[u][q][0] = hi.x; reg.v[u][q][1] = hi.y; reg.v[u][q][2] = hi.z; reg.v[u][q][3] = hi.w;
+        reg.v[u][q][4] = lo.x; reg.v[u][q][5] = lo.y; reg.v[u][q][6] = lo.z; reg.v[u][q][7] = lo.w;
+      }
       if constexpr (NPL == 3)
         reg.third[u] = *reinterpret_cast<const u4_t *>(p + 2u * plane_bytes + off);
     }
@@ -497,9 +500,12 @@ struct tile_loader {
 #pragma unroll
     for (int u = 0; u < U; u++) {
       const int off = (tid + u * NT) * 16;
-      const f8_t v = reg.v[u][0];
-      *reinterpret_cast<float4 *>(lds_op + off) = make_float4(v[0], v[1], v[2], v[3]);
-      *reinterpret_cast<float4 *>(lds_op + PLANE + off) = make_float4(v[4], v[5], v[6], v[7]);
+#pragma unroll
+      for (int q = 0; q < (NPL == 4 ? 2 : 1); q++) {
+        const f8_t v = reg.v[u][q];
+        *reinterpret_cast<float4 *>(lds_op + 2 * q * PLANE + off) = make_float4(v[0], v[1], v[2], v[3]);
+        *reinterpret_cast<float4 *>(lds_op + (2 * q + 1) * PLANE + off) = make_float4(v[4], v[5], v[6], v[7]);
+      }
       if constexpr (NPL == 3) *reinterpret_cast<u4_t *>(lds_op + 2 * PLANE + off) = reg.third[u];
     }
   }
@@ -663,15 +669,15 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
   // Pre-split operands: lda / ldb are the padded row counts; one K-step holds
   // NP planes of (rows x 64 bytes), i.e. 16 floats per row and plane.
   auto packed_origin = [&](const float *base, uint64_t rows_pad, uint32_t row0) {
-    return base + ((uint64_t)(kbeg / BK) * NP * rows_pad + row0) * 16;
+    return base + ((uint64_t)(kbeg / BK) * (NP * NCOMP) * rows_pad + row0) * 16;
   };
   if constexpr (Cfg::PACKED) {
     a_tile = packed_origin(a, args.lda, ml0);
     b_tile = packed_origin(b, args.ldb, nl0);
   }
-  const uint64_t a_kstep = Cfg::PACKED ? (uint64_t)NP * args.lda * 16
+  const uint64_t a_kstep = Cfg::PACKED ? (uint64_t)(NP * NCOMP) * args.lda * 16
                            : Cfg::A_KC ? (uint64_t)BK * ES : (uint64_t)BK * args.lda * ES;
-  const uint64_t b_kstep = Cfg::PACKED ? (uint64_t)NP * args.ldb * 16
+  const uint64_t b_kstep = Cfg::PACKED ? (uint64_t)(NP * NCOMP) * args.ldb * 16
                            : Cfg::B_KC ? (uint64_t)BK * ES : (uint64_t)BK * args.ldb * ES;
 
   using LA = tile_loader<CPLX, Cfg::A_KC, BM, Cfg::UA, NT>;
@@ -723,8 +729,8 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
     const float *ap = a_tile + (uint64_t)kt * a_kstep;
     const float *bp = b_tile + (uint64_t)kt * b_kstep;
     if constexpr (Cfg::PACKED) {
-      LA::template load_packed<NP>(ra, ap, (uint32_t)args.lda * 64u);
-      LB::template load_packed<NP>(rb, bp, (uint32_t)args.ldb * 64u);
+      LA::template load_packed<NP * NCOMP>(ra, ap, (uint32_t)args.lda * 64u);
+      LB::template load_packed<NP * NCOMP>(rb, bp, (uint32_t)args.ldb * 64u);
     } else if constexpr (FAST) {
       LA::load_fast(ra, ap, args.lda, offa);
       LB::load_fast(rb, bp, args.ldb, offb);
@@ -738,8 +744,8 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
     char *sa = lds + stage * Cfg::STAGE_BYTES;
     char *sb = sa + Cfg::A_STAGE_BYTES;
     if constexpr (Cfg::PACKED) {
-      LA::template store_packed<NP>(ra, sa, tid);
-      LB::template store_packed<NP>(rb, sb, tid);
+      LA::template store_packed<NP * NCOMP>(ra, sa, tid);
+      LB::template store_packed<NP * NCOMP>(rb, sb, tid);
     } else {
       LA::template store<P, Cfg::SCALED>(ra, sa, tid, coef_a, coef_a2048);
       LB::template store<P, Cfg::SCALED>(rb, sb, tid, coef_b, coef_b2048);

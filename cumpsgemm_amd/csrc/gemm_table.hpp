@@ -86,6 +86,8 @@ void launch_packed_scaled_fp16tcec_s(const GemmArgs &args, dim3 grid, hipStream_
 void launch_packed_bf16x3_s(const GemmArgs &args, dim3 grid, hipStream_t stream, bool walk);
 constexpr int kPackedBM = 256, kPackedBN = 128;             // FP16TCEC
 constexpr int kPackedBf16BM = 128, kPackedBf16BN = 128;     // bf16x3
+void launch_packed_fp16tcec_c(const GemmArgs &args, dim3 grid, hipStream_t stream, bool walk, bool scaled);
+constexpr int kPackedCplxBM = 128, kPackedCplxBN = 64;      // complex FP16TCEC
 
 // One table = the same three tile classes for each of the four layout pairs.
 // ROW(AKC, BKC) must expand to three make_entry<...>() initialisers.

@@ -1,5 +1,5 @@
-// Pre-split of a whole FP32 operand into fp16 hi / lo planes (FP16TCEC) or three
-// bf16 planes (bf16x3) for the packed kernels.  For large problems every element of A is otherwise split
+// Pre-split of a whole FP32 / complex64 operand into fp16 hi / lo planes
+// (FP16TCEC) or three bf16 planes (bf16x3) for the packed kernels.  For large problems every element of A is otherwise split
 // once per column of tiles (and B once per row of tiles) inside the GEMM's K
 // loop; doing it once up front takes the vector arithmetic out of that loop.
 //
@@ -25,7 +25,7 @@ constexpr uint32_t kRowsPerBlock = 64;
 // bits of 2^floor(log2 max|x|) recorded by the statistics pass) while it is
 // split, if that maximum is non-zero and *scale_flag has `flag_bit` set -- the
 // coefficient of the stand-alone scaling kernels, read on the device.
-template <bool KC, Prec P>
+template <bool KC, Prec P, bool CPLX>
 __global__ __launch_bounds__(256) void pack_split_kernel(const float *__restrict__ src, uint64_t ld,
                                                          uint32_t rows, uint32_t k,
                                                          char *__restrict__ dst, uint32_t rows_pad,
@@ -45,12 +45,16 @@ __global__ __launch_bounds__(256) void pack_split_kernel(const float *__restrict
   // One workgroup converts `steps_per_block` K-steps of 64 rows, thread = (row,
   // 16-byte chunk), two steps in flight.  Lanes run along the contiguous
   // direction of the source:
-  //   KC:  4 lanes per row -> steps_per_block * 128 contiguous bytes of every
-  //        row; the 4 lanes of a row write its whole 64-byte plane rows;
-  //   !KC: 64 lanes along the rows -> 256 contiguous bytes of each K-line; a
-  //        lane's chunks are 16 bytes out of every 64 of the destination, so
-  //        they are gathered in LDS -- which then holds the destination image
-  //        of the block, 4 KiB per plane -- and written out as a linear copy.
+  //   KC:  4 lanes per row -> steps_per_block * 128 (complex: 256) contiguous
+  //        bytes of every row; the 4 lanes of a row write its whole 64-byte
+  //        plane rows;
+  //   !KC: 64 lanes along the rows -> 256 (512) contiguous bytes of each
+  //        K-line; a lane's chunks are 16 bytes out of every 64 of the
+  //        destination, so they are gathered in LDS -- which then holds the
+  //        destination image of the block, 4 KiB per plane -- and written out
+  //        as a linear copy.
+  // Complex sources are interleaved (re, im); their planes are re hi, re lo,
+  // im hi, im lo.
   const uint32_t k_steps = (k + 31) / 32;
   const uint32_t kb0 = blockIdx.y * steps_per_block;
   const uint32_t t = threadIdx.x;
@@ -58,67 +62,100 @@ __global__ __launch_bounds__(256) void pack_split_kernel(const float *__restrict
   const uint32_t row = blockIdx.x * kRowsPerBlock + lrow;
   const uint32_t chunk = KC ? t % 4 : t / kRowsPerBlock;
   const bool row_in = row < rows;
+  constexpr int NC = CPLX ? 2 : 1;
   constexpr int NP = prec_traits<P>::NP;
+  constexpr int NPL = NP * NC; // planes per K-step
   typedef float f4u_t __attribute__((ext_vector_type(4), aligned(4)));
-  __shared__ __attribute__((aligned(16))) char stage[KC ? 1 : 2][NP][KC ? 16 : kRowsPerBlock * 64];
+  typedef float f2u_t __attribute__((ext_vector_type(2), aligned(4)));
+  __shared__ __attribute__((aligned(16))) char stage[KC ? 1 : 2][NPL][KC ? 16 : kRowsPerBlock * 64];
 
-  auto load = [&](uint32_t kb, f8_t &x) {
+  struct Vals {
+    f8_t c[NC]; // the 8 K-values of the thread's chunk: real parts, imaginary parts
+  };
+  auto load = [&](uint32_t kb, Vals &x) {
     const uint32_t k0 = kb * 32 + chunk * 8;
     if (row_in && k0 + 8 <= k) {
       if constexpr (KC) {
-        const float *p = src + (uint64_t)row * ld + k0;
-        const f4u_t lo = *reinterpret_cast<const f4u_t *>(p), hi = *reinterpret_cast<const f4u_t *>(p + 4);
-        x = f8_t{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-      } else {
-        const float *p = src + (uint64_t)k0 * ld + row;
+        const float *p = src + ((uint64_t)row * ld + k0) * NC;
+        if constexpr (!CPLX) {
+          const f4u_t lo = *reinterpret_cast<const f4u_t *>(p), hi = *reinterpret_cast<const f4u_t *>(p + 4);
+          x.c[0] = f8_t{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        } else {
 #pragma unroll
-        for (int j = 0; j < 8; j++) x[j] = p[(uint64_t)j * ld];
+          for (int j = 0; j < 4; j++) {
+            const f4u_t v = *reinterpret_cast<const f4u_t *>(p + 4 * j); // two complex values
+            x.c[0][2 * j] = v[0];
+            x.c[1][2 * j] = v[1];
+            x.c[0][2 * j + 1] = v[2];
+            x.c[1][2 * j + 1] = v[3];
+          }
+        }
+      } else {
+        const float *p = src + ((uint64_t)k0 * ld + row) * NC;
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+          if constexpr (!CPLX) {
+            x.c[0][j] = p[(uint64_t)j * ld];
+          } else {
+            const f2u_t v = *reinterpret_cast<const f2u_t *>(p + (uint64_t)j * ld * 2);
+            x.c[0][j] = v[0];
+            x.c[1][j] = v[1];
+          }
+        }
       }
     } else {
 #pragma unroll
       for (int j = 0; j < 8; j++) {
         const uint32_t kk = k0 + j;
-        float v = 0.0f;
-        if (row_in && kk < k) v = KC ? src[(uint64_t)row * ld + kk] : src[(uint64_t)kk * ld + row];
-        x[j] = v;
+#pragma unroll
+        for (int q = 0; q < NC; q++) {
+          float v = 0.0f;
+          if (row_in && kk < k)
+            v = KC ? src[((uint64_t)row * ld + kk) * NC + q] : src[((uint64_t)kk * ld + row) * NC + q];
+          x.c[q][j] = v;
+        }
       }
     }
   };
   // position of the thread's chunk inside the 64-row block image of one plane
   const uint32_t pos = lrow * 64 + ((chunk ^ (uint32_t)lds_swizzle((int)row)) << 4);
-  auto split_to = [&](const f8_t &x, uint32_t kb, int buf) {
-    u4_t out[NP];
-    if constexpr (P == Prec::FP16TCEC) {
-      if (scale_max != nullptr) {
-        splitter<P>::run_scaled(x, out, coef, coef * 2048.0f);
-      } else {
-        splitter<P>::run(x, out);
-      }
-    } else {
-      splitter<P>::run(x, out); // (bf16 has FP32's exponent range: never scaled)
-    }
+  auto split_to = [&](const Vals &x, uint32_t kb, int buf) {
 #pragma unroll
-    for (int pl = 0; pl < NP; pl++) {
-      if constexpr (KC) {
-        char *p = dst + (((uint64_t)kb * NP + pl) * rows_pad + (uint64_t)blockIdx.x * kRowsPerBlock) * 64;
-        *reinterpret_cast<u4_t *>(p + pos) = out[pl];
+    for (int q = 0; q < NC; q++) {
+      u4_t out[NP];
+      if constexpr (P == Prec::FP16TCEC) {
+        if (scale_max != nullptr) {
+          splitter<P>::run_scaled(x.c[q], out, coef, coef * 2048.0f);
+        } else {
+          splitter<P>::run(x.c[q], out);
+        }
       } else {
-        *reinterpret_cast<u4_t *>(&stage[buf][pl][pos]) = out[pl];
+        splitter<P>::run(x.c[q], out); // (bf16 has FP32's exponent range: never scaled)
+      }
+#pragma unroll
+      for (int pl = 0; pl < NP; pl++) {
+        const int plane = q * NP + pl;
+        if constexpr (KC) {
+          char *p = dst + (((uint64_t)kb * NPL + plane) * rows_pad + (uint64_t)blockIdx.x * kRowsPerBlock) * 64;
+          *reinterpret_cast<u4_t *>(p + pos) = out[pl];
+        } else {
+          *reinterpret_cast<u4_t *>(&stage[buf][plane][pos]) = out[pl];
+        }
       }
     }
   };
   auto copy_out = [&](uint32_t kb, int buf) { // !KC: 256 threads x 16 bytes = one plane of the block
 #pragma unroll
-    for (int pl = 0; pl < NP; pl++) {
-      char *p = dst + (((uint64_t)kb * NP + pl) * rows_pad + (uint64_t)blockIdx.x * kRowsPerBlock) * 64;
-      *reinterpret_cast<u4_t *>(p + t * 16) = *reinterpret_cast<const u4_t *>(&stage[buf][pl][t * 16]);
+    for (int plane = 0; plane < NPL; plane++) {
+      char *p = dst + (((uint64_t)kb * NPL + plane) * rows_pad + (uint64_t)blockIdx.x * kRowsPerBlock) * 64;
+      *reinterpret_cast<u4_t *>(p + t * 16) = *reinterpret_cast<const u4_t *>(&stage[buf][plane][t * 16]);
     }
   };
   for (uint32_t s = 0; s < steps_per_block; s += 2) {
     const uint32_t ka = kb0 + s, kb = ka + 1;
     if (ka >= k_steps) break; // uniform
     const bool two = (s + 1 < steps_per_block) && (kb < k_steps);
-    f8_t xa, xb;
+    Vals xa, xb;
     load(ka, xa);
     if (two) load(kb, xb);
     if constexpr (!KC) {
@@ -136,7 +173,7 @@ __global__ __launch_bounds__(256) void pack_split_kernel(const float *__restrict
 } // namespace
 
 void launch_pack_split(hipStream_t stream, const float *src, bool k_contiguous, uint64_t ld,
-                       uint32_t rows, uint32_t k, void *dst, uint32_t rows_pad, bool bf16x3,
+                       uint32_t rows, uint32_t k, void *dst, uint32_t rows_pad, PackKind kind,
                        const uint32_t *scale_max, const int *scale_flag, int flag_bit,
                        const int *launch_flag, uint32_t flag_accept_mask) {
   // up to 8 K-steps per workgroup, fewer while that would leave under ~2048 workgroups
@@ -147,12 +184,19 @@ void launch_pack_split(hipStream_t stream, const float *src, bool k_contiguous, 
     hipLaunchKernelGGL(kernel, grid, dim3(256), 0, stream, src, ld, rows, k, static_cast<char *>(dst),
                        rows_pad, scale_max, scale_flag, flag_bit, launch_flag, flag_accept_mask, spb);
   };
-  if (bf16x3) {
-    if (k_contiguous) launch(pack_split_kernel<true, Prec::BF16X3>);
-    else launch(pack_split_kernel<false, Prec::BF16X3>);
-  } else {
-    if (k_contiguous) launch(pack_split_kernel<true, Prec::FP16TCEC>);
-    else launch(pack_split_kernel<false, Prec::FP16TCEC>);
+  switch (kind) {
+  case PackKind::BF16X3_REAL:
+    if (k_contiguous) launch(pack_split_kernel<true, Prec::BF16X3, false>);
+    else launch(pack_split_kernel<false, Prec::BF16X3, false>);
+    break;
+  case PackKind::FP16_COMPLEX:
+    if (k_contiguous) launch(pack_split_kernel<true, Prec::FP16TCEC, true>);
+    else launch(pack_split_kernel<false, Prec::FP16TCEC, true>);
+    break;
+  default:
+    if (k_contiguous) launch(pack_split_kernel<true, Prec::FP16TCEC, false>);
+    else launch(pack_split_kernel<false, Prec::FP16TCEC, false>);
+    break;
   }
 }
 } // namespace cumpsgemm_amd

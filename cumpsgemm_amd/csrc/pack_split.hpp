@@ -9,11 +9,13 @@ inline uint64_t packed_bytes(uint64_t rows_pad, uint64_t k, unsigned planes = 2)
   return ((k + 31) / 32) * planes * rows_pad * 64;
 }
 inline uint32_t packed_rows(uint64_t rows) { return (uint32_t)((rows + 255) / 256 * 256); }
+enum class PackKind { FP16_REAL, FP16_COMPLEX, BF16X3_REAL };
+// `ld` in elements of the source (complex: complex elements).
 // scale_max / scale_flag / flag_bit: optional power-of-two scaling fused into
 // the split (nullptr: none); launch_flag / flag_accept_mask: optional AUTO-mode
 // gate, as in GemmArgs
 void launch_pack_split(hipStream_t stream, const float *src, bool k_contiguous, uint64_t ld,
-                       uint32_t rows, uint32_t k, void *dst, uint32_t rows_pad, bool bf16x3,
+                       uint32_t rows, uint32_t k, void *dst, uint32_t rows_pad, PackKind kind,
                        const uint32_t *scale_max = nullptr, const int *scale_flag = nullptr,
                        int flag_bit = 0, const int *launch_flag = nullptr,
                        uint32_t flag_accept_mask = 0);

@@ -315,6 +315,33 @@ def test_packed_path_matches_in_loop_split(O, handle, dev, monkeypatch, mode, op
         assert np.array_equal(outs[0].reshape(n, ldc)[:, m:], c0.reshape(n, ldc)[:, m:])
 
 
+@pytest.mark.parametrize("opa,opb,m,n,k,pads,alpha,beta", [
+    (N, N, 2048, 2048, 256, (0, 0, 0), 1.0, 0.0),
+    (C, N, 2000, 1700, 300, (1, 3, 2), 1.5 - 0.5j, -0.5 + 0.25j),   # ragged M, N, K, conjugated A
+    (N, T, 1280, 2100, 520, (0, 5, 0), 1.0, 1.0),
+    (T, C, 1700, 1500, 129, (2, 0, 1), -1.0j, 0.25),
+])
+def test_complex_packed_path_matches_in_loop_split(O, handle, dev, monkeypatch, opa, opb, m, n, k, pads, alpha, beta):
+    gen = _gen(True)
+    a, lda = make_operand(gen, 65, opa, m, k, pads[0])
+    b, ldb = make_operand(gen, 66, opb, k, n, pads[1])
+    ldc = m + pads[2]
+    c0 = gen(67, ldc * n)
+    outs = []
+    for packed in ("1", "0"):
+        monkeypatch.setenv("CUMPSGEMM_PACKED", packed)
+        c, st, mid = run_gemm(handle, dev, FP16TCEC, opa, opb, m, n, k, alpha, a, lda, b, ldb, beta, c0, ldc, True,
+                              want_module_id=True)
+        assert st == 0 and (mid == 200) == (packed == "1")
+        outs.append(c)
+    assert np.array_equal(outs[0].view(np.uint32), outs[1].view(np.uint32))
+    ref = O.gemm_fp64(opa, opb, m, n, k, alpha, a, lda, b, ldb, beta, c0, ldc)
+    cf = oracle_gemm(O, FP32, opa, opb, m, n, k, alpha, a, lda, b, ldb, beta, c0, ldc)
+    assert O.residual(ref, outs[0], m, n, ldc) <= 2.0 * O.residual(ref, cf, m, n, ldc)
+    if pads[2]:
+        assert np.array_equal(outs[0].reshape(n, ldc)[:, m:], c0.reshape(n, ldc)[:, m:])
+
+
 # ---- column split for a partial last round --------------------------------------
 # When the tile count is just above a multiple of the CU slots, C is cut into two
 # column blocks that are planned separately.  Same numbers as the single launch up
