@@ -149,6 +149,33 @@ def test_fused_scaling_matches_in_place_scaling(O, handle, dev, monkeypatch, mod
 # scaled and split once into fp16 planes (workspace of the handle) and the GEMM
 # kernel only folds the inverse scaling of C into alpha.  Same scaling, same
 # split, same order of accumulation as the two other forms -> same bits.
+def test_complex_scaled_pre_split_path_matches_in_loop(cg, torch_gpu, dev, monkeypatch):
+    """FP16TCEC_SCALING on a large complex problem: the pre-pass scales, splits and
+    de-interleaves; same bits as the in-loop fused form."""
+    m, n, k = 3800, 3700, 288
+    C_OP = 113
+    a = (inputs.complex_normal(75, m * k, 1.0) * np.float32(2.0 ** -21)).astype(np.complex64)
+    b = (inputs.complex_normal(76, n * k, 1.0) * np.float32(2.0 ** 4)).astype(np.complex64)
+    h = cg.Handle()
+    h.set_stream(torch_gpu.cuda.current_stream())
+    try:
+        outs = []
+        for packed in ("0", None):
+            if packed is None:
+                monkeypatch.delenv("CUMPSGEMM_PACKED", raising=False)
+            else:
+                monkeypatch.setenv("CUMPSGEMM_PACKED", packed)
+            c, a_after, b_after, _ = _pipeline(h, dev, SCALING, N, C_OP, m, n, k, a, b, cplx=True)
+            assert (h.workspace_size() >= (m + n) * k * 8) == (packed is None)
+            assert np.array_equal(a_after.view(np.uint32), a.view(np.uint32))
+            outs.append(c)
+        assert np.array_equal(outs[0].view(np.uint32), outs[1].view(np.uint32))
+        assert float(np.abs(outs[0]).max()) > 0
+    finally:
+        torch_gpu.cuda.synchronize()
+        h.close()
+
+
 @pytest.mark.parametrize("opa,opb,m,n,k", [
     (N, N, 4096, 4096, 256),      # (the path is taken from m*n/(m+n) >= 1800 on)
     (T, N, 4000, 3700, 300),      # ragged M, N and K
