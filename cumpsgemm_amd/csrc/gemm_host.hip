@@ -371,8 +371,12 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
         force_split <= 1) {
       const uint32_t mp = packed_rows(m), np = packed_rows(n);
       const uint64_t a_bytes = packed_bytes(mp, k, planes), b_bytes = packed_bytes(np, k, planes);
-      if (a_bytes + b_bytes <= (16ull << 30) && mp * 64ull < 0xffffffffull && np * 64ull < 0xffffffffull) {
-        if (h->pack_ws_bytes < a_bytes + b_bytes) {
+      // AUTO: the bf16x3 candidate gets its own (gated) pre-pass and planes behind the fp16 ones
+      const bool auto_bf16 = auto_ok && k >= 512 && mn_ratio >= 2000.0 && !never;
+      const uint64_t a3_bytes = auto_bf16 ? packed_bytes(mp, k, 3) : 0, b3_bytes = auto_bf16 ? packed_bytes(np, k, 3) : 0;
+      const uint64_t ws_bytes = a_bytes + b_bytes + a3_bytes + b3_bytes;
+      if (ws_bytes <= (16ull << 30) && mp * 64ull < 0xffffffffull && np * 64ull < 0xffffffffull) {
+        if (h->pack_ws_bytes < ws_bytes) {
           // the previous workspace may still be in use by work queued on the stream
           if (hipStreamSynchronize(h->stream) != hipSuccess) {
             log_error("stream synchronisation failed before growing the pack workspace");
@@ -381,8 +385,8 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
           if (h->pack_ws != nullptr) (void)hipFree(h->pack_ws);
           h->pack_ws = nullptr;
           h->pack_ws_bytes = 0;
-          if (hipMalloc(&h->pack_ws, a_bytes + b_bytes) == hipSuccess) {
-            h->pack_ws_bytes = a_bytes + b_bytes;
+          if (hipMalloc(&h->pack_ws, ws_bytes) == hipSuccess) {
+            h->pack_ws_bytes = ws_bytes;
           } else {
             (void)hipGetLastError();
             h->pack_ws = nullptr;
@@ -444,6 +448,39 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
             return HIPBLAS_STATUS_EXECUTION_FAILED;
           }
           if (!auto_ok) return HIPBLAS_STATUS_SUCCESS;
+          if (auto_bf16) { // the other candidate, same path: three bf16 planes, its own accept mask
+            char *pa3 = pb + b_bytes, *pb3 = pa3 + a3_bytes;
+            const uint32_t accept3 = launches[0].accept;
+            launch_pack_split(h->stream, reinterpret_cast<const float *>(a), a_kc, lda, (uint32_t)m,
+                              (uint32_t)k, pa3, mp, PackKind::BF16X3_REAL, nullptr, nullptr, 0, gate, accept3);
+            launch_pack_split(h->stream, reinterpret_cast<const float *>(b), b_kc, ldb, (uint32_t)n,
+                              (uint32_t)k, pb3, np, PackKind::BF16X3_REAL, nullptr, nullptr, 0, gate, accept3);
+            GemmArgs qargs = args;
+            qargs.a = pa3;
+            qargs.b = pb3;
+            qargs.lda = mp;
+            qargs.ldb = np;
+            qargs.k = pargs.k;
+            qargs.k_chunk = pargs.k;
+            qargs.tiles_m = (uint32_t)((m + kPackedBf16BM - 1) / kPackedBf16BM);
+            qargs.tiles_n = (uint32_t)((n + kPackedBf16BN - 1) / kPackedBf16BN);
+            qargs.batch = 1;
+            qargs.atomic_out = 0;
+            qargs.launch_flag = gate;
+            qargs.flag_accept_mask = accept3;
+            const uint64_t total3 = (uint64_t)qargs.tiles_m * qargs.tiles_n;
+            const bool walk3 = qargs.k / 32 <= persistent_max_steps();
+            const dim3 grid3 = walk3 ? dim3((unsigned)std::min<uint64_t>(total3, h->num_cus), 1, 1)
+                                     : dim3((unsigned)total3, 1, 1);
+            launch_packed_bf16x3_s(qargs, grid3, h->stream, walk3);
+            const hipError_t qerr = hipGetLastError();
+            if (qerr != hipSuccess) {
+              log_error(std::string("packed GEMM launch failed: ") + hipGetErrorString(qerr));
+              return HIPBLAS_STATUS_EXECUTION_FAILED;
+            }
+            if (used_id != nullptr) *used_id = ~0u; // AUTO
+            return HIPBLAS_STATUS_SUCCESS;
+          }
           nlaunch = 1;        // the FP16TCEC candidate is served; bf16x3 remains
           fp16_served = true; // (and is not cut into column blocks: they would come back here)
         }

@@ -220,11 +220,13 @@ def test_scaled_pre_split_path_matches_the_other_forms(O, cg, torch_gpu, dev, mo
         assert O.residual(ref, outs["pre_split"], m, n, m) <= 2.0 * O.residual(ref, cf, m, n, m)
 
 
-def test_auto_pre_split_path_steps_aside_for_bf16x3(O, cg, torch_gpu, dev, monkeypatch):
+@pytest.mark.parametrize("k", [256, 512])
+def test_auto_pre_split_path_steps_aside_for_bf16x3(O, cg, torch_gpu, dev, monkeypatch, k):
     """Same shape class, but AUTO decides for TF32TCEC (no underflow tolerated):
     the gated pre-pass and the gated FP16TCEC kernel do nothing, the bf16x3
-    kernel produces C -- the same bits as with the pre-split path forbidden."""
-    m, n, k = 4096, 4096, 256
+    kernel (k = 256: the in-loop one; k = 512: its own gated pre-split form)
+    produces C -- the same bits as with the pre-split path forbidden."""
+    m, n = 4096, 4096
     a = (inputs.uniform(81, m * k) * np.float32(2.0 ** -22)).astype(np.float32)
     b = (inputs.uniform(82, k * n) * np.float32(2.0 ** 5)).astype(np.float32)
     h = cg.Handle()
