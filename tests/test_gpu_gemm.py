@@ -342,6 +342,26 @@ def test_complex_packed_path_matches_in_loop_split(O, handle, dev, monkeypatch, 
         assert np.array_equal(outs[0].reshape(n, ldc)[:, m:], c0.reshape(n, ldc)[:, m:])
 
 
+@pytest.mark.parametrize("mode,cplx", [(FP16TCEC, False), (TF32TCEC, False), (FP16TCEC, True)])
+def test_packed_kernels_walk_and_one_tile_forms_agree(handle, dev, monkeypatch, mode, cplx):
+    """The pre-split kernels exist as persistent (tile-walking) and one-tile-per-workgroup
+    forms, chosen by K; both do the same arithmetic in the same order."""
+    m, n, k = 3100, 2900, 600   # (the path needs at least one 256x128 tile per CU)
+    gen = _gen(cplx)
+    a, lda = make_operand(gen, 91, T, m, k, 3)
+    b, ldb = make_operand(gen, 92, N, k, n, 0)
+    c0 = gen(93, m * n)
+    monkeypatch.setenv("CUMPSGEMM_PACKED", "1")
+    outs = []
+    for walk in ("1", "0"):
+        monkeypatch.setenv("CUMPSGEMM_PACKED_WALK", walk)
+        c, st, mid = run_gemm(handle, dev, mode, T, N, m, n, k, 1.25, a, lda, b, ldb, 0.5, c0, m, cplx,
+                              want_module_id=True)
+        assert st == 0 and mid == 200
+        outs.append(c)
+    assert np.array_equal(outs[0].view(np.uint32), outs[1].view(np.uint32))
+
+
 # ---- column split for a partial last round --------------------------------------
 # When the tile count is just above a multiple of the CU slots, C is cut into two
 # column blocks that are planned separately.  Same numbers as the single launch up
