@@ -225,9 +225,10 @@ __device__ inline f16v_t mfma32(const u4_t a, const u4_t b, const f16v_t c) {
 //   SCALED (FP16TCEC only): op(A), op(B) are multiplied by powers of two read
 //         from device memory while they are split, and the result by the
 //         inverse product when it is written out (see GemmArgs).
-//   PACKED (three-buffer kernels, real FP16TCEC / bf16x3): A and B were split beforehand into
-//         fp16 planes laid out as the LDS image of every (tile, K-step), see
-//         pack_split_kernel; staging is a plain 16-byte copy, no arithmetic.
+//   PACKED (three-buffer kernels; FP16TCEC real and complex, real bf16x3): A
+//         and B were split beforehand into fp16 / bf16 planes laid out as the
+//         LDS image of every (tile, K-step), see pack_split_kernel; staging is
+//         a plain 16-byte copy, no arithmetic.
 template <Prec P_, bool CPLX_, bool A_KC_, bool B_KC_, int BM_, int BN_, int WM_,
           int WN_, int OCC_ = 1, bool DEEP_ = false, bool PERSIST_ = false, bool SCALED_ = false,
           bool PACKED_ = false>
