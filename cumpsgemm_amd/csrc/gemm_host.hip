@@ -234,6 +234,209 @@ template <> struct scalar_parts<hipComplex> {
   static void get(const hipComplex *s, float &re, float &im) { re = s->x; im = s->y; }
 };
 
+// ---------------------------------------------------------------------------
+// Pre-split path (FP16TCEC real and complex, bf16x3 real): split A and B once,
+// up front, into fp16 / bf16 planes held in the handle's workspace, and run the
+// kernel that only copies them into LDS.  Results are bit-identical to the
+// in-loop split (same split, same order of accumulation).  The pre-pass is one
+// read + write of A and B at 5 - 6 TB/s; what it buys is a K loop without split
+// arithmetic, which runs at a higher clock under the power limit.  It pays for
+// large problems (rules below, per mode and layout); the in-loop kernels serve
+// the rest and need no workspace.  CUMPSGEMM_PACKED=1 / 0 forces / forbids it.
+enum class PreSplit {
+  NOT_TAKEN,   // the caller launches the in-loop kernels
+  DONE,        // C is (being) computed; nothing left to launch
+  FP16_SERVED, // AUTO: the FP16TCEC candidate is launched, bf16x3 is left to the caller
+  FAILED       // a launch or the stream failed (logged)
+};
+
+struct PreSplitChoice {
+  bool take = false;
+  bool bf16 = false;      // explicit TF32TCEC: three bf16 planes
+  bool auto_ok = false;   // AUTO: the gated FP16TCEC candidate goes this way
+  bool auto_bf16 = false; // AUTO: and so does the gated bf16x3 candidate
+  int bm = 0, bn = 0;     // tile of the kernel that reads the planes
+  unsigned planes = 0;    // planes per K-step of one operand
+};
+
+template <bool CPLX>
+PreSplitChoice choose_pre_split(const cuMpSGEMM_handle *h, bool a_kc, bool b_kc, uint64_t m, uint64_t n,
+                                uint64_t k, uint64_t batch, cuMpSGEMM_compute_mode_t mode,
+                                int force_cls, int force_split, int depth) {
+  PreSplitChoice ch;
+  if (CPLX && mode != CUMPSGEMM_FP16TCEC) return ch; // (complex: FP16TCEC only, also under FP16TCEC_SCALING)
+  const char *fp = std::getenv("CUMPSGEMM_PACKED"); // "0" never, "1" whenever possible
+  const bool never = fp != nullptr && fp[0] == '0', always = fp != nullptr && fp[0] == '1';
+  // bf16x3 (explicit TF32TCEC mode): its in-loop three-way split costs 5.4
+  // vector instructions per MFMA, so the pre-pass pays for every layout
+  ch.bf16 = (mode == CUMPSGEMM_TF32TCEC);
+  ch.bm = CPLX ? kPackedCplxBM : (ch.bf16 ? kPackedBf16BM : kPackedBM);
+  ch.bn = CPLX ? kPackedCplxBN : (ch.bf16 ? kPackedBf16BN : kPackedBN);
+  ch.planes = CPLX ? 4u : (ch.bf16 ? 3u : 2u);
+  // (the pre-pass launches workgroups of 64 rows x 32 .. 256 K-values on a 2-D grid)
+  const bool shape_ok = batch == 1 && k >= 128 &&
+                        (uint64_t)m * n >= (uint64_t)h->num_cus * ch.bm * ch.bn && k / 32 < 65535;
+  const double mn_ratio = (double)m * (double)n / ((double)m + (double)n);
+  const bool pays_nt = !a_kc && !b_kc && k >= 256 && mn_ratio >= 1800.0;
+  // Every other layout: the pre-split kernel, freed of the split arithmetic,
+  // outruns the in-loop one by more than the pre-pass costs once the problem
+  // is large (8192^3: 381 vs 361 - 372 TFLOP/s; 8192^2 x 1024: 351 vs 318 -
+  // 343) -- provided the last round of CU slots is at least half full or one
+  // of many: the path has no column split for a mostly empty last round.
+  const uint64_t ptiles = ((m + ch.bm - 1) / ch.bm) * ((n + ch.bn - 1) / ch.bn);
+  const uint64_t last_round = ptiles % h->num_cus;
+  const bool rounds_ok = last_round == 0 || 2 * last_round >= h->num_cus || ptiles >= 6ull * h->num_cus;
+  // (complex: four times the MFMA work per element split, so the pre-pass weighs less)
+  const bool pays = pays_nt || (k >= 1024 && mn_ratio >= (CPLX ? 1500.0 : 3000.0) && rounds_ok);
+  // With fused scaling the in-loop split costs one more instruction per pair
+  // and those kernels run 8 - 25 % below the plain ones, so the pre-pass (which
+  // scales as it splits) pays for every layout.
+  const bool pays_scaled = h->fused_scaling && k >= 256 && mn_ratio >= 1800.0;
+  // AUTO: the FP16TCEC candidate may take the path as well, gated by the
+  // launch flag like every AUTO kernel (pre-pass included).  Both candidates
+  // write C directly, which needs the bf16x3 plan to be free of split-K.
+  if (!CPLX && mode == CUMPSGEMM_AUTO && pays_scaled && depth == 0) {
+    ch.auto_ok = make_plan(h, Prec::BF16X3, CPLX, a_kc, b_kc, m, n, k, batch, force_cls, force_split).ksplit == 1;
+  }
+  // (measured: - 4 % at 3072^3, + 5 % at 4096^3, + 8 % at 6144^3, + 10 % from 8192^2 on)
+  const bool pays_bf16 = k >= 512 && mn_ratio >= 2000.0;
+  const bool mode_ok = mode == CUMPSGEMM_FP16TCEC || ch.bf16 || ch.auto_ok;
+  const bool worth = ch.bf16 ? (pays_bf16 || always) : (pays || pays_scaled || always);
+  ch.take = mode_ok && !never && shape_ok && worth && force_cls <= 0 && force_split <= 1;
+  // AUTO: the bf16x3 candidate gets its own (gated) pre-pass and planes behind the fp16 ones
+  ch.auto_bf16 = ch.take && ch.auto_ok && pays_bf16;
+  return ch;
+}
+
+// The handle's workspace only grows.  false: no memory (the caller falls back
+// to the in-loop kernels) or, with *failed set, the stream is broken.
+bool ensure_pack_workspace(cuMpSGEMM_handle *h, uint64_t bytes, bool *failed) {
+  *failed = false;
+  if (h->pack_ws_bytes >= bytes) return h->pack_ws != nullptr;
+  // the previous workspace may still be in use by work queued on the stream
+  if (hipStreamSynchronize(h->stream) != hipSuccess) {
+    log_error("stream synchronisation failed before growing the pack workspace");
+    *failed = true;
+    return false;
+  }
+  if (h->pack_ws != nullptr) (void)hipFree(h->pack_ws);
+  h->pack_ws = nullptr;
+  h->pack_ws_bytes = 0;
+  if (hipMalloc(&h->pack_ws, bytes) != hipSuccess) {
+    (void)hipGetLastError();
+    h->pack_ws = nullptr;
+    return false;
+  }
+  h->pack_ws_bytes = bytes;
+  return true;
+}
+
+// `args`: the call's arguments (scalars, C, conj flags, launch flag); `accept_*`:
+// the launch-flag masks of the two AUTO candidates.
+template <class T>
+PreSplit run_pre_split(cuMpSGEMM_handle *h, const GemmArgs &args, bool a_kc, bool b_kc, uint64_t m,
+                       uint64_t n, uint64_t k, const T *a, uint64_t lda, const T *b, uint64_t ldb,
+                       uint64_t batch, cuMpSGEMM_compute_mode_t mode, uint32_t accept_bf16,
+                       uint32_t accept_fp16, int force_cls, int force_split, int depth,
+                       unsigned *used_id) {
+  constexpr bool CPLX = std::is_same<T, hipComplex>::value;
+  const PreSplitChoice ch = choose_pre_split<CPLX>(h, a_kc, b_kc, m, n, k, batch, mode, force_cls, force_split, depth);
+  if (!ch.take) return PreSplit::NOT_TAKEN;
+  const uint32_t mp = packed_rows(m), np = packed_rows(n);
+  const uint64_t a_bytes = packed_bytes(mp, k, ch.planes), b_bytes = packed_bytes(np, k, ch.planes);
+  const uint64_t a3_bytes = ch.auto_bf16 ? packed_bytes(mp, k, 3) : 0;
+  const uint64_t b3_bytes = ch.auto_bf16 ? packed_bytes(np, k, 3) : 0;
+  const uint64_t ws_bytes = a_bytes + b_bytes + a3_bytes + b3_bytes;
+  if (ws_bytes > (16ull << 30) || mp * 64ull >= 0xffffffffull || np * 64ull >= 0xffffffffull)
+    return PreSplit::NOT_TAKEN;
+  bool failed = false;
+  if (!ensure_pack_workspace(h, ws_bytes, &failed)) return failed ? PreSplit::FAILED : PreSplit::NOT_TAKEN;
+
+  const float *af = reinterpret_cast<const float *>(a), *bf = reinterpret_cast<const float *>(b);
+  const int *gate = ch.auto_ok ? args.launch_flag : nullptr;
+  // one candidate: pre-pass of both operands, then the kernel over their planes
+  auto run = [&](PackKind kind, char *pa, char *pb, int bm, int bn, uint32_t accept, bool scaled,
+                 auto launch_kernel, bool walk_short_only) -> bool {
+    GemmArgs pargs = args;
+    const uint32_t *max_a = nullptr, *max_b = nullptr;
+    const int *sflag = nullptr;
+    if (scaled) {
+      max_a = &h->stats_slots[h->fused_slot_a].max_exp_bits;
+      max_b = &h->stats_slots[h->fused_slot_b].max_exp_bits;
+      sflag = h->flag_buffer + h->fused_flag;
+      pargs.scale_max_a = max_a; // the kernel derives the inverse scaling of C from them
+      pargs.scale_max_b = max_b;
+      pargs.scale_flag = sflag;
+    }
+    launch_pack_split(h->stream, af, a_kc, lda, (uint32_t)m, (uint32_t)k, pa, mp, kind, max_a, sflag, 0x40,
+                      gate, accept);
+    launch_pack_split(h->stream, bf, b_kc, ldb, (uint32_t)n, (uint32_t)k, pb, np, kind, max_b, sflag, 0x20,
+                      gate, accept);
+    pargs.a = pa;
+    pargs.b = pb;
+    pargs.lda = mp; // padded row counts of the packed operands
+    pargs.ldb = np;
+    pargs.k = (uint32_t)((k + 31) / 32 * 32); // zero-padded to whole K-steps
+    pargs.k_chunk = pargs.k;
+    pargs.tiles_m = (uint32_t)((m + bm - 1) / bm);
+    pargs.tiles_n = (uint32_t)((n + bn - 1) / bn);
+    pargs.batch = 1;
+    pargs.atomic_out = 0;
+    pargs.launch_flag = gate;
+    pargs.flag_accept_mask = accept;
+    const uint64_t total = (uint64_t)pargs.tiles_m * pargs.tiles_n;
+    // short tiles are walked by persistent workgroups, long ones get a workgroup each
+    // (measured cross-over: 16 K-steps for the fp16 kernel, which gains 6 - 8 % from
+    // the one-tile form at 8192^3, the usual 32 for bf16x3, which gains nothing)
+    bool walk = walk_short_only ? pargs.k / 32 < 16 : pargs.k / 32 <= persistent_max_steps();
+    if (const char *w = std::getenv("CUMPSGEMM_PACKED_WALK")) walk = w[0] == '1';
+    const dim3 grid = walk ? dim3((unsigned)std::min<uint64_t>(total, h->num_cus), 1, 1)
+                           : dim3((unsigned)total, 1, 1);
+    launch_kernel(pargs, grid, walk);
+    const hipError_t err = hipGetLastError();
+    if (err != hipSuccess) {
+      log_error(std::string("packed GEMM launch failed: ") + hipGetErrorString(err));
+      return false;
+    }
+    return true;
+  };
+
+  char *pa = static_cast<char *>(h->pack_ws), *pb = pa + a_bytes;
+  const uint32_t accept = ch.auto_ok ? accept_fp16 : 0u;
+  bool ok;
+  if constexpr (CPLX) {
+    ok = run(PackKind::FP16_COMPLEX, pa, pb, ch.bm, ch.bn, accept, h->fused_scaling,
+             [&](const GemmArgs &g, dim3 grid, bool walk) {
+               launch_packed_fp16tcec_c(g, grid, h->stream, walk, h->fused_scaling);
+             }, false);
+  } else if (ch.bf16) {
+    ok = run(PackKind::BF16X3_REAL, pa, pb, ch.bm, ch.bn, accept, false,
+             [&](const GemmArgs &g, dim3 grid, bool walk) { launch_packed_bf16x3_s(g, grid, h->stream, walk); },
+             false);
+  } else {
+    ok = run(PackKind::FP16_REAL, pa, pb, ch.bm, ch.bn, accept, h->fused_scaling,
+             [&](const GemmArgs &g, dim3 grid, bool walk) {
+               if (h->fused_scaling) launch_packed_scaled_fp16tcec_s(g, grid, h->stream, walk);
+               else launch_packed_fp16tcec_s(g, grid, h->stream, walk);
+             }, true);
+  }
+  if (!ok) return PreSplit::FAILED;
+  if (used_id != nullptr) *used_id = 200u; // pre-split path
+  if (!ch.auto_ok) return PreSplit::DONE;
+  if (!ch.auto_bf16) return PreSplit::FP16_SERVED;
+  // AUTO, the other candidate by the same path: three bf16 planes, its own accept mask
+  if constexpr (!CPLX) {
+    char *pa3 = pb + b_bytes, *pb3 = pa3 + a3_bytes;
+    ok = run(PackKind::BF16X3_REAL, pa3, pb3, kPackedBf16BM, kPackedBf16BN, accept_bf16, false,
+             [&](const GemmArgs &g, dim3 grid, bool walk) { launch_packed_bf16x3_s(g, grid, h->stream, walk); },
+             false);
+    if (!ok) return PreSplit::FAILED;
+  }
+  if (used_id != nullptr) *used_id = ~0u; // AUTO
+  return PreSplit::DONE;
+}
+
+
 template <class T>
 hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
                          hipblasOperation_t op_B, uint64_t m, uint64_t n, uint64_t k,
@@ -319,172 +522,22 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
     return HIPBLAS_STATUS_SUCCESS;
   }
 
-  // Pre-split path (real FP16TCEC and bf16x3): split A and B once, up front, into
-  // fp16 / bf16 planes held in the handle's workspace, and run the kernel that
-  // only copies them into LDS.  Results are bit-identical to the in-loop split
-  // (same split, same order of accumulation).  The pre-pass is one read + write
-  // of A and B at 5 - 6 TB/s; what it buys is a K loop without split arithmetic,
-  // which runs at a higher clock under the power limit.  It pays for large
-  // problems (rules below, per mode and layout); the in-loop kernels serve the
-  // rest and need no workspace.  CUMPSGEMM_PACKED=1 / 0 forces / forbids the path.
+  // large problems: operands split once, up front (see run_pre_split)
   bool fp16_served = false;
-  if (!CPLX || mode == CUMPSGEMM_FP16TCEC) { // (complex: FP16TCEC only, also under FP16TCEC_SCALING)
-    const char *fp = std::getenv("CUMPSGEMM_PACKED"); // "0" never, "1" whenever possible
-    const bool never = fp != nullptr && fp[0] == '0', always = fp != nullptr && fp[0] == '1';
-    // bf16x3 (explicit TF32TCEC mode): its in-loop three-way split costs 5.4
-    // vector instructions per MFMA, so the pre-pass pays for every layout
-    const bool bf16 = (mode == CUMPSGEMM_TF32TCEC);
-    const int pbm = CPLX ? kPackedCplxBM : (bf16 ? kPackedBf16BM : kPackedBM);
-    const int pbn = CPLX ? kPackedCplxBN : (bf16 ? kPackedBf16BN : kPackedBN);
-    const unsigned planes = CPLX ? 4u : (bf16 ? 3u : 2u);
-    // (the pre-pass launches workgroups of 64 rows x 32 .. 256 K-values on a 2-D grid)
-    const bool shape_ok = batch == 1 && k >= 128 && (uint64_t)m * n >= (uint64_t)h->num_cus * pbm * pbn &&
-                          k / 32 < 65535;
-    const double mn_ratio = (double)m * (double)n / ((double)m + (double)n);
-    const bool pays_nt = !a_kc && !b_kc && k >= 256 && mn_ratio >= 1800.0;
-    // Every other layout: the pre-split kernel, freed of the split arithmetic,
-    // outruns the in-loop one by more than the pre-pass costs once the problem
-    // is large (8192^3: 381 vs 361 - 372 TFLOP/s; 8192^2 x 1024: 351 vs 318 -
-    // 343) -- provided the last round of CU slots is at least half full or one
-    // of many: the path has no column split for a mostly empty last round.
-    const uint64_t ptiles = ((m + pbm - 1) / pbm) * ((n + pbn - 1) / pbn);
-    const uint64_t last_round = ptiles % h->num_cus;
-    const bool rounds_ok = last_round == 0 || 2 * last_round >= h->num_cus || ptiles >= 6ull * h->num_cus;
-    // (complex: four times the MFMA work per element split, so the pre-pass weighs less)
-    const bool pays = pays_nt || (k >= 1024 && mn_ratio >= (CPLX ? 1500.0 : 3000.0) && rounds_ok);
-    // With fused scaling the in-loop split costs one more instruction per pair
-    // and those kernels run 8 - 25 % below the plain ones, so the pre-pass (which
-    // scales as it splits) pays for every layout.
-    const bool pays_scaled = h->fused_scaling && k >= 256 && mn_ratio >= 1800.0;
-    // AUTO: the FP16TCEC candidate may take the path as well, gated by the
-    // launch flag like every AUTO kernel (pre-pass included); the bf16x3
-    // candidate then goes through the ordinary launch below, alone.  Both
-    // write C directly, which needs the bf16x3 plan to be free of split-K.
-    bool auto_ok = false;
-    if (!CPLX && mode == CUMPSGEMM_AUTO && pays_scaled && depth == 0) {
-      auto_ok = make_plan(h, launches[0].p, CPLX, a_kc, b_kc, m, n, k, batch, force_cls, force_split).ksplit == 1;
-    }
-    // (measured: - 4 % at 3072^3, + 5 % at 4096^3, + 8 % at 6144^3, + 10 % from 8192^2 on)
-    const bool pays_bf16 = bf16 && k >= 512 && mn_ratio >= 2000.0;
-    if ((mode == CUMPSGEMM_FP16TCEC || bf16 || auto_ok) && !never && shape_ok &&
-        (bf16 ? (pays_bf16 || always) : (pays || pays_scaled || always)) && force_cls <= 0 &&
-        force_split <= 1) {
-      const uint32_t mp = packed_rows(m), np = packed_rows(n);
-      const uint64_t a_bytes = packed_bytes(mp, k, planes), b_bytes = packed_bytes(np, k, planes);
-      // AUTO: the bf16x3 candidate gets its own (gated) pre-pass and planes behind the fp16 ones
-      const bool auto_bf16 = auto_ok && k >= 512 && mn_ratio >= 2000.0 && !never;
-      const uint64_t a3_bytes = auto_bf16 ? packed_bytes(mp, k, 3) : 0, b3_bytes = auto_bf16 ? packed_bytes(np, k, 3) : 0;
-      const uint64_t ws_bytes = a_bytes + b_bytes + a3_bytes + b3_bytes;
-      if (ws_bytes <= (16ull << 30) && mp * 64ull < 0xffffffffull && np * 64ull < 0xffffffffull) {
-        if (h->pack_ws_bytes < ws_bytes) {
-          // the previous workspace may still be in use by work queued on the stream
-          if (hipStreamSynchronize(h->stream) != hipSuccess) {
-            log_error("stream synchronisation failed before growing the pack workspace");
-            return HIPBLAS_STATUS_EXECUTION_FAILED;
-          }
-          if (h->pack_ws != nullptr) (void)hipFree(h->pack_ws);
-          h->pack_ws = nullptr;
-          h->pack_ws_bytes = 0;
-          if (hipMalloc(&h->pack_ws, ws_bytes) == hipSuccess) {
-            h->pack_ws_bytes = ws_bytes;
-          } else {
-            (void)hipGetLastError();
-            h->pack_ws = nullptr;
-          }
-        }
-        if (h->pack_ws != nullptr) {
-          char *pa = static_cast<char *>(h->pack_ws), *pb = pa + a_bytes;
-          GemmArgs pargs = args;
-          const uint32_t *max_a = nullptr, *max_b = nullptr;
-          const int *sflag = nullptr;
-          if (h->fused_scaling && !bf16) {
-            max_a = &h->stats_slots[h->fused_slot_a].max_exp_bits;
-            max_b = &h->stats_slots[h->fused_slot_b].max_exp_bits;
-            sflag = h->flag_buffer + h->fused_flag;
-            pargs.scale_max_a = max_a; // the kernel derives the inverse scaling of C from them
-            pargs.scale_max_b = max_b;
-            pargs.scale_flag = sflag;
-          }
-          const PackKind kind = CPLX ? PackKind::FP16_COMPLEX : (bf16 ? PackKind::BF16X3_REAL : PackKind::FP16_REAL);
-          const int *gate = auto_ok ? args.launch_flag : nullptr;
-          const uint32_t accept = auto_ok ? launches[1].accept : 0u;
-          launch_pack_split(h->stream, reinterpret_cast<const float *>(a), a_kc, lda, (uint32_t)m,
-                            (uint32_t)k, pa, mp, kind, max_a, sflag, 0x40, gate, accept);
-          launch_pack_split(h->stream, reinterpret_cast<const float *>(b), b_kc, ldb, (uint32_t)n,
-                            (uint32_t)k, pb, np, kind, max_b, sflag, 0x20, gate, accept);
-          pargs.a = pa;
-          pargs.b = pb;
-          pargs.lda = mp; // padded row counts of the packed operands
-          pargs.ldb = np;
-          pargs.k = (uint32_t)((k + 31) / 32 * 32); // zero-padded to whole K-steps
-          pargs.k_chunk = pargs.k;
-          pargs.tiles_m = (uint32_t)((m + pbm - 1) / pbm);
-          pargs.tiles_n = (uint32_t)((n + pbn - 1) / pbn);
-          pargs.batch = 1;
-          pargs.atomic_out = 0;
-          pargs.launch_flag = gate;
-          pargs.flag_accept_mask = accept;
-          const uint64_t total = (uint64_t)pargs.tiles_m * pargs.tiles_n;
-          // short tiles are walked by persistent workgroups, long ones get a workgroup each
-          // (measured cross-over: 16 K-steps for the fp16 kernel, which gains 6 - 8 % from
-          // the one-tile form at 8192^3, the usual 32 for bf16x3, which gains nothing)
-          bool walk = (bf16 || CPLX) ? pargs.k / 32 <= persistent_max_steps() : pargs.k / 32 < 16;
-          if (const char *w = std::getenv("CUMPSGEMM_PACKED_WALK")) walk = w[0] == '1';
-          const dim3 grid = walk ? dim3((unsigned)std::min<uint64_t>(total, h->num_cus), 1, 1)
-                                 : dim3((unsigned)total, 1, 1);
-          if constexpr (CPLX) {
-            launch_packed_fp16tcec_c(pargs, grid, h->stream, walk, h->fused_scaling);
-          } else if (bf16) {
-            launch_packed_bf16x3_s(pargs, grid, h->stream, walk);
-          } else if (h->fused_scaling) {
-            launch_packed_scaled_fp16tcec_s(pargs, grid, h->stream, walk);
-          } else {
-            launch_packed_fp16tcec_s(pargs, grid, h->stream, walk);
-          }
-          if (used_id != nullptr) *used_id = 200u; // pre-split path
-          const hipError_t perr = hipGetLastError();
-          if (perr != hipSuccess) {
-            log_error(std::string("packed GEMM launch failed: ") + hipGetErrorString(perr));
-            return HIPBLAS_STATUS_EXECUTION_FAILED;
-          }
-          if (!auto_ok) return HIPBLAS_STATUS_SUCCESS;
-          if (auto_bf16) { // the other candidate, same path: three bf16 planes, its own accept mask
-            char *pa3 = pb + b_bytes, *pb3 = pa3 + a3_bytes;
-            const uint32_t accept3 = launches[0].accept;
-            launch_pack_split(h->stream, reinterpret_cast<const float *>(a), a_kc, lda, (uint32_t)m,
-                              (uint32_t)k, pa3, mp, PackKind::BF16X3_REAL, nullptr, nullptr, 0, gate, accept3);
-            launch_pack_split(h->stream, reinterpret_cast<const float *>(b), b_kc, ldb, (uint32_t)n,
-                              (uint32_t)k, pb3, np, PackKind::BF16X3_REAL, nullptr, nullptr, 0, gate, accept3);
-            GemmArgs qargs = args;
-            qargs.a = pa3;
-            qargs.b = pb3;
-            qargs.lda = mp;
-            qargs.ldb = np;
-            qargs.k = pargs.k;
-            qargs.k_chunk = pargs.k;
-            qargs.tiles_m = (uint32_t)((m + kPackedBf16BM - 1) / kPackedBf16BM);
-            qargs.tiles_n = (uint32_t)((n + kPackedBf16BN - 1) / kPackedBf16BN);
-            qargs.batch = 1;
-            qargs.atomic_out = 0;
-            qargs.launch_flag = gate;
-            qargs.flag_accept_mask = accept3;
-            const uint64_t total3 = (uint64_t)qargs.tiles_m * qargs.tiles_n;
-            const bool walk3 = qargs.k / 32 <= persistent_max_steps();
-            const dim3 grid3 = walk3 ? dim3((unsigned)std::min<uint64_t>(total3, h->num_cus), 1, 1)
-                                     : dim3((unsigned)total3, 1, 1);
-            launch_packed_bf16x3_s(qargs, grid3, h->stream, walk3);
-            const hipError_t qerr = hipGetLastError();
-            if (qerr != hipSuccess) {
-              log_error(std::string("packed GEMM launch failed: ") + hipGetErrorString(qerr));
-              return HIPBLAS_STATUS_EXECUTION_FAILED;
-            }
-            if (used_id != nullptr) *used_id = ~0u; // AUTO
-            return HIPBLAS_STATUS_SUCCESS;
-          }
-          nlaunch = 1;        // the FP16TCEC candidate is served; bf16x3 remains
-          fp16_served = true; // (and is not cut into column blocks: they would come back here)
-        }
-      }
+  if (nlaunch > 0) {
+    const uint32_t accept_bf16 = launches[0].accept, accept_fp16 = nlaunch > 1 ? launches[1].accept : 0u;
+    switch (run_pre_split<T>(h, args, a_kc, b_kc, m, n, k, a, lda, b, ldb, batch, mode, accept_bf16,
+                             accept_fp16, force_cls, force_split, depth, used_id)) {
+    case PreSplit::DONE:
+      return HIPBLAS_STATUS_SUCCESS;
+    case PreSplit::FAILED:
+      return HIPBLAS_STATUS_EXECUTION_FAILED;
+    case PreSplit::FP16_SERVED:
+      nlaunch = 1;        // the FP16TCEC candidate is served; bf16x3 remains
+      fp16_served = true; // (and is not cut into column blocks: they would come back here)
+      break;
+    case PreSplit::NOT_TAKEN:
+      break;
     }
   }
 
