@@ -515,10 +515,8 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
   const bool beta_zero = args.beta_re == 0.0f && args.beta_im == 0.0f;
 
   if (k == 0) { // C = beta * C
-    const unsigned blocks = (unsigned)std::min<uint64_t>((m * n + 255) / 256, 65535);
-    hipLaunchKernelGGL(prescale_c_kernel<CPLX>, dim3(blocks, (unsigned)batch), dim3(256), 0,
-                       h->stream, reinterpret_cast<float *>(c), args.m, args.n, ldc, stridec,
-                       args.beta_re, args.beta_im);
+    launch_prescale_c<CPLX>(h->stream, c, args.m, args.n, ldc, stridec, (uint32_t)batch, args.beta_re,
+                            args.beta_im);
     return HIPBLAS_STATUS_SUCCESS;
   }
 
@@ -574,10 +572,8 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
   }
 
   if (split) {
-    const unsigned blocks = (unsigned)std::min<uint64_t>((m * n + 255) / 256, 65535);
-    hipLaunchKernelGGL(prescale_c_kernel<CPLX>, dim3(blocks, (unsigned)batch), dim3(256), 0,
-                       h->stream, reinterpret_cast<float *>(c), args.m, args.n, ldc, stridec,
-                       args.beta_re, args.beta_im);
+    launch_prescale_c<CPLX>(h->stream, c, args.m, args.n, ldc, stridec, (uint32_t)batch, args.beta_re,
+                            args.beta_im);
   }
   (void)beta_zero;
 

@@ -13,6 +13,7 @@
 // (src/cumpsgemm_kernel.cuh:58-585, src/dmem_accessor.hpp) and of the external
 // mtk::wmma::tcec fragment arithmetic (src/device_tcec_wrapper.hpp:64-106).
 #pragma once
+#include <algorithm>
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <type_traits>
@@ -1096,28 +1097,74 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
   }
 }
 
-// C (m x n, ldc, batched) *= beta before a split-K accumulation, or = 0.
+// C (m x n, ldc, batched) *= beta before a split-K accumulation, or = 0
+// (beta == 0 stores zeros whatever C held, NaN included).
+// Block = 64 lanes along a column x 4 columns; grid = (row chunks, column
+// groups, batch).  `vec`: every column starts on a 16-byte boundary, so lanes
+// move 16 bytes each.
 template <bool CPLX>
-__global__ void prescale_c_kernel(float *c, uint32_t m, uint32_t n, uint64_t ldc,
-                                  uint64_t stride_c, float beta_re, float beta_im) {
-  const uint64_t total = (uint64_t)m * n;
-  float *cb = c + (uint64_t)blockIdx.y * stride_c * (CPLX ? 2 : 1);
-  for (uint64_t id = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; id < total;
-       id += (uint64_t)gridDim.x * blockDim.x) {
-    const uint64_t i = id % m, j = id / m;
+__global__ __launch_bounds__(256) void prescale_c_kernel(float *c, uint32_t m, uint32_t n, uint64_t ldc,
+                                                         uint64_t stride_c, float beta_re, float beta_im,
+                                                         uint32_t vec) {
+  constexpr uint32_t ES = CPLX ? 2 : 1;
+  const uint64_t mf = (uint64_t)m * ES; // floats per column
+  float *cb = c + (uint64_t)blockIdx.z * stride_c * ES;
+  const bool zero = beta_re == 0.0f && (!CPLX || beta_im == 0.0f);
+  const uint32_t tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  // one element (a float, or a complex pair of floats)
+  auto scale_one = [&](float *p) {
     if constexpr (!CPLX) {
-      float *p = cb + j * ldc + i;
-      *p = (beta_re == 0.0f) ? 0.0f : beta_re * (*p);
+      *p = zero ? 0.0f : beta_re * (*p);
     } else {
-      float2 *p = reinterpret_cast<float2 *>(cb) + j * ldc + i;
-      if (beta_re == 0.0f && beta_im == 0.0f) {
-        *p = make_float2(0.f, 0.f);
+      float2 *q = reinterpret_cast<float2 *>(p);
+      if (zero) {
+        *q = make_float2(0.f, 0.f);
       } else {
-        const float2 o = *p;
-        *p = make_float2(beta_re * o.x - beta_im * o.y, beta_im * o.x + beta_re * o.y);
+        const float2 o = *q;
+        *q = make_float2(beta_re * o.x - beta_im * o.y, beta_im * o.x + beta_re * o.y);
       }
     }
+  };
+  for (uint64_t j = (uint64_t)blockIdx.y * 4 + ty; j < n; j += (uint64_t)gridDim.y * 4) {
+    float *col = cb + j * ldc * ES;
+    if (vec) {
+      for (uint64_t i = ((uint64_t)blockIdx.x * 64 + tx) * 4; i < mf; i += (uint64_t)gridDim.x * 256) {
+        if (i + 4 <= mf) {
+          float4 *q = reinterpret_cast<float4 *>(col + i);
+          if (zero) {
+            *q = make_float4(0.f, 0.f, 0.f, 0.f);
+          } else {
+            const float4 o = *q;
+            if constexpr (!CPLX) {
+              *q = make_float4(beta_re * o.x, beta_re * o.y, beta_re * o.z, beta_re * o.w);
+            } else {
+              *q = make_float4(beta_re * o.x - beta_im * o.y, beta_im * o.x + beta_re * o.y,
+                               beta_re * o.z - beta_im * o.w, beta_im * o.z + beta_re * o.w);
+            }
+          }
+        } else {
+          for (uint64_t t = i; t < mf; t += ES) scale_one(col + t);
+        }
+      }
+    } else {
+      for (uint64_t i = ((uint64_t)blockIdx.x * 64 + tx) * ES; i < mf; i += (uint64_t)gridDim.x * 64 * ES)
+        scale_one(col + i);
+    }
   }
+}
+
+template <bool CPLX>
+inline void launch_prescale_c(hipStream_t stream, void *c, uint32_t m, uint32_t n, uint64_t ldc,
+                              uint64_t stride_c, uint32_t batch, float beta_re, float beta_im) {
+  constexpr uint64_t ES = CPLX ? 2 : 1;
+  const bool vec = (reinterpret_cast<uintptr_t>(c) % 16 == 0) && (ldc * ES % 4 == 0) &&
+                   (batch == 1 || stride_c * ES % 4 == 0);
+  const uint64_t per_pass = vec ? 256 : 64; // floats (complex: elements) of a column per block and pass
+  const uint64_t chunks = ((uint64_t)m * (vec ? ES : 1) + per_pass - 1) / per_pass;
+  const dim3 grid((unsigned)std::min<uint64_t>(chunks, 64), (unsigned)std::min<uint64_t>(((uint64_t)n + 3) / 4, 65535),
+                  batch);
+  hipLaunchKernelGGL(prescale_c_kernel<CPLX>, grid, dim3(256), 0, stream, static_cast<float *>(c), m, n, ldc,
+                     stride_c, beta_re, beta_im, vec ? 1u : 0u);
 }
 
 } // namespace cumpsgemm_amd

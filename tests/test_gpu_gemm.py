@@ -412,6 +412,45 @@ def test_k_zero_scales_c(O, handle, dev, cplx):
     assert np.array_equal(c.reshape(n, m + 2)[:, m:], c0.reshape(n, m + 2)[:, m:])
 
 
+@pytest.mark.parametrize("cplx", [False, True])
+@pytest.mark.parametrize("m,n,ldc,batch,stride_pad,offset", [
+    (1030, 77, 1032, 1, 0, 0),   # 16-byte aligned columns, a tail of 2 floats per column
+    (1027, 5, 1027, 1, 0, 0),    # odd ldc: element-wise path
+    (513, 9, 516, 3, 8, 0),      # batches, aligned
+    (513, 9, 516, 3, 3, 0),      # batch stride breaks the alignment
+    (300, 300, 304, 1, 0, 1),    # base pointer off by one element
+    (3, 70000, 4, 1, 0, 0),      # more column groups than a grid dimension holds
+])
+@pytest.mark.parametrize("beta", [0.0, -0.75])
+def test_k_zero_prepares_c_exactly(handle, dev, torch_gpu, cplx, m, n, ldc, batch, stride_pad, offset, beta):
+    """k = 0 is C = beta * C (the same kernel prepares C for split-K): exact products, padding and
+    gaps between batches untouched, beta = 0 overwrites NaN."""
+    torch = torch_gpu
+    es = 2 if cplx else 1
+    stride = ldc * n + stride_pad
+    total = (offset + stride * batch) * es
+    g = torch.Generator(device=dev.dev).manual_seed(77)
+    c0 = torch.rand(total, generator=g, device=dev.dev) - 0.5
+    if beta == 0.0:
+        c0[offset * es] = float("nan")
+    c = c0.clone()
+    x = torch.zeros(64, device=dev.dev)
+    ptr = c.data_ptr() + offset * es * 4
+    if batch == 1:
+        st = handle.gemm(N, N, m, n, 0, 1.0, x, m, x, 1, beta, ptr, ldc, FP16TCEC, cplx=cplx)
+    else:
+        st = handle.gemm_strided_batch(N, N, m, n, 0, 1.0, x, m, 0, x, 1, 0, beta, ptr, ldc, stride, batch,
+                                       FP16TCEC, cplx=cplx)
+    assert st == 0
+    torch.cuda.synchronize()
+    want = c0.clone()
+    for bi in range(batch):
+        first = (offset + bi * stride) * es
+        body = want[first:first + ldc * n * es].view(n, ldc * es)
+        body[:, :m * es] = 0.0 if beta == 0.0 else body[:, :m * es] * beta   # a real beta: exact products
+    assert torch.equal(c.view(torch.int32), want.view(torch.int32))
+
+
 @pytest.mark.parametrize("mode", [FP16TCEC, TF32TCEC])
 @pytest.mark.parametrize("opa,opb,m,n,k", [
     (N, N, 1, 4096, 4096),      # row vector times matrix
