@@ -234,7 +234,7 @@ def main():
             "traffic": GEMM_TRAFFIC_BYTES if n == 8192 else None,
             # one call = two pre-split passes (about 0.2 ms) + the GEMM kernel: all inside
             "kernel_ms": round(ev_ms, 4),
-            "kernels_per_step": "2 x pack_split_kernel + gemm_tcec_kernel (packed)" if module_id == 200 else
+            "kernels_per_step": "pack_split_pair_kernel + gemm_tcec_kernel (packed)" if module_id == 200 else
                                 "gemm_tcec_kernel",
             # the split-and-correct algorithm issues 3 MFMA products per logical product
             "mfma_products_per_flop": 3,

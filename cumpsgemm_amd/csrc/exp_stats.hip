@@ -43,14 +43,40 @@ __device__ inline void count_one(Acc &a, float x, float ignore_thr, float under_
 // MODE 1: stage 2 (counts only, thresholds relative to the slot's max exponent;
 //                  runs only if the slot is UNDEFINED)
 // MODE 2: max exponent only
+// One matrix to scan: result slot, scratch for the per-workgroup partials,
+// arrival counter, the view of the data and how many workgroups work on it.
+struct StatsJob {
+  StatsSlot *slot;
+  StatsPartial *partials;
+  unsigned *ticket;
+  const float *ptr;
+  unsigned long long count_f; // flat path: number of floats; 0 = strided path
+  unsigned m_f, n;
+  unsigned long long ld_f;
+  unsigned nbatch;
+  unsigned long long stride_f;
+  unsigned blocks;
+};
+
+// A launch scans one matrix or two (A and B of a GEMM: one launch instead of
+// two saves a kernel boundary, which costs about as much as scanning 30 MB):
+// workgroups [0, job0.blocks) take job0, the rest job1, each job with its own
+// partials and arrival counter.
 template <int MODE>
-__global__ __launch_bounds__(kBlock) void exp_stats_kernel(
-    StatsSlot *slot, StatsPartial *partials, unsigned *ticket, const float *ptr,
-    unsigned long long count_f, // flat path: number of floats; 0 = strided path
-    unsigned m_f, unsigned n, unsigned long long ld_f, unsigned nbatch,
-    unsigned long long stride_f, float ignore_thr, float under_thr, float tolerance) {
+__global__ __launch_bounds__(kBlock) void exp_stats_kernel(const StatsJob job0, const StatsJob job1,
+                                                           float ignore_thr, float under_thr,
+                                                           float tolerance) {
+  const bool second = blockIdx.x >= job0.blocks; // uniform
+  const StatsJob &job = second ? job1 : job0;
+  StatsSlot *const slot = job.slot;
+  StatsPartial *const partials = job.partials;
+  unsigned *const ticket = job.ticket;
+  const float *const ptr = job.ptr;
+  const unsigned long long count_f = job.count_f, ld_f = job.ld_f, stride_f = job.stride_f;
+  const unsigned m_f = job.m_f, n = job.n, nbatch = job.nbatch;
+  const unsigned nblocks = job.blocks, bid = blockIdx.x - (second ? job0.blocks : 0u);
   if (MODE == 1) {
-    if (slot->mode != CUMPSGEMM_UNDEFINED) return; // uniform across the grid
+    if (slot->mode != CUMPSGEMM_UNDEFINED) return; // uniform across the job's workgroups
     const float max_exp = __uint_as_float(slot->max_exp_bits);
     ignore_thr *= max_exp;
     under_thr *= max_exp;
@@ -63,8 +89,8 @@ __global__ __launch_bounds__(kBlock) void exp_stats_kernel(
     const unsigned long long head = mis < count_f ? mis : count_f;
     const float4 *body = reinterpret_cast<const float4 *>(ptr + head);
     const unsigned long long nvec = (count_f - head) / 4;
-    const unsigned long long gsz = (unsigned long long)gridDim.x * kBlock;
-    unsigned long long i = (unsigned long long)blockIdx.x * kBlock + tid;
+    const unsigned long long gsz = (unsigned long long)nblocks * kBlock;
+    unsigned long long i = (unsigned long long)bid * kBlock + tid;
     auto count4 = [&](const float4 &v) {
       count_one(acc, v.x, ignore_thr, under_thr); count_one(acc, v.y, ignore_thr, under_thr);
       count_one(acc, v.z, ignore_thr, under_thr); count_one(acc, v.w, ignore_thr, under_thr);
@@ -75,7 +101,7 @@ __global__ __launch_bounds__(kBlock) void exp_stats_kernel(
     // stride apart would fall on the same memory channels).
     constexpr unsigned long long kChunk = 8ull * kBlock;
     const unsigned long long nfull = nvec / kChunk;
-    for (unsigned long long c = blockIdx.x; c < nfull; c += gridDim.x) {
+    for (unsigned long long c = bid; c < nfull; c += nblocks) {
       const float4 *cp = body + c * kChunk + tid;
       float4 v[8];
 #pragma unroll
@@ -87,7 +113,7 @@ __global__ __launch_bounds__(kBlock) void exp_stats_kernel(
     for (; i < nvec; i += gsz) {
       count4(body[i]);
     }
-    if (blockIdx.x == 0) {
+    if (bid == 0) {
       if (tid < head) count_one(acc, ptr[tid], ignore_thr, under_thr);
       const unsigned long long tail0 = head + nvec * 4;
       if (tail0 + tid < count_f) count_one(acc, ptr[tail0 + tid], ignore_thr, under_thr);
@@ -96,8 +122,8 @@ __global__ __launch_bounds__(kBlock) void exp_stats_kernel(
     // strided view: one column (of m_f floats) per wave iteration
     const unsigned long long ncols = (unsigned long long)n * nbatch;
     const unsigned lane = tid & 63;
-    for (unsigned long long col = (unsigned long long)blockIdx.x * kWaves + (tid >> 6); col < ncols;
-         col += (unsigned long long)gridDim.x * kWaves) {
+    for (unsigned long long col = (unsigned long long)bid * kWaves + (tid >> 6); col < ncols;
+         col += (unsigned long long)nblocks * kWaves) {
       const float *cp = ptr + (col / n) * stride_f + (col % n) * ld_f;
       unsigned i = lane;
       for (; i + 192 < m_f; i += 256) {
@@ -141,7 +167,7 @@ __global__ __launch_bounds__(kBlock) void exp_stats_kernel(
       // for them to be acknowledged, then take a ticket.  A device-scope release
       // fence here instead would write back the whole L2 once per workgroup, and
       // those write-backs serialise: they cost several times the streaming loop.
-      StatsPartial *p = partials + blockIdx.x;
+      StatsPartial *p = partials + bid;
       __hip_atomic_store(&p->max_bits, __float_as_uint(mx) & 0x7f800000u, __ATOMIC_RELAXED,
                          __HIP_MEMORY_SCOPE_AGENT);
       __hip_atomic_store(&p->total, t, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -150,7 +176,7 @@ __global__ __launch_bounds__(kBlock) void exp_stats_kernel(
       __builtin_amdgcn_s_waitcnt(0);
       const unsigned arrived =
           __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      s_last = (arrived == gridDim.x - 1);
+      s_last = (arrived == nblocks - 1);
     }
   }
   __syncthreads();
@@ -161,7 +187,7 @@ __global__ __launch_bounds__(kBlock) void exp_stats_kernel(
   __threadfence();
   unsigned mxb = 0;
   unsigned long long t = 0, u = 0;
-  for (unsigned i = tid; i < gridDim.x; i += kBlock) {
+  for (unsigned i = tid; i < nblocks; i += kBlock) {
     StatsPartial *p = partials + i;
     const unsigned b = __hip_atomic_load(&p->max_bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     const unsigned long long pt = __hip_atomic_load(&p->total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -270,38 +296,76 @@ unsigned next_slot(cuMpSGEMM_handle *h) {
 }
 
 template <class T>
+StatsJob make_job(cuMpSGEMM_handle *h, const View &v, const T *ptr, unsigned slot_id, unsigned which,
+                  unsigned first_partial) {
+  StatsJob j{};
+  j.slot = h->stats_slots + slot_id;
+  j.partials = h->stats_partials + first_partial;
+  j.ticket = h->stats_ticket + which;
+  j.ptr = reinterpret_cast<const float *>(ptr);
+  j.count_f = v.count_f;
+  j.m_f = v.m_f;
+  j.n = v.n;
+  j.ld_f = v.ld_f;
+  j.nbatch = v.nbatch;
+  j.stride_f = v.stride_f;
+  j.blocks = v.grid;
+  return j;
+}
+
+// MODE 0 + 1 (full statistics) or 2 (maximum only) over one job or two
+template <bool FULL>
+void launch_stats(cuMpSGEMM_handle *h, const StatsJob &j0, const StatsJob &j1) {
+  const dim3 grid(j0.blocks + j1.blocks);
+  if (FULL) {
+    {
+      ProfileScope prof(h, "exp_stats_1");
+      hipLaunchKernelGGL(exp_stats_kernel<0>, grid, dim3(kBlock), 0, h->stream, j0, j1, h->ignore_threshold,
+                         h->underflow_threshold, h->underflow_tolerance_rate);
+    }
+    {
+      ProfileScope prof(h, "exp_stats_2");
+      // stage-2 thresholds are half the stage-1 ones, times the max exponent
+      // (reference src/exp_stats.cu:360-361, :205-206)
+      hipLaunchKernelGGL(exp_stats_kernel<1>, grid, dim3(kBlock), 0, h->stream, j0, j1, h->ignore_threshold / 2,
+                         h->underflow_threshold / 2, h->underflow_tolerance_rate);
+    }
+  } else {
+    ProfileScope prof(h, "exp_max");
+    hipLaunchKernelGGL(exp_stats_kernel<2>, grid, dim3(kBlock), 0, h->stream, j0, j1, 0.0f, 0.0f, 0.0f);
+  }
+}
+
+template <class T>
 void run_exp_stats(cuMpSGEMM_handle *h, unsigned m, unsigned n, const T *ptr, unsigned ld,
                    unsigned batch, unsigned stride, unsigned slot_id) {
   const View v = make_view<T>(h, m, n, ld, batch, stride);
-  StatsSlot *slot = h->stats_slots + slot_id;
-  const float *p = reinterpret_cast<const float *>(ptr);
-  {
-    ProfileScope prof(h, "exp_stats_1");
-    hipLaunchKernelGGL(exp_stats_kernel<0>, dim3(v.grid), dim3(kBlock), 0, h->stream, slot,
-                       h->stats_partials, h->stats_ticket, p, v.count_f, v.m_f, v.n, v.ld_f,
-                       v.nbatch, v.stride_f, h->ignore_threshold, h->underflow_threshold,
-                       h->underflow_tolerance_rate);
-  }
-  {
-    ProfileScope prof(h, "exp_stats_2");
-    // stage-2 thresholds are half the stage-1 ones, times the max exponent
-    // (reference src/exp_stats.cu:360-361, :205-206)
-    hipLaunchKernelGGL(exp_stats_kernel<1>, dim3(v.grid), dim3(kBlock), 0, h->stream, slot,
-                       h->stats_partials, h->stats_ticket, p, v.count_f, v.m_f, v.n, v.ld_f,
-                       v.nbatch, v.stride_f, h->ignore_threshold / 2, h->underflow_threshold / 2,
-                       h->underflow_tolerance_rate);
-  }
+  launch_stats<true>(h, make_job<T>(h, v, ptr, slot_id, 0, 0), StatsJob{});
 }
 
 template <class T>
 void run_exp_max(cuMpSGEMM_handle *h, unsigned m, unsigned n, const T *ptr, unsigned ld,
                  unsigned batch, unsigned stride, unsigned slot_id) {
   const View v = make_view<T>(h, m, n, ld, batch, stride);
-  ProfileScope prof(h, "exp_max");
-  hipLaunchKernelGGL(exp_stats_kernel<2>, dim3(v.grid), dim3(kBlock), 0, h->stream,
-                     h->stats_slots + slot_id, h->stats_partials, h->stats_ticket,
-                     reinterpret_cast<const float *>(ptr), v.count_f, v.m_f, v.n, v.ld_f,
-                     v.nbatch, v.stride_f, 0.0f, 0.0f, 0.0f);
+  launch_stats<false>(h, make_job<T>(h, v, ptr, slot_id, 0, 0), StatsJob{});
+}
+
+// Two matrices in one launch; the workgroups (one per CU) are shared out in
+// proportion to the sizes.
+template <class T, bool FULL>
+void run_pair(cuMpSGEMM_handle *h, const MatrixView<T> &a, unsigned slot_a, const MatrixView<T> &b,
+              unsigned slot_b) {
+  View va = make_view<T>(h, a.m, a.n, a.ld, a.batch, a.stride);
+  View vb = make_view<T>(h, b.m, b.n, b.ld, b.batch, b.stride);
+  const unsigned long long cap = std::min<unsigned long long>((unsigned long long)h->num_cus, kMaxStatsBlocks);
+  if ((unsigned long long)va.grid + vb.grid > cap) {
+    const double wa = (double)a.m * a.n * va.nbatch, wb = (double)b.m * b.n * vb.nbatch;
+    unsigned ga = (unsigned)((double)cap * wa / (wa + wb) + 0.5);
+    ga = std::max(1u, std::min(ga, (unsigned)cap - 1u));
+    va.grid = std::min(va.grid, ga);
+    vb.grid = std::min(vb.grid, (unsigned)cap - va.grid);
+  }
+  launch_stats<FULL>(h, make_job<T>(h, va, a.ptr, slot_a, 0, 0), make_job<T>(h, vb, b.ptr, slot_b, 1, va.grid));
 }
 
 void read_slot(cuMpSGEMM_handle *h, unsigned id, StatsSlot &out) {
@@ -311,6 +375,29 @@ void read_slot(cuMpSGEMM_handle *h, unsigned id, StatsSlot &out) {
   check_hip(hipStreamSynchronize(h->stream), "sync after stats read");
 }
 } // namespace
+
+template <class T>
+void exp_stats_pair(cuMpSGEMM_handle *h, const MatrixView<T> &a, const MatrixView<T> &b, unsigned &a_id,
+                    unsigned &b_id) {
+  a_id = next_slot(h);
+  b_id = next_slot(h);
+  run_pair<T, true>(h, a, a_id, b, b_id);
+}
+template <class T>
+void exp_max_pair(cuMpSGEMM_handle *h, const MatrixView<T> &a, const MatrixView<T> &b, unsigned &a_id,
+                  unsigned &b_id) {
+  a_id = next_slot(h);
+  b_id = next_slot(h);
+  run_pair<T, false>(h, a, a_id, b, b_id);
+}
+template void exp_stats_pair<float>(cuMpSGEMM_handle *, const MatrixView<float> &, const MatrixView<float> &,
+                                    unsigned &, unsigned &);
+template void exp_stats_pair<hipComplex>(cuMpSGEMM_handle *, const MatrixView<hipComplex> &,
+                                         const MatrixView<hipComplex> &, unsigned &, unsigned &);
+template void exp_max_pair<float>(cuMpSGEMM_handle *, const MatrixView<float> &, const MatrixView<float> &,
+                                  unsigned &, unsigned &);
+template void exp_max_pair<hipComplex>(cuMpSGEMM_handle *, const MatrixView<hipComplex> &,
+                                       const MatrixView<hipComplex> &, unsigned &, unsigned &);
 } // namespace cumpsgemm_amd
 
 using namespace cumpsgemm_amd;

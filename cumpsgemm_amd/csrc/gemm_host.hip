@@ -63,7 +63,8 @@ __global__ void init_rings_kernel(StatsSlot *slots, int *flags, unsigned *ticket
     slots[1].mode = CUMPSGEMM_FP16TCEC;
     flags[0] = CUMPSGEMM_TF32TCEC;
     flags[1] = (3 << 5) | CUMPSGEMM_FP16TCEC;
-    *ticket = 0;
+    ticket[0] = 0;
+    ticket[1] = 0;
   }
 }
 
@@ -368,10 +369,9 @@ PreSplit run_pre_split(cuMpSGEMM_handle *h, const GemmArgs &args, bool a_kc, boo
       pargs.scale_max_b = max_b;
       pargs.scale_flag = sflag;
     }
-    launch_pack_split(h->stream, af, a_kc, lda, (uint32_t)m, (uint32_t)k, pa, mp, kind, max_a, sflag, 0x40,
-                      gate, accept);
-    launch_pack_split(h->stream, bf, b_kc, ldb, (uint32_t)n, (uint32_t)k, pb, np, kind, max_b, sflag, 0x20,
-                      gate, accept);
+    launch_pack_split_pair(h->stream, PackOperand{af, a_kc, lda, (uint32_t)m, pa, mp, max_a},
+                           PackOperand{bf, b_kc, ldb, (uint32_t)n, pb, np, max_b}, (uint32_t)k, kind, sflag, gate,
+                           accept);
     pargs.a = pa;
     pargs.b = pb;
     pargs.lda = mp; // padded row counts of the packed operands
@@ -701,7 +701,7 @@ hipblasStatus_t cuMpSGEMM_create(cuMpSGEMM_handle_t *handle) {
   bool ok = true;
   ok = ok && hipMalloc(&h->stats_slots, sizeof(StatsSlot) * h->stats_ring_length) == hipSuccess;
   ok = ok && hipMalloc(&h->stats_partials, sizeof(StatsPartial) * kMaxStatsBlocks) == hipSuccess;
-  ok = ok && hipMalloc(&h->stats_ticket, sizeof(unsigned)) == hipSuccess;
+  ok = ok && hipMalloc(&h->stats_ticket, 2 * sizeof(unsigned)) == hipSuccess;
   ok = ok && hipMalloc(&h->flag_buffer, sizeof(int) * h->flag_ring_length) == hipSuccess;
   ok = ok && hipHostMalloc(&h->host_scratch, sizeof(unsigned long long) * 4, hipHostMallocDefault) ==
                  hipSuccess;

@@ -54,7 +54,7 @@ struct cuMpSGEMM_handle {
   bool exp_stats_enabled = false;
   cumpsgemm_amd::StatsSlot *stats_slots = nullptr;       // [ring_length]
   cumpsgemm_amd::StatsPartial *stats_partials = nullptr; // [kMaxStatsBlocks]
-  unsigned *stats_ticket = nullptr;                      // self-resetting arrival counter
+  unsigned *stats_ticket = nullptr;                      // [2] self-resetting arrival counters
   unsigned stats_ring_length = cumpsgemm_amd::kRingLength;
   unsigned stats_current_id = 1; // slots 0 / 1 are reserved presets
   float ignore_threshold = 0.0f;
@@ -96,4 +96,18 @@ struct ProfileScope {
 };
 
 void check_hip(hipError_t err, const char *what);
+
+// Statistics of the two operands of a GEMM with one launch per pass instead
+// of two; same results and slot numbering as exp_stats_ext / exp_max_ext
+// called for A, then for B.
+template <class T> struct MatrixView {
+  const T *ptr;
+  unsigned m, n, ld, batch, stride;
+};
+template <class T>
+void exp_stats_pair(cuMpSGEMM_handle *h, const MatrixView<T> &a, const MatrixView<T> &b, unsigned &a_id,
+                    unsigned &b_id);
+template <class T>
+void exp_max_pair(cuMpSGEMM_handle *h, const MatrixView<T> &a, const MatrixView<T> &b, unsigned &a_id,
+                  unsigned &b_id);
 } // namespace cumpsgemm_amd

@@ -19,27 +19,37 @@ namespace cumpsgemm_amd {
 namespace {
 constexpr uint32_t kRowsPerBlock = 64;
 
+// One operand of a pre-pass launch.
+struct PackJob {
+  const float *src;
+  uint64_t ld;
+  uint32_t rows, k;
+  char *dst;
+  uint32_t rows_pad;
+  const uint32_t *scale_max; // nullptr: no scaling
+  int flag_bit;
+  uint32_t grid_x, grid_y, steps_per_block;
+};
+
 // KC: the source is K-contiguous (element (row, kk) at src[row * ld + kk]);
 // else row-contiguous (src[kk * ld + row]).
 // scale_max != nullptr: the operand is multiplied by 2^14 / *scale_max (the
 // bits of 2^floor(log2 max|x|) recorded by the statistics pass) while it is
 // split, if that maximum is non-zero and *scale_flag has `flag_bit` set -- the
 // coefficient of the stand-alone scaling kernels, read on the device.
+// `stage_mem`: LDS of the workgroup (used by the !KC form only).
 template <bool KC, Prec P, bool CPLX>
-__global__ __launch_bounds__(256) void pack_split_kernel(const float *__restrict__ src, uint64_t ld,
-                                                         uint32_t rows, uint32_t k,
-                                                         char *__restrict__ dst, uint32_t rows_pad,
-                                                         const uint32_t *scale_max,
-                                                         const int *scale_flag, int flag_bit,
-                                                         const int *launch_flag,
-                                                         uint32_t flag_accept_mask,
-                                                         uint32_t steps_per_block) {
-  // AUTO mode: nothing to do unless the launch flag names a mode this pass serves
-  if (launch_flag != nullptr && ((1u << (*launch_flag & 31)) & flag_accept_mask) == 0) return;
+__device__ inline void pack_split_body(const PackJob &job, const int *scale_flag, char *stage_mem,
+                                       const uint32_t block_x, const uint32_t block_y) {
+  const float *__restrict__ src = job.src;
+  char *__restrict__ dst = job.dst;
+  const uint64_t ld = job.ld;
+  const uint32_t rows = job.rows, k = job.k, rows_pad = job.rows_pad, steps_per_block = job.steps_per_block;
+  const uint32_t *scale_max = job.scale_max;
   float coef = 1.0f;
   if (scale_max != nullptr) {
     const float mx = __uint_as_float(*scale_max);
-    if ((*scale_flag & flag_bit) && mx != 0.0f) coef = 16384.0f / mx;
+    if ((*scale_flag & job.flag_bit) && mx != 0.0f) coef = 16384.0f / mx;
     coef = __uint_as_float(__builtin_amdgcn_readfirstlane(__float_as_uint(coef)));
   }
   // One workgroup converts `steps_per_block` K-steps of 64 rows, thread = (row,
@@ -56,10 +66,10 @@ __global__ __launch_bounds__(256) void pack_split_kernel(const float *__restrict
   // Complex sources are interleaved (re, im); their planes are re hi, re lo,
   // im hi, im lo.
   const uint32_t k_steps = (k + 31) / 32;
-  const uint32_t kb0 = blockIdx.y * steps_per_block;
+  const uint32_t kb0 = block_y * steps_per_block;
   const uint32_t t = threadIdx.x;
   const uint32_t lrow = KC ? t / 4 : t % kRowsPerBlock; // row within the block
-  const uint32_t row = blockIdx.x * kRowsPerBlock + lrow;
+  const uint32_t row = block_x * kRowsPerBlock + lrow;
   const uint32_t chunk = KC ? t % 4 : t / kRowsPerBlock;
   const bool row_in = row < rows;
   constexpr int NC = CPLX ? 2 : 1;
@@ -67,7 +77,8 @@ __global__ __launch_bounds__(256) void pack_split_kernel(const float *__restrict
   constexpr int NPL = NP * NC; // planes per K-step
   typedef float f4u_t __attribute__((ext_vector_type(4), aligned(4)));
   typedef float f2u_t __attribute__((ext_vector_type(2), aligned(4)));
-  __shared__ __attribute__((aligned(16))) char stage[KC ? 1 : 2][NPL][KC ? 16 : kRowsPerBlock * 64];
+  // (!KC) two K-steps x NPL planes x the 4 KiB image of the block
+  auto stage = [&](int buf, int plane) { return stage_mem + (buf * NPL + plane) * (int)(kRowsPerBlock * 64); };
 
   struct Vals {
     f8_t c[NC]; // the 8 K-values of the thread's chunk: real parts, imaginary parts
@@ -136,10 +147,10 @@ __global__ __launch_bounds__(256) void pack_split_kernel(const float *__restrict
       for (int pl = 0; pl < NP; pl++) {
         const int plane = q * NP + pl;
         if constexpr (KC) {
-          char *p = dst + (((uint64_t)kb * NPL + plane) * rows_pad + (uint64_t)blockIdx.x * kRowsPerBlock) * 64;
+          char *p = dst + (((uint64_t)kb * NPL + plane) * rows_pad + (uint64_t)block_x * kRowsPerBlock) * 64;
           *reinterpret_cast<u4_t *>(p + pos) = out[pl];
         } else {
-          *reinterpret_cast<u4_t *>(&stage[buf][plane][pos]) = out[pl];
+          *reinterpret_cast<u4_t *>(stage(buf, plane) + pos) = out[pl];
         }
       }
     }
@@ -147,8 +158,8 @@ __global__ __launch_bounds__(256) void pack_split_kernel(const float *__restrict
   auto copy_out = [&](uint32_t kb, int buf) { // !KC: 256 threads x 16 bytes = one plane of the block
 #pragma unroll
     for (int plane = 0; plane < NPL; plane++) {
-      char *p = dst + (((uint64_t)kb * NPL + plane) * rows_pad + (uint64_t)blockIdx.x * kRowsPerBlock) * 64;
-      *reinterpret_cast<u4_t *>(p + t * 16) = *reinterpret_cast<const u4_t *>(&stage[buf][plane][t * 16]);
+      char *p = dst + (((uint64_t)kb * NPL + plane) * rows_pad + (uint64_t)block_x * kRowsPerBlock) * 64;
+      *reinterpret_cast<u4_t *>(p + t * 16) = *reinterpret_cast<const u4_t *>(stage(buf, plane) + t * 16);
     }
   };
   for (uint32_t s = 0; s < steps_per_block; s += 2) {
@@ -170,32 +181,83 @@ __global__ __launch_bounds__(256) void pack_split_kernel(const float *__restrict
     }
   }
 }
+
+template <Prec P, bool CPLX> constexpr int stage_bytes(bool kc) {
+  return kc ? 16 : 2 * prec_traits<P>::NP * (CPLX ? 2 : 1) * (int)kRowsPerBlock * 64;
+}
+
+// AUTO mode: nothing to do unless the launch flag names a mode this pass serves
+__device__ inline bool gated_off(const int *launch_flag, uint32_t flag_accept_mask) {
+  return launch_flag != nullptr && ((1u << (*launch_flag & 31)) & flag_accept_mask) == 0;
+}
+
+// Both operands of a GEMM in one launch (blockIdx.z picks the operand; the grid
+// covers the larger of the two and the surplus workgroups of the other leave).
+template <bool KCA, bool KCB, Prec P, bool CPLX>
+__global__ __launch_bounds__(256) void pack_split_pair_kernel(const PackJob job_a, const PackJob job_b,
+                                                              const int *scale_flag, const int *launch_flag,
+                                                              uint32_t flag_accept_mask) {
+  if (gated_off(launch_flag, flag_accept_mask)) return;
+  __shared__ __attribute__((aligned(16))) char stage_mem[stage_bytes<P, CPLX>(KCA && KCB)];
+  if (blockIdx.z == 0) {
+    if (blockIdx.x < job_a.grid_x && blockIdx.y < job_a.grid_y)
+      pack_split_body<KCA, P, CPLX>(job_a, scale_flag, stage_mem, blockIdx.x, blockIdx.y);
+  } else {
+    if (blockIdx.x < job_b.grid_x && blockIdx.y < job_b.grid_y)
+      pack_split_body<KCB, P, CPLX>(job_b, scale_flag, stage_mem, blockIdx.x, blockIdx.y);
+  }
+}
+
+PackJob make_job(const PackOperand &o, uint32_t k, int flag_bit) {
+  PackJob j{};
+  j.src = o.src;
+  j.ld = o.ld;
+  j.rows = o.rows;
+  j.k = k;
+  j.dst = static_cast<char *>(o.dst);
+  j.rows_pad = o.rows_pad;
+  j.scale_max = o.scale_max;
+  j.flag_bit = flag_bit;
+  // up to 8 K-steps per workgroup, fewer while that would leave under ~2048 workgroups
+  const unsigned k_steps = (k + 31) / 32, row_blocks = o.rows_pad / kRowsPerBlock;
+  const unsigned spb = (unsigned)std::max<uint64_t>(1, std::min<uint64_t>(8, (uint64_t)k_steps * row_blocks / 2048));
+  j.grid_x = row_blocks;
+  j.grid_y = (k_steps + spb - 1) / spb;
+  j.steps_per_block = spb;
+  return j;
+}
+
+template <Prec P, bool CPLX>
+void launch_pair_of(hipStream_t stream, const PackJob &ja, bool a_kc, const PackJob &jb, bool b_kc,
+                    const int *scale_flag, const int *launch_flag, uint32_t flag_accept_mask) {
+  const dim3 grid(std::max(ja.grid_x, jb.grid_x), std::max(ja.grid_y, jb.grid_y), 2);
+  auto launch = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, grid, dim3(256), 0, stream, ja, jb, scale_flag, launch_flag, flag_accept_mask);
+  };
+  if (a_kc && b_kc) launch(pack_split_pair_kernel<true, true, P, CPLX>);
+  else if (a_kc) launch(pack_split_pair_kernel<true, false, P, CPLX>);
+  else if (b_kc) launch(pack_split_pair_kernel<false, true, P, CPLX>);
+  else launch(pack_split_pair_kernel<false, false, P, CPLX>);
+}
 } // namespace
 
-void launch_pack_split(hipStream_t stream, const float *src, bool k_contiguous, uint64_t ld,
-                       uint32_t rows, uint32_t k, void *dst, uint32_t rows_pad, PackKind kind,
-                       const uint32_t *scale_max, const int *scale_flag, int flag_bit,
-                       const int *launch_flag, uint32_t flag_accept_mask) {
-  // up to 8 K-steps per workgroup, fewer while that would leave under ~2048 workgroups
-  const unsigned k_steps = (k + 31) / 32, row_blocks = rows_pad / kRowsPerBlock;
-  const unsigned spb = (unsigned)std::max<uint64_t>(1, std::min<uint64_t>(8, (uint64_t)k_steps * row_blocks / 2048));
-  const dim3 grid(row_blocks, (k_steps + spb - 1) / spb);
-  auto launch = [&](auto kernel) {
-    hipLaunchKernelGGL(kernel, grid, dim3(256), 0, stream, src, ld, rows, k, static_cast<char *>(dst),
-                       rows_pad, scale_max, scale_flag, flag_bit, launch_flag, flag_accept_mask, spb);
-  };
+void launch_pack_split_pair(hipStream_t stream, const PackOperand &a, const PackOperand &b, uint32_t k,
+                            PackKind kind, const int *scale_flag, const int *launch_flag,
+                            uint32_t flag_accept_mask) {
+  // (the scale bits of the launch flag: 0x40 for A, 0x20 for B)
+  const PackJob ja = make_job(a, k, 0x40), jb = make_job(b, k, 0x20);
   switch (kind) {
   case PackKind::BF16X3_REAL:
-    if (k_contiguous) launch(pack_split_kernel<true, Prec::BF16X3, false>);
-    else launch(pack_split_kernel<false, Prec::BF16X3, false>);
+    launch_pair_of<Prec::BF16X3, false>(stream, ja, a.k_contiguous, jb, b.k_contiguous, scale_flag, launch_flag,
+                                        flag_accept_mask);
     break;
   case PackKind::FP16_COMPLEX:
-    if (k_contiguous) launch(pack_split_kernel<true, Prec::FP16TCEC, true>);
-    else launch(pack_split_kernel<false, Prec::FP16TCEC, true>);
+    launch_pair_of<Prec::FP16TCEC, true>(stream, ja, a.k_contiguous, jb, b.k_contiguous, scale_flag, launch_flag,
+                                         flag_accept_mask);
     break;
   default:
-    if (k_contiguous) launch(pack_split_kernel<true, Prec::FP16TCEC, false>);
-    else launch(pack_split_kernel<false, Prec::FP16TCEC, false>);
+    launch_pair_of<Prec::FP16TCEC, false>(stream, ja, a.k_contiguous, jb, b.k_contiguous, scale_flag,
+                                          launch_flag, flag_accept_mask);
     break;
   }
 }

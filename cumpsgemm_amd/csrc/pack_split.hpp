@@ -10,13 +10,21 @@ inline uint64_t packed_bytes(uint64_t rows_pad, uint64_t k, unsigned planes = 2)
 }
 inline uint32_t packed_rows(uint64_t rows) { return (uint32_t)((rows + 255) / 256 * 256); }
 enum class PackKind { FP16_REAL, FP16_COMPLEX, BF16X3_REAL };
-// `ld` in elements of the source (complex: complex elements).
-// scale_max / scale_flag / flag_bit: optional power-of-two scaling fused into
-// the split (nullptr: none); launch_flag / flag_accept_mask: optional AUTO-mode
-// gate, as in GemmArgs
-void launch_pack_split(hipStream_t stream, const float *src, bool k_contiguous, uint64_t ld,
-                       uint32_t rows, uint32_t k, void *dst, uint32_t rows_pad, PackKind kind,
-                       const uint32_t *scale_max = nullptr, const int *scale_flag = nullptr,
-                       int flag_bit = 0, const int *launch_flag = nullptr,
-                       uint32_t flag_accept_mask = 0);
+// One pre-pass launch converts both operands of a GEMM (same K).  `ld` in
+// elements of the source (complex: complex elements).  scale_max / scale_flag:
+// optional power-of-two scaling fused into the split (nullptr: none; A's is
+// governed by bit 0x40 of *scale_flag, B's by bit 0x20); launch_flag /
+// flag_accept_mask: optional AUTO-mode gate, as in GemmArgs.
+struct PackOperand {
+  const float *src;
+  bool k_contiguous;
+  uint64_t ld;
+  uint32_t rows;
+  void *dst;
+  uint32_t rows_pad;
+  const uint32_t *scale_max; // nullptr: no scaling
+};
+void launch_pack_split_pair(hipStream_t stream, const PackOperand &a, const PackOperand &b, uint32_t k,
+                            PackKind kind, const int *scale_flag = nullptr, const int *launch_flag = nullptr,
+                            uint32_t flag_accept_mask = 0);
 } // namespace cumpsgemm_amd

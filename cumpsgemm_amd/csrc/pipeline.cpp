@@ -27,6 +27,9 @@ hipblasStatus_t gemm_pipeline(cuMpSGEMM_handle_t h, hipblasOperation_t op_A,
   const unsigned sb_stride = batched ? (unsigned)strideb : 0u;
   const unsigned sc_stride = batched ? (unsigned)stridec : 0u;
 
+  // (the statistics of A and B share one launch per pass)
+  const MatrixView<T> va{a, a_rows, a_cols, (unsigned)lda, sb, sa_stride};
+  const MatrixView<T> vb{b, b_rows, b_cols, (unsigned)ldb, sb, sb_stride};
   unsigned a_id = 0, b_id = 0, flag_id = 0;
   const bool scaled = (mode == CUMPSGEMM_AUTO || mode == CUMPSGEMM_FP16TCEC_SCALING);
   // When A and B are to come out unchanged (restore_AB, the default) the
@@ -40,8 +43,7 @@ hipblasStatus_t gemm_pipeline(cuMpSGEMM_handle_t h, hipblasOperation_t op_A,
   // alpha*A*B + beta*C, while rescaling the finished C also rescales beta*C.
   const bool fused = scaled && restore_AB && std::getenv("CUMPSGEMM_NO_FUSED_SCALING") == nullptr;
   if (mode == CUMPSGEMM_AUTO) {
-    a_id = cumpsgemm::exp_stats_ext<T>(h, a_rows, a_cols, a, (unsigned)lda, sb, sa_stride);
-    b_id = cumpsgemm::exp_stats_ext<T>(h, b_rows, b_cols, b, (unsigned)ldb, sb, sb_stride);
+    exp_stats_pair<T>(h, va, vb, a_id, b_id);
     flag_id = cumpsgemm::get_next_dynamic_launch_buffer_id(h);
     cumpsgemm::set_dynamic_launch_buffer_by_exp_stats(h, flag_id, a_id, b_id);
     if (!fused) {
@@ -51,8 +53,7 @@ hipblasStatus_t gemm_pipeline(cuMpSGEMM_handle_t h, hipblasOperation_t op_A,
     cumpsgemm::set_dynamic_launch_flag_buffer_id(h, flag_id);
   } else if (mode == CUMPSGEMM_FP16TCEC_SCALING) {
     flag_id = 1; // preset: FP16TCEC with both scale bits
-    a_id = cumpsgemm::exp_max_ext<T>(h, a_rows, a_cols, a, (unsigned)lda, sb, sa_stride);
-    b_id = cumpsgemm::exp_max_ext<T>(h, b_rows, b_cols, b, (unsigned)ldb, sb, sb_stride);
+    exp_max_pair<T>(h, va, vb, a_id, b_id);
     if (!fused) {
       cumpsgemm::scale_A<T>(h, a_id, flag_id, a_rows, a_cols, a, (unsigned)lda, sb, sa_stride);
       cumpsgemm::scale_B<T>(h, b_id, flag_id, b_rows, b_cols, b, (unsigned)ldb, sb, sb_stride);
