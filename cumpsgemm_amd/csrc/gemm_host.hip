@@ -729,6 +729,7 @@ hipblasStatus_t cuMpSGEMM_destroy(cuMpSGEMM_handle_t handle) {
   (void)hipFree(handle->stats_ticket);
   (void)hipFree(handle->flag_buffer);
   if (handle->pack_ws != nullptr) (void)hipFree(handle->pack_ws);
+  if (handle->order_event != nullptr) (void)hipEventDestroy(handle->order_event);
   if (handle->host_scratch) (void)hipHostFree(handle->host_scratch);
   delete handle;
   return HIPBLAS_STATUS_SUCCESS;
@@ -736,6 +737,30 @@ hipblasStatus_t cuMpSGEMM_destroy(cuMpSGEMM_handle_t handle) {
 
 hipblasStatus_t cuMpSGEMM_set_stream(cuMpSGEMM_handle_t handle, hipStream_t stream) {
   if (handle == nullptr) return HIPBLAS_STATUS_INVALID_VALUE;
+  if (stream != handle->stream) {
+    // order the new stream behind the handle's work on the old one (a stream
+    // under graph capture is left alone: its work runs when the graph does)
+    hipStreamCaptureStatus old_cap = hipStreamCaptureStatusNone, new_cap = hipStreamCaptureStatusNone;
+    (void)hipStreamIsCapturing(handle->stream, &old_cap);
+    (void)hipStreamIsCapturing(stream, &new_cap);
+    if (old_cap == hipStreamCaptureStatusNone && new_cap == hipStreamCaptureStatusNone) {
+      if (handle->order_event == nullptr &&
+          hipEventCreateWithFlags(&handle->order_event, hipEventDisableTiming) != hipSuccess) {
+        handle->order_event = nullptr;
+        (void)hipGetLastError();
+      }
+      if (handle->order_event != nullptr) {
+        if (hipEventRecord(handle->order_event, handle->stream) != hipSuccess ||
+            hipStreamWaitEvent(stream, handle->order_event, 0) != hipSuccess) {
+          (void)hipGetLastError();
+          (void)hipStreamSynchronize(handle->stream); // the blunt way
+        }
+      } else {
+        (void)hipStreamSynchronize(handle->stream);
+      }
+    }
+    (void)hipGetLastError();
+  }
   handle->stream = stream;
   return HIPBLAS_STATUS_SUCCESS;
 }

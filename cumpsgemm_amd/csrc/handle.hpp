@@ -79,6 +79,12 @@ struct cuMpSGEMM_handle {
   void *pack_ws = nullptr;
   unsigned long long pack_ws_bytes = 0;
 
+  // The rings, partials and workspaces above are shared by every call on the
+  // handle, so work of the handle on two streams must not overlap: when the
+  // stream changes, the new one is made to wait (on the device, through this
+  // event) for what was queued on the old one.
+  hipEvent_t order_event = nullptr;
+
   // pinned host word for small read-backs
   unsigned long long *host_scratch = nullptr; // [4]
 

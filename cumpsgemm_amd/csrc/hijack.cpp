@@ -235,6 +235,13 @@ hipblasStatus_t hijack_core(const char *func_name, hipblasHandle_t hb, hipblasOp
     return HIPBLAS_STATUS_INVALID_VALUE;
   }
   const cuMpSGEMM_compute_mode_t mode = query_mode(func_name, hb, op_A, op_B, m, n, k);
+  // One intercepted call at a time from here on: the process-wide handle, the
+  // record of the last call and the stream it runs on are shared by all host
+  // threads.  (The rule hook above runs outside the lock: it may call back
+  // into user code.  Recursive, in case the vendor library's own GEMM entry
+  // points call each other through the dynamic symbol table.)
+  static std::recursive_mutex call_mutex;
+  const std::lock_guard<std::recursive_mutex> lock(call_mutex);
   // a dry run only logs: it must not need a device, so the handle is created after it
   cuMpSGEMM_handle_t h = (mode == CUMPSGEMM_DRY_RUN) ? g_handle : global_handle();
 

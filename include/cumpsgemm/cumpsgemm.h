@@ -7,7 +7,9 @@
  * Matrices are column-major device pointers that are only borrowed for the
  * duration of the (asynchronous) call; alpha/beta are HOST pointers and are
  * read before the call returns; work is enqueued on the handle's stream and
- * never synchronised.  The handle is not thread-safe (as in the reference).
+ * never synchronised.  The handle is not thread-safe (as in the reference);
+ * its scratch is shared by all its calls, so changing its stream orders the
+ * new stream behind the work queued on the old one.
  */
 #ifndef CUMPSGEMM_AMD_H
 #define CUMPSGEMM_AMD_H

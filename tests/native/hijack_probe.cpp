@@ -13,6 +13,7 @@
 #include <cstdint>
 #include <cstdio>
 #include <cstdlib>
+#include <thread>
 #include <vector>
 
 #define CHECK_HIP(x)                                                                      \
@@ -46,7 +47,9 @@ static void report(const char *name, hipblasStatus_t st, double num, double den)
 }
 
 int main(int argc, char **argv) {
-  const int n = (argc > 1) ? std::atoi(argv[1]) : 1280; // > 1024 so the default rule engages
+  // > 1024 so the default rule engages
+  const char *env_n = std::getenv("PROBE_N");
+  const int n = (argc > 1) ? std::atoi(argv[1]) : (env_n != nullptr ? std::atoi(env_n) : 1280);
   const int batch = 3;
   hipblasHandle_t hb;
   if (hipblasCreate(&hb) != HIPBLAS_STATUS_SUCCESS) {
@@ -158,6 +161,63 @@ int main(int argc, char **argv) {
       den += (double)n * n;
     }
     report("hipblasGemmEx_f16_in", st, num, den);
+  }
+
+  // ---- several host threads, each with its own hipBLAS handle and stream ----
+  // (PROBE_THREADS=<count>: every thread repeats two products of different
+  // shapes and compares each result with the one the main thread computed)
+  if (const char *pt = std::getenv("PROBE_THREADS")) {
+    const int nthreads = std::atoi(pt), reps = 12;
+    const int n2 = n - 256; // a second shape, so that consecutive calls differ in their workspace use
+    std::vector<float> ref1(e), ref2((size_t)n2 * n2);
+    CHECK_HIP(hipMemsetAsync(dc.p, 0, e * 4, stream));
+    st = hipblasSgemm(hb, HIPBLAS_OP_N, HIPBLAS_OP_T, n, n, n, &one, da.p, n, db.p, n, &zero, dc.p, n);
+    CHECK_HIP(hipMemcpyAsync(ref1.data(), dc.p, e * 4, hipMemcpyDeviceToHost, stream));
+    st = hipblasSgemm(hb, HIPBLAS_OP_N, HIPBLAS_OP_T, n2, n2, n2, &one, da.p, n, db.p, n, &zero, dc.p, n2);
+    CHECK_HIP(hipMemcpyAsync(ref2.data(), dc.p, (size_t)n2 * n2 * 4, hipMemcpyDeviceToHost, stream));
+    CHECK_HIP(hipStreamSynchronize(stream));
+    std::vector<long> bad(nthreads, 0);
+    std::vector<int> status(nthreads, 0);
+    std::vector<std::thread> pool;
+    for (int t = 0; t < nthreads; t++) {
+      pool.emplace_back([&, t]() {
+        hipblasHandle_t hbt;
+        hipStream_t st_t;
+        if (hipblasCreate(&hbt) != HIPBLAS_STATUS_SUCCESS || hipStreamCreate(&st_t) != hipSuccess) {
+          status[t] = -1;
+          return;
+        }
+        hipblasSetStream(hbt, st_t);
+        dev_buf<float> dct(e);
+        std::vector<float> got(e);
+        for (int r = 0; r < reps; r++) {
+          const bool big = ((r + t) % 2) == 0;
+          const int nn = big ? n : n2;
+          const size_t ee = (size_t)nn * nn;
+          (void)hipMemsetAsync(dct.p, 0, ee * 4, st_t);
+          const hipblasStatus_t s2 =
+              hipblasSgemm(hbt, HIPBLAS_OP_N, HIPBLAS_OP_T, nn, nn, nn, &one, da.p, n, db.p, n, &zero, dct.p, nn);
+          if (s2 != HIPBLAS_STATUS_SUCCESS) status[t] = (int)s2;
+          (void)hipMemcpyAsync(got.data(), dct.p, ee * 4, hipMemcpyDeviceToHost, st_t);
+          (void)hipStreamSynchronize(st_t);
+          const std::vector<float> &ref = big ? ref1 : ref2;
+          for (size_t i = 0; i < ee; i++) {
+            if (std::fabs(got[i] - ref[i]) > 1e-3f) bad[t]++;
+          }
+        }
+        hipblasDestroy(hbt);
+        (void)hipStreamDestroy(st_t);
+      });
+    }
+    for (auto &th : pool) th.join();
+    long total_bad = 0;
+    int worst = 0;
+    for (int t = 0; t < nthreads; t++) {
+      total_bad += bad[t];
+      if (status[t] != 0) worst = status[t];
+    }
+    std::printf("RESULT threads status=%d relerr=%.3e\n", worst, (double)total_bad);
+    std::fflush(stdout);
   }
 
   hipblasDestroy(hb);

@@ -103,3 +103,11 @@ def test_culip_profiling_lines():
     env["CUMPSGEMM_ENABLE_CULIP_PROFILING"] = "0"
     r0 = subprocess.run([PROBE], env=env, text=True, capture_output=True, timeout=300)
     assert "[CULiP Result]" not in r0.stdout
+
+
+def test_host_threads_with_their_own_streams_share_the_interposer():
+    """Four host threads, each with its own hipBLAS handle and stream, call the intercepted
+    hipblasSgemm at the same time (shapes large enough for the pre-split path and its shared
+    workspace): every result equals the one computed alone."""
+    res, _ = _probe({"CUMPSGEMM_COMPUTE_MODE": "FP16TCEC", "PROBE_THREADS": "4", "PROBE_N": "4096"})
+    assert res["threads"] == (0, 0.0)
