@@ -22,8 +22,20 @@
 namespace {
 using namespace cumpsgemm_amd;
 
-cuMpSGEMM_handle_t g_handle = nullptr;
-std::once_flag g_handle_once;
+// one library handle per device, created at the first intercepted call made
+// with that device current (the reference keeps a single one for the process,
+// src/cumpsgemm_cublas.cu:101-157)
+constexpr int kMaxDevices = 64;
+cuMpSGEMM_handle_t g_handles[kMaxDevices] = {};
+std::once_flag g_handle_once[kMaxDevices];
+int current_device() {
+  int d = 0;
+  if (hipGetDevice(&d) != hipSuccess) {
+    (void)hipGetLastError();
+    d = 0;
+  }
+  return (d >= 0 && d < kMaxDevices) ? d : 0;
+}
 std::string g_last_called;
 bool g_mx2x2_enabled = false;
 bool g_restore_AB = true;
@@ -83,7 +95,9 @@ int env_int(const char *name, int dflt) {
 }
 
 cuMpSGEMM_handle_t global_handle() {
-  std::call_once(g_handle_once, []() {
+  const int dev = current_device();
+  std::call_once(g_handle_once[dev], [dev]() {
+    cuMpSGEMM_handle_t &g_handle = g_handles[dev];
     log_info("Initialize cuMpSGEMM handle...");
     if (cuMpSGEMM_create(&g_handle) != HIPBLAS_STATUS_SUCCESS) {
       log_error("Initialization failed.");
@@ -103,7 +117,7 @@ cuMpSGEMM_handle_t global_handle() {
     cumpsgemm::set_exp_stats_params(g_handle, ignore_thr, under_thr, tol);
     g_restore_AB = restore != 0;
   });
-  return g_handle;
+  return g_handles[dev];
 }
 
 using rule_fn_t = cuMpSGEMM_compute_mode_t (*)(const char *, hipblasHandle_t, hipblasOperation_t,
@@ -243,7 +257,7 @@ hipblasStatus_t hijack_core(const char *func_name, hipblasHandle_t hb, hipblasOp
   static std::recursive_mutex call_mutex;
   const std::lock_guard<std::recursive_mutex> lock(call_mutex);
   // a dry run only logs: it must not need a device, so the handle is created after it
-  cuMpSGEMM_handle_t h = (mode == CUMPSGEMM_DRY_RUN) ? g_handle : global_handle();
+  cuMpSGEMM_handle_t h = (mode == CUMPSGEMM_DRY_RUN) ? g_handles[current_device()] : global_handle();
 
   log_info(std::string(func_name) + " op=(" + op_str(op_A) + ", " + op_str(op_B) + "), shape=(" +
            std::to_string(m) + ", " + std::to_string(n) + ", " + std::to_string(k) + ")" +
