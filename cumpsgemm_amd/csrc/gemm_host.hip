@@ -314,6 +314,11 @@ PreSplitChoice choose_pre_split(const cuMpSGEMM_handle *h, bool a_kc, bool b_kc,
 bool ensure_pack_workspace(cuMpSGEMM_handle *h, uint64_t bytes, bool *failed) {
   *failed = false;
   if (h->pack_ws_bytes >= bytes) return h->pack_ws != nullptr;
+  // no allocation or synchronisation while the stream is being captured into a
+  // graph: the call takes the path that needs no workspace instead
+  hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(h->stream, &cap) != hipSuccess) (void)hipGetLastError();
+  if (cap != hipStreamCaptureStatusNone) return false;
   // the previous workspace may still be in use by work queued on the stream
   if (hipStreamSynchronize(h->stream) != hipSuccess) {
     log_error("stream synchronisation failed before growing the pack workspace");

@@ -62,3 +62,47 @@ def test_captured_calls_replay_like_eager_calls(cg, torch_gpu, mode, cplx):
     finally:
         torch.cuda.synchronize()
         h.close()
+
+
+def test_capture_never_grows_the_workspace(cg, torch_gpu, monkeypatch):
+    """A call that would take the pre-split path while its workspace is still missing must not
+    allocate or synchronise under capture: it runs the in-loop kernels instead (same bits)."""
+    torch = torch_gpu
+    m, n, k = 4096, 3840, 768
+    dev = torch.device("cuda:0")
+    h = cg.Handle()
+    side = torch.cuda.Stream()
+    a = torch.from_numpy(inputs.uniform(31, m * k)).to(dev)
+    b = torch.from_numpy(inputs.uniform(32, k * n)).to(dev)
+    c_graph = torch.zeros(m * n, device=dev)
+    c_eager = torch.zeros(m * n, device=dev)
+
+    def call(c_out):
+        # op_A = N, op_B = T: both operands M/N-contiguous, the layout that pre-splits from K = 256 on
+        return h.gemm(N_OP, 112, m, n, k, 1.0, a, m, b, n, 0.0, c_out, m, FP16TCEC, want_module_id=True)
+
+    try:
+        h.set_stream(side)
+        monkeypatch.setenv("CUMPSGEMM_PACKED", "0")
+        with torch.cuda.stream(side):
+            assert call(c_graph)[0] == 0        # loads the in-loop kernels, leaves the workspace alone
+        torch.cuda.synchronize()
+        monkeypatch.delenv("CUMPSGEMM_PACKED")
+        assert h.workspace_size() == 0
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=side):
+            h.set_stream(torch.cuda.current_stream())
+            st, mid = call(c_graph)
+        assert st == 0 and mid != 200 and h.workspace_size() == 0
+        c_graph.zero_()
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        h.set_stream(torch.cuda.current_stream())
+        st, mid = call(c_eager)                 # eager: allocates and takes the pre-split path
+        torch.cuda.synchronize()
+        assert st == 0 and mid == 200 and h.workspace_size() >= (m + n) * k * 4
+        assert torch.equal(c_graph, c_eager)
+    finally:
+        torch.cuda.synchronize()
+        h.close()
