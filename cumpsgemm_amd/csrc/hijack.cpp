@@ -315,9 +315,13 @@ hipblasStatus_t hijack_core(const char *func_name, hipblasHandle_t hb, hipblasOp
                 : forward_gemm<T>(hb, op_A, op_B, m, n, k, alpha, a, lda, b, ldb, beta, c, ldc);
     if (h->exp_stats_enabled) {
       // statistics of the result, as the reference does for forwarded calls
-      // (src/cumpsgemm_cublas.cu:420-425)
-      cumpsgemm::exp_stats_ext<T>(h, (unsigned)m, (unsigned)n, c, (unsigned)ldc,
-                                  batched ? (unsigned)batch : 1u, batched ? (unsigned)sc : 0u);
+      // (src/cumpsgemm_cublas.cu:420-425); the statistics take a 32-bit stride
+      if (batched && (sc < 0 || sc > 0xffffffffll)) {
+        log_warning("exp_stats of C skipped: the batch stride does not fit 32 bits");
+      } else {
+        cumpsgemm::exp_stats_ext<T>(h, (unsigned)m, (unsigned)n, c, (unsigned)ldc,
+                                    batched ? (unsigned)batch : 1u, batched ? (unsigned)sc : 0u);
+      }
     }
     return st;
   }

@@ -6,6 +6,7 @@
 #include "pipeline.hpp"
 #include <cstdlib>
 #include "handle.hpp"
+#include "utils.hpp"
 #include <cumpsgemm/cumpsgemm_ext.h>
 
 namespace cumpsgemm_amd {
@@ -16,6 +17,15 @@ hipblasStatus_t gemm_pipeline(cuMpSGEMM_handle_t h, hipblasOperation_t op_A,
                               uint64_t ldb, uint64_t strideb, const T *beta, T *c, uint64_t ldc,
                               uint64_t stridec, uint64_t batch, bool batched,
                               cuMpSGEMM_compute_mode_t mode, bool restore_AB, PipelineIds *ids) {
+  // the statistics and scaling entry points take 32-bit sizes, leading
+  // dimensions and strides (reference include/cumpsgemm/cumpsgemm.hpp:37-46)
+  const bool needs_stats = (mode == CUMPSGEMM_AUTO || mode == CUMPSGEMM_FP16TCEC_SCALING);
+  const uint64_t lim = 0xffffffffull;
+  if (needs_stats && (m > lim || n > lim || k > lim || lda > lim || ldb > lim || ldc > lim ||
+                      (batched && (stridea > lim || strideb > lim || stridec > lim || batch > lim)))) {
+    log_error("FP16TCEC_SCALING / AUTO: a size, leading dimension or stride does not fit 32 bits");
+    return HIPBLAS_STATUS_INVALID_VALUE;
+  }
   // stored shapes of A and B (rows x cols as laid out in memory)
   const unsigned a_rows = (unsigned)(op_A == HIPBLAS_OP_N ? m : k);
   const unsigned a_cols = (unsigned)(op_A == HIPBLAS_OP_N ? k : m);

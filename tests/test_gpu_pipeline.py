@@ -248,3 +248,21 @@ def test_auto_pre_split_path_steps_aside_for_bf16x3(O, cg, torch_gpu, dev, monke
     ref = O.gemm_fp64(N, N, m, n, k, 1.0, a, m, b, k)
     cf = oracle_gemm(O, FP32, N, N, m, n, k, 1.0, a, m, b, k, 0.0, np.zeros(m * n, np.float32), m)
     assert O.residual(ref, outs[1], m, n, m) <= 2.0 * O.residual(ref, cf, m, n, m)
+
+
+@pytest.mark.parametrize("mode", [SCALING, AUTO])
+def test_pipeline_rejects_what_the_statistics_cannot_address(handle, dev, mode):
+    """The statistics and scaling passes take 32-bit leading dimensions and strides (as in the
+    reference); a scaled call that needs more is refused before anything is launched."""
+    x = dev.up(np.ones(64, np.float32))
+    big = (1 << 32) + 8
+    # batched, stride of A beyond 32 bits (nothing is read: the call returns at once)
+    st, _ = handle.gemm_pipeline(N, N, 4, 4, 4, 1.0, x, 4, x, 4, 0.0, x, 4, mode, stridea=big, strideb=16,
+                                 stridec=16, batch=2)
+    assert st == 3                       # HIPBLAS_STATUS_INVALID_VALUE
+    st, _ = handle.gemm_pipeline(N, N, 4, 4, 4, 1.0, x, big, x, 4, 0.0, x, 4, mode)
+    assert st == 3
+    # the plain modes address with 64 bits and take the same arguments
+    c = dev.up(np.zeros(16, np.float32))
+    st, _ = handle.gemm_pipeline(N, N, 4, 4, 1, 1.0, x, big, x, 4, 0.0, c, 4, FP16TCEC)
+    assert st == 0 and np.array_equal(dev.down(c), np.ones(16, np.float32))
