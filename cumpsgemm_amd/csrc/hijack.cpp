@@ -273,6 +273,11 @@ hipblasStatus_t hijack_core(const char *func_name, hipblasHandle_t hb, hipblasOp
   if (mode == CUMPSGEMM_DRY_RUN) return HIPBLAS_STATUS_SUCCESS;
   if (h == nullptr) return HIPBLAS_STATUS_NOT_INITIALIZED;
 
+  if (batched && (sa < 0 || sb < 0 || sc < 0)) {
+    // not something this library's kernels address; the vendor library decides what it means
+    log_warning("negative batch stride: forwarding to hipBLAS");
+    return forward_gemm_sb<T>(hb, op_A, op_B, m, n, k, alpha, a, lda, sa, b, ldb, sb, beta, c, ldc, sc, batch);
+  }
   // kernels of this library run on the caller's stream so that ordering with
   // the application's other work is preserved
   cuMpSGEMM_set_stream(h, caller_stream(hb));
