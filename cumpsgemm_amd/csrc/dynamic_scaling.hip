@@ -95,6 +95,10 @@ void launch_scaling(cuMpSGEMM_handle *h, int kind, unsigned slot_a, unsigned slo
                     unsigned flag_id, unsigned m, unsigned n, T *ptr, unsigned ld, unsigned batch,
                     unsigned stride, const char *label) {
   constexpr unsigned ES = std::is_same<T, hipComplex>::value ? 2 : 1;
+  if (ptr == nullptr || m == 0 || n == 0) {
+    if (ptr == nullptr && m != 0 && n != 0) log_error(std::string(label) + ": null matrix pointer, nothing scaled");
+    return;
+  }
   const unsigned nbatch = (stride == 0) ? 1 : batch;
   const bool dense_cols = (ld == m) || n == 1;
   const bool dense_batch = nbatch == 1 || (unsigned long long)stride == (unsigned long long)m * n;

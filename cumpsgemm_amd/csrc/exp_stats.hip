@@ -316,6 +316,13 @@ StatsJob make_job(cuMpSGEMM_handle *h, const View &v, const T *ptr, unsigned slo
 // MODE 0 + 1 (full statistics) or 2 (maximum only) over one job or two
 template <bool FULL>
 void launch_stats(cuMpSGEMM_handle *h, const StatsJob &j0, const StatsJob &j1) {
+  // (a null matrix would fault on the device; an empty one has nothing to read)
+  const bool bad0 = j0.ptr == nullptr && j0.m_f != 0 && j0.n != 0;
+  const bool bad1 = j1.blocks != 0 && j1.ptr == nullptr && j1.m_f != 0 && j1.n != 0;
+  if (bad0 || bad1) {
+    log_error("exponent statistics: null matrix pointer, nothing scanned");
+    return;
+  }
   const dim3 grid(j0.blocks + j1.blocks);
   if (FULL) {
     {

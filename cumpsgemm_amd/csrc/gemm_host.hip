@@ -457,9 +457,10 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
     return HIPBLAS_STATUS_INVALID_VALUE;
   const bool a_kc = (op_A != HIPBLAS_OP_N);
   const bool b_kc = (op_B == HIPBLAS_OP_N);
-  if (lda < (a_kc ? k : m) || ldb < (b_kc ? k : n) || ldc < m) {
-    if (k != 0) return HIPBLAS_STATUS_INVALID_VALUE;
-  }
+  if (ldc < m) return HIPBLAS_STATUS_INVALID_VALUE;
+  if (k != 0 && (lda < (a_kc ? k : m) || ldb < (b_kc ? k : n))) return HIPBLAS_STATUS_INVALID_VALUE;
+  // a null operand would fault on the device, not fail: refuse it here
+  if (c == nullptr || (k != 0 && (a == nullptr || b == nullptr))) return HIPBLAS_STATUS_INVALID_VALUE;
 
   GemmArgs args{};
   args.m = (uint32_t)m;

@@ -136,6 +136,8 @@ hipblasStatus_t run_long2x2(cuMpSGEMM_handle *h, bool long_is_A, hipblasOperatio
                             uint64_t batch) {
   using E = typename elem_of<T>::type;
   if (h == nullptr || L == 0 || batch == 0 || batch > 65535) return HIPBLAS_STATUS_INVALID_VALUE;
+  if (alpha == nullptr || beta == nullptr || a == nullptr || b == nullptr || c == nullptr)
+    return HIPBLAS_STATUS_INVALID_VALUE; // (a null operand would fault on the device)
   LongArgs<E> args{};
   args.L = L;
   static_assert(sizeof(E) == sizeof(T), "element size");

@@ -178,6 +178,17 @@ def test_invalid_arguments(handle, dev, cg):
     assert handle.gemm(N, N, 8, 8, 8, 1.0, x, 4, x, 8, 0.0, x, 8, cg.FP16TCEC) == cg.STATUS_INVALID_VALUE
     assert handle.gemm(N, N, 8, 8, 8, 1.0, x, 8, x, 8, 0.0, x, 7, cg.FP16TCEC) == cg.STATUS_INVALID_VALUE
     assert handle.gemm(N, N, 0, 8, 8, 1.0, x, 8, x, 8, 0.0, x, 8, cg.FP16TCEC) == cg.STATUS_SUCCESS
+    # null operands are refused on the host (on the device they would fault)
+    assert handle.gemm(N, N, 8, 8, 8, 1.0, 0, 8, x, 8, 0.0, x, 8, cg.FP16TCEC) == cg.STATUS_INVALID_VALUE
+    assert handle.gemm(N, N, 8, 8, 8, 1.0, x, 8, 0, 8, 0.0, x, 8, cg.FP16TCEC) == cg.STATUS_INVALID_VALUE
+    assert handle.gemm(N, N, 8, 8, 8, 1.0, x, 8, x, 8, 0.0, 0, 8, cg.FP16TCEC) == cg.STATUS_INVALID_VALUE
+    assert handle.gemm(N, N, 8, 8, 0, 1.0, 0, 8, 0, 8, 0.0, x, 8, cg.FP16TCEC) == cg.STATUS_SUCCESS   # k = 0 reads neither
+    assert handle.gemm_Mx2x2(N, N, 16, 1.0, 0, 16, x, 2, 0.0, x, 16) == cg.STATUS_INVALID_VALUE
+    before = handle.get_current_exp_stats_buffer_id()
+    sid = handle.exp_max_ext(8, 8, 0, 8)              # logged, nothing launched; the ring still advances
+    assert sid != before
+    handle.scale_A(1, 1, 8, 8, 0, 8)
+    assert not dev.down(x).any()
 
 
 # ---- persistent (tile-walking) kernels -----------------------------------------
