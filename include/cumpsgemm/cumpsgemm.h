@@ -50,7 +50,11 @@ cuMpSGEMM_get_compute_mode(const char *func_name, hipblasHandle_t hipblas_handle
 
 /* reference cumpsgemm.h:23-30 (src/cumpsgemm.cu:549-563).
  * compute_mode in {FP16TCEC, TF32TCEC, FP16TC, TF32TC, AUTO}; any other value
- * returns HIPBLAS_STATUS_INVALID_VALUE (the reference has undefined behaviour).
+ * returns HIPBLAS_STATUS_INVALID_VALUE (the reference has undefined behaviour),
+ * and so do a null handle, scalar or operand pointer, a leading dimension
+ * smaller than the stored rows, and sizes beyond 2^31 - 1 (the reference
+ * returns success for everything, src/cumpsgemm.cu:418).  m, n or batch 0 is a
+ * successful no-op; k = 0 computes C = beta * C and reads neither A nor B.
  * op C is accepted for real data and means T (reference asserts). */
 hipblasStatus_t cuMpSGEMM_sgemm(cuMpSGEMM_handle_t handle,
                                 hipblasOperation_t op_A, hipblasOperation_t op_B,
