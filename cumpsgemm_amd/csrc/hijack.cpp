@@ -36,7 +36,30 @@ int current_device() {
   }
   return (d >= 0 && d < kMaxDevices) ? d : 0;
 }
-std::string g_last_called;
+// Record of the last intercepted call; its text form is only made when somebody
+// asks for it (an intercepted call that is forwarded must stay cheap).
+struct LastCall {
+  bool from_call = false;
+  const char *func_name = "";
+  hipblasOperation_t op_A = HIPBLAS_OP_N, op_B = HIPBLAS_OP_N;
+  int m = 0, n = 0, k = 0, batch = 1;
+  cuMpSGEMM_compute_mode_t mode = CUMPSGEMM_CUBLAS;
+  std::string text; // set through the control API, or cached
+} g_last;
+const char *op_str(hipblasOperation_t op);
+const std::string &last_called_text() {
+  if (g_last.from_call) {
+    g_last.text = std::string(g_last.func_name) + "," + op_str(g_last.op_A) + "," + op_str(g_last.op_B) + "," +
+                  std::to_string(g_last.m) + "," + std::to_string(g_last.n) + "," + std::to_string(g_last.k) +
+                  "," + std::to_string(g_last.batch) + "," + cuMpSGEMM_get_compute_mode_string(g_last.mode);
+    g_last.from_call = false;
+  }
+  return g_last.text;
+}
+void set_last_called_text(const std::string &s) {
+  g_last.from_call = false;
+  g_last.text = s;
+}
 bool g_mx2x2_enabled = false;
 bool g_restore_AB = true;
 cumpsgemm::hijack_control::control_function_t g_control_func;
@@ -259,16 +282,23 @@ hipblasStatus_t hijack_core(const char *func_name, hipblasHandle_t hb, hipblasOp
   // a dry run only logs: it must not need a device, so the handle is created after it
   cuMpSGEMM_handle_t h = (mode == CUMPSGEMM_DRY_RUN) ? g_handles[current_device()] : global_handle();
 
-  log_info(std::string(func_name) + " op=(" + op_str(op_A) + ", " + op_str(op_B) + "), shape=(" +
-           std::to_string(m) + ", " + std::to_string(n) + ", " + std::to_string(k) + ")" +
-           (batched ? ", batch=" + std::to_string(batch) : std::string()) +
-           ", mode=" + cuMpSGEMM_get_compute_mode_string(mode) + "[" +
-           (g_hijack_mode == DYNAMIC_MODE ? "dynamic" : "static") +
-           "][exp_stats:" + ((h && h->exp_stats_enabled) ? "1" : "0") + "]");
-  g_last_called = std::string(func_name) + "," + op_str(op_A) + "," + op_str(op_B) + "," +
-                  std::to_string(m) + "," + std::to_string(n) + "," + std::to_string(k) + "," +
-                  std::to_string(batched ? batch : 1) + "," +
-                  cuMpSGEMM_get_compute_mode_string(mode);
+  if (env_flag("CUMPSGEMM_INFO", false)) {
+    log_info(std::string(func_name) + " op=(" + op_str(op_A) + ", " + op_str(op_B) + "), shape=(" +
+             std::to_string(m) + ", " + std::to_string(n) + ", " + std::to_string(k) + ")" +
+             (batched ? ", batch=" + std::to_string(batch) : std::string()) +
+             ", mode=" + cuMpSGEMM_get_compute_mode_string(mode) + "[" +
+             (g_hijack_mode == DYNAMIC_MODE ? "dynamic" : "static") +
+             "][exp_stats:" + ((h && h->exp_stats_enabled) ? "1" : "0") + "]");
+  }
+  g_last.from_call = true;
+  g_last.func_name = func_name;
+  g_last.op_A = op_A;
+  g_last.op_B = op_B;
+  g_last.m = m;
+  g_last.n = n;
+  g_last.k = k;
+  g_last.batch = batched ? batch : 1;
+  g_last.mode = mode;
 
   if (mode == CUMPSGEMM_DRY_RUN) return HIPBLAS_STATUS_SUCCESS;
   if (h == nullptr) return HIPBLAS_STATUS_NOT_INITIALIZED;
@@ -483,9 +513,9 @@ void disable_restoring_AB_after_scaling() {
   g_restore_AB = false;
   log_info(std::string("AUTO config: restore_AB_scaling=False @") + __func__);
 }
-std::string get_last_called_function_str() { return g_last_called; }
-void set_last_called_function_str(const std::string func_str) { g_last_called = func_str; }
-void clear_last_called_function_str() { g_last_called.clear(); }
+std::string get_last_called_function_str() { return last_called_text(); }
+void set_last_called_function_str(const std::string func_str) { set_last_called_text(func_str); }
+void clear_last_called_function_str() { set_last_called_text(std::string()); }
 bool is_library_loaded() { return true; }
 void set_control_function(const control_function_t control_function) {
   g_control_func = control_function;
@@ -510,14 +540,14 @@ void cuMpSGEMM_hijack_disable_custom_gemm_Mx2x2(void) { g_mx2x2_enabled = false;
 void cuMpSGEMM_hijack_set_restore_AB(int enable) { g_restore_AB = enable != 0; }
 size_t cuMpSGEMM_hijack_get_last_called_function_str(char *buf, size_t buf_len) {
   if (buf != nullptr && buf_len > 0) {
-    std::snprintf(buf, buf_len, "%s", g_last_called.c_str());
+    std::snprintf(buf, buf_len, "%s", last_called_text().c_str());
   }
-  return g_last_called.size();
+  return last_called_text().size();
 }
-void cuMpSGEMM_hijack_clear_last_called_function_str(void) { g_last_called.clear(); }
+void cuMpSGEMM_hijack_clear_last_called_function_str(void) { set_last_called_text(std::string()); }
 int cuMpSGEMM_hijack_is_library_loaded(void) { return 1; }
 void cuMpSGEMM_hijack_set_last_called_function_str(const char *str) {
-  g_last_called = (str != nullptr) ? str : "";
+  set_last_called_text((str != nullptr) ? str : "");
 }
 void cuMpSGEMM_hijack_reset_exp_stats_buffer_id(void) {
   cumpsgemm::hijack_control::reset_exp_stats_buffer_id();
