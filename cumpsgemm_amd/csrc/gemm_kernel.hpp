@@ -99,6 +99,7 @@ struct GemmArgs {
   uint32_t tiles_m, tiles_n;
   uint32_t batch;      // persistent kernels walk (tile, batch) pairs themselves
   uint32_t atomic_out; // split-K: C += alpha*acc with float atomics
+  uint32_t raster_group; // tile rows per column group of the tile order (0: 8)
   // AUTO mode: device flag consulted before doing any work.  The kernel runs
   // only if ((1u << (flag & 31)) & flag_accept_mask) != 0.
   const int *launch_flag;
@@ -311,7 +312,7 @@ __device__ inline void block_sync_lds() {
 // share that XCD's L2, (b) tiles are walked in column groups of GROUP tile
 // rows so that the A rows / B columns in flight stay small.
 __device__ inline void map_tile(uint32_t bid, uint32_t tiles_m, uint32_t tiles_n,
-                                uint32_t &tm, uint32_t &tn) {
+                                uint32_t &tm, uint32_t &tn, const uint32_t GROUP = 8) {
   const uint32_t total = tiles_m * tiles_n;
   constexpr uint32_t NXCD = 8;
   uint32_t id = bid;
@@ -321,7 +322,6 @@ __device__ inline void map_tile(uint32_t bid, uint32_t tiles_m, uint32_t tiles_n
     // XCD x owns a contiguous range; the first r XCDs own one tile more
     id = xcd * q + (xcd < r ? xcd : r) + loc;
   }
-  constexpr uint32_t GROUP = 8;
   const uint32_t per_group = GROUP * tiles_n;
   const uint32_t g = id / per_group;
   const uint32_t first_m = g * GROUP;
@@ -638,7 +638,7 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
   if constexpr (Cfg::PERSIST) {
     map_tile_batched(blockIdx.x, args.tiles_m, args.tiles_n, args.batch, tile_m, tile_n, tile_b);
   } else {
-    map_tile(blockIdx.x, args.tiles_m, args.tiles_n, tile_m, tile_n);
+    map_tile(blockIdx.x, args.tiles_m, args.tiles_n, tile_m, tile_n, args.raster_group ? args.raster_group : 8u);
   }
   const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
   // A tile that sticks out over the edge of C is computed from an origin moved
