@@ -392,11 +392,8 @@ PreSplit run_pre_split(cuMpSGEMM_handle *h, const GemmArgs &args, bool a_kc, boo
     // best (the in-loop kernels keep 8); measured + 1 - 4 % over 8 for every
     // pre-split kernel, except that the fp16 one runs best with 2 from
     // K = 8192 on (12288^2 x 8192: 391 with 2, 384 with 4, 377 TFLOP/s with 8).
-    pargs.raster_group = (kind == PackKind::FP16_REAL && k >= 8192) ? 2u : 4u;
-    if (const char *g = std::getenv("CUMPSGEMM_RASTER_GROUP")) { // experiments
-      const int v = std::atoi(g);
-      if (v >= 1 && v <= 64) pargs.raster_group = (uint32_t)v;
-    }
+    // (args.raster_group != 0: set by CUMPSGEMM_RASTER_GROUP)
+    if (args.raster_group == 0) pargs.raster_group = (kind == PackKind::FP16_REAL && k >= 8192) ? 2u : 4u;
     pargs.launch_flag = gate;
     pargs.flag_accept_mask = accept;
     const uint64_t total = (uint64_t)pargs.tiles_m * pargs.tiles_n;
@@ -489,6 +486,10 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
   scalar_parts<T>::get(beta, args.beta_re, args.beta_im);
   args.conj_a = (CPLX && op_A == HIPBLAS_OP_C) ? 1u : 0u;
   args.conj_b = (CPLX && op_B == HIPBLAS_OP_C) ? 1u : 0u;
+  if (const char *g = std::getenv("CUMPSGEMM_RASTER_GROUP")) { // experiments: tile order of the one-tile kernels
+    const int v = std::atoi(g);
+    if (v >= 1 && v <= 64) args.raster_group = (uint32_t)v;
+  }
 
   // which kernels to launch: one for a fixed mode; for AUTO both candidates,
   // each gated on the device flag so that no host synchronisation is needed
