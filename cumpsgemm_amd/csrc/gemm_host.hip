@@ -667,6 +667,27 @@ hipblasStatus_t cumpsgemm::gemm_stridedBatch(
     const T *b_dmem_ptr, uint64_t ldb, uint64_t strideb, const T *beta, T *c_dmem_ptr,
     uint64_t ldc, uint64_t stridec, uint64_t batch_count, cuMpSGEMM_compute_mode_t compute_mode,
     unsigned *used_kernel_module_id) {
+  // A few large matrices: each is worth the pre-split path on its own (which
+  // handles one matrix at a time), so they are issued one by one, like the
+  // reference does for large batches (src/cumpsgemm.cu:431-439).
+  if (handle != nullptr && batch_count > 1 && batch_count <= 1024 && m <= 0x7fffffffull && n <= 0x7fffffffull &&
+      k <= 0x7fffffffull) {
+    constexpr bool CPLX = std::is_same<T, hipComplex>::value;
+    int force_cls = -1, force_split = 0;
+    if (const char *f = std::getenv("CUMPSGEMM_FORCE_TILE_CLASS")) force_cls = std::atoi(f);
+    if (const char *f = std::getenv("CUMPSGEMM_FORCE_KSPLIT")) force_split = std::atoi(f);
+    const PreSplitChoice ch = choose_pre_split<CPLX>(handle, op_A != HIPBLAS_OP_N, op_B == HIPBLAS_OP_N, m, n, k, 1,
+                                                     compute_mode, force_cls, force_split, 0);
+    if (ch.take) {
+      hipblasStatus_t st1 = HIPBLAS_STATUS_SUCCESS;
+      for (uint64_t i = 0; i < batch_count && st1 == HIPBLAS_STATUS_SUCCESS; i++) {
+        st1 = run_gemm<T>(handle, op_A, op_B, m, n, k, alpha, a_dmem_ptr + i * stridea, lda, 0,
+                          b_dmem_ptr + i * strideb, ldb, 0, beta, c_dmem_ptr + i * stridec, ldc, 0, 1,
+                          compute_mode, used_kernel_module_id, "batched_gemm_kernel");
+      }
+      return st1;
+    }
+  }
   // batches beyond the grid's y limit are issued in slices
   uint64_t done = 0;
   hipblasStatus_t st = HIPBLAS_STATUS_SUCCESS;

@@ -353,6 +353,58 @@ def test_complex_packed_path_matches_in_loop_split(O, handle, dev, monkeypatch, 
         assert np.array_equal(outs[0].reshape(n, ldc)[:, m:], c0.reshape(n, ldc)[:, m:])
 
 
+@pytest.mark.parametrize("cplx,opa,opb,m,n,k,batch", [
+    (False, N, T, 3700, 3700, 320, 3),      # both operands M/N-contiguous: pre-split from K = 256 on
+    (True, N, N, 3072, 3072, 1024, 2),
+])
+def test_batch_of_large_matrices_takes_the_pre_split_path_one_by_one(cg, torch_gpu, monkeypatch, cplx, opa, opb,
+                                                                     m, n, k, batch):
+    """A strided batch whose matrices are each worth the pre-split path is issued matrix by
+    matrix through it; same bits as the batched in-loop kernels."""
+    torch = torch_gpu
+    dev_t = torch.device("cuda:0")
+    es = 2 if cplx else 1
+    h = cg.Handle()
+    h.set_stream(torch.cuda.current_stream())
+    try:
+        g = torch.Generator(device=dev_t).manual_seed(123)
+        sa, sb, sc = m * k + 64, k * n + 32, m * n + 16      # gaps between the matrices
+        a = torch.rand(sa * batch * es, generator=g, device=dev_t) - 0.5
+        b = torch.rand(sb * batch * es, generator=g, device=dev_t) - 0.5
+        c0 = torch.rand(sc * batch * es, generator=g, device=dev_t) - 0.5
+        lda = m                                   # op N: m x k
+        ldb = n if opb == T else k
+        outs = {}
+        for packed in ("0", None):
+            if packed is None:
+                monkeypatch.delenv("CUMPSGEMM_PACKED", raising=False)
+            else:
+                monkeypatch.setenv("CUMPSGEMM_PACKED", packed)
+            c = c0.clone()
+            st = h.gemm_strided_batch(opa, opb, m, n, k, 1.5, a, lda, sa, b, ldb, sb, -0.5, c, m, sc, batch,
+                                      FP16TCEC, cplx=cplx)
+            torch.cuda.synchronize()
+            assert st == 0
+            assert (h.workspace_size() > 0) == (packed is None)
+            outs[packed] = c
+        assert torch.equal(outs["0"].view(torch.int32), outs[None].view(torch.int32))
+        # ... and right: the last matrix against FP64
+        i = batch - 1
+        dt = torch.complex128 if cplx else torch.float64
+        def mat(buf, off, rows, cols):
+            x = buf[off * es:(off + rows * cols) * es].double()
+            x = torch.view_as_complex(x.view(-1, 2)) if cplx else x
+            return x.view(cols, rows).t()                                # column-major rows x cols
+        A = mat(a, i * sa, m, k)
+        B = mat(b, i * sb, n, k).t() if opb == T else mat(b, i * sb, k, n)
+        ref = 1.5 * (A @ B) - 0.5 * mat(c0, i * sc, m, n)
+        got = mat(outs[None], i * sc, m, n)
+        assert (torch.linalg.norm(got - ref) / torch.linalg.norm(ref)).item() < 4 * 2.0 ** -23 * k ** 0.5
+    finally:
+        torch.cuda.synchronize()
+        h.close()
+
+
 @pytest.mark.parametrize("mode,cplx", [(FP16TCEC, False), (TF32TCEC, False), (FP16TCEC, True)])
 def test_packed_kernels_walk_and_one_tile_forms_agree(handle, dev, monkeypatch, mode, cplx):
     """The pre-split kernels exist as persistent (tile-walking) and one-tile-per-workgroup
