@@ -278,7 +278,8 @@ PreSplitChoice choose_pre_split(const cuMpSGEMM_handle *h, bool a_kc, bool b_kc,
   const bool shape_ok = batch == 1 && k >= 128 &&
                         (uint64_t)m * n >= (uint64_t)h->num_cus * ch.bm * ch.bn && k / 32 < 65535;
   const double mn_ratio = (double)m * (double)n / ((double)m + (double)n);
-  const bool pays_nt = !a_kc && !b_kc && k >= 256 && mn_ratio >= 1800.0;
+  // (K = 256: 6144^2 + 8 %, 4096^2 - 4 %)
+  const bool pays_nt = !a_kc && !b_kc && ((k >= 512 && mn_ratio >= 1800.0) || (k >= 256 && mn_ratio >= 2800.0));
   // Every other layout: the pre-split kernel, freed of the split arithmetic,
   // outruns the in-loop one by more than the pre-pass costs once the problem
   // is large (8192^3: 381 vs 361 - 372 TFLOP/s; 8192^2 x 1024: 351 vs 318 -

@@ -354,7 +354,7 @@ def test_complex_packed_path_matches_in_loop_split(O, handle, dev, monkeypatch, 
 
 
 @pytest.mark.parametrize("cplx,opa,opb,m,n,k,batch", [
-    (False, N, T, 3700, 3700, 320, 3),      # both operands M/N-contiguous: pre-split from K = 256 on
+    (False, N, T, 3700, 3700, 512, 3),      # both operands M/N-contiguous: pre-split from K = 512 on
     (True, N, N, 3072, 3072, 1024, 2),
 ])
 def test_batch_of_large_matrices_takes_the_pre_split_path_one_by_one(cg, torch_gpu, monkeypatch, cplx, opa, opb,
