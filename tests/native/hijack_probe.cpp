@@ -142,6 +142,37 @@ int main(int argc, char **argv) {
       den += std::norm(ref);
     }
     report("hipblasCgemm_CN", st, num, den);
+
+    // the other complex entry points: batches of nc x nc matrices, stride nc * nc
+    const long long cs = (long long)nc * nc;
+    auto check_cplx = [&](const char *name, hipblasStatus_t status, int nb) {
+      CHECK_HIP(hipMemcpyAsync(hc.data(), dc.p, (size_t)cs * nb * 8, hipMemcpyDeviceToHost, stream));
+      CHECK_HIP(hipStreamSynchronize(stream));
+      double nu = 0, de = 0;
+      for (int t = 0; t < nb; t++)
+        for (int s = 0; s < 300; s++) {
+          const int i = (int)(mix(s * 2 + 51) % nc), j = (int)(mix(s * 2 + 52) % nc);
+          std::complex<double> ref = 0;
+          for (int p = 0; p < nc; p++)
+            ref += std::complex<double>(A[t * cs + i + (size_t)p * nc]) * std::complex<double>(B[t * cs + p + (size_t)j * nc]);
+          nu += std::norm(ref - std::complex<double>(Cc[t * cs + i + (size_t)j * nc]));
+          de += std::norm(ref);
+        }
+      report(name, status, nu, de);
+    };
+    CHECK_HIP(hipMemsetAsync(dc.p, 0, e * batch * 4, stream));
+    st = hipblasCgemmStridedBatched(hb, HIPBLAS_OP_N, HIPBLAS_OP_N, nc, nc, nc, &cone, ca, nc, cs, cb, nc, cs, &czero,
+                                    cc, nc, cs, 2);
+    check_cplx("hipblasCgemmStridedBatched", st, 2);
+    CHECK_HIP(hipMemsetAsync(dc.p, 0, e * batch * 4, stream));
+    st = hipblasGemmEx(hb, HIPBLAS_OP_N, HIPBLAS_OP_N, nc, nc, nc, &cone, ca, HIP_C_32F, nc, cb, HIP_C_32F, nc, &czero,
+                       cc, HIP_C_32F, nc, HIPBLAS_COMPUTE_32F, HIPBLAS_GEMM_DEFAULT);
+    check_cplx("hipblasGemmEx_c32", st, 1);
+    CHECK_HIP(hipMemsetAsync(dc.p, 0, e * batch * 4, stream));
+    st = hipblasGemmStridedBatchedEx(hb, HIPBLAS_OP_N, HIPBLAS_OP_N, nc, nc, nc, &cone, ca, HIP_C_32F, nc, cs, cb,
+                                     HIP_C_32F, nc, cs, &czero, cc, HIP_C_32F, nc, cs, 2, HIPBLAS_COMPUTE_32F,
+                                     HIPBLAS_GEMM_DEFAULT);
+    check_cplx("hipblasGemmStridedBatchedEx_c32", st, 2);
   }
 
   // a non-FP32 GemmEx must go to hipBLAS untouched whatever the mode

@@ -111,3 +111,21 @@ def test_host_threads_with_their_own_streams_share_the_interposer():
     workspace): every result equals the one computed alone."""
     res, _ = _probe({"CUMPSGEMM_COMPUTE_MODE": "FP16TCEC", "PROBE_THREADS": "4", "PROBE_N": "4096"})
     assert res["threads"] == (0, 0.0)
+
+
+CPLX_CALLS = ["hipblasCgemm_CN", "hipblasCgemmStridedBatched", "hipblasGemmEx_c32", "hipblasGemmStridedBatchedEx_c32"]
+
+
+def test_complex_entry_points_reach_the_tcec_kernels():
+    """With 1100 x 1100 complex matrices (every dimension above the default rule's 1024) the four
+    complex entry points are served by this library and keep complex64 accuracy."""
+    base, _ = _probe({"PROBE_N": "2200"}, preload=False)
+    res, logs = _probe({"CUMPSGEMM_COMPUTE_MODE": "FP16TCEC", "CUMPSGEMM_INFO": "1", "PROBE_N": "2200"})
+    text = "\n".join(logs)
+    for name in CPLX_CALLS:
+        assert res[name][0] == 0 and base[name][0] == 0
+        assert res[name][1] <= 2.0 * base[name][1] + 1e-9 and res[name][1] < 2.0 ** -23 * 1100 ** 0.5, (name, res[name])
+    assert "hipblasCgemm op=(C, N), shape=(1100, 1100, 1100), mode=FP16TCEC" in text
+    assert "hipblasCgemmStridedBatched op=(N, N), shape=(1100, 1100, 1100), batch=2, mode=FP16TCEC" in text
+    assert text.count("hipblasGemmEx op=(N, N), shape=(1100, 1100, 1100), mode=FP16TCEC") == 1
+    assert "hipblasGemmStridedBatchedEx op=(N, N), shape=(1100, 1100, 1100), batch=2, mode=FP16TCEC" in text
