@@ -194,6 +194,45 @@ int main(int argc, char **argv) {
     report("hipblasGemmEx_f16_in", st, num, den);
   }
 
+  // ---- gate-application shapes: (2^18 x 2) = (2^18 x 2) * (2 x 2) and its transpose-side twin ----
+  if (std::getenv("PROBE_MX2X2") != nullptr) {
+    const int L = 1 << 18;
+    const hipComplex cone = make_hipComplex(1.f, 0.f), czero = make_hipComplex(0.f, 0.f);
+    const hipComplex *ca = reinterpret_cast<const hipComplex *>(da.p); // L x 2 complex, ld L
+    const hipComplex *cb = reinterpret_cast<const hipComplex *>(db.p); // 2 x 2 complex, ld 2
+    hipComplex *cc = reinterpret_cast<hipComplex *>(dc.p);
+    auto A = reinterpret_cast<const std::complex<float> *>(ha.data());
+    auto B = reinterpret_cast<const std::complex<float> *>(hb_.data());
+    auto Cc = reinterpret_cast<const std::complex<float> *>(hc.data());
+    CHECK_HIP(hipMemsetAsync(dc.p, 0, (size_t)L * 2 * 8, stream));
+    st = hipblasCgemm(hb, HIPBLAS_OP_N, HIPBLAS_OP_N, L, 2, 2, &cone, ca, L, cb, 2, &czero, cc, L);
+    CHECK_HIP(hipMemcpyAsync(hc.data(), dc.p, (size_t)L * 2 * 8, hipMemcpyDeviceToHost, stream));
+    CHECK_HIP(hipStreamSynchronize(stream));
+    double num = 0, den = 0;
+    for (int j = 0; j < 2; j++)
+      for (int i = 0; i < L; i += 7) {
+        const std::complex<double> ref = std::complex<double>(A[i]) * std::complex<double>(B[2 * j]) +
+                                         std::complex<double>(A[i + L]) * std::complex<double>(B[2 * j + 1]);
+        num += std::norm(ref - std::complex<double>(Cc[i + (size_t)j * L]));
+        den += std::norm(ref);
+      }
+    report("cgemm_Mx2x2", st, num, den);
+    // real, (2 x L) = (2 x 2) * (2 x L)
+    CHECK_HIP(hipMemsetAsync(dc.p, 0, (size_t)L * 2 * 4, stream));
+    st = hipblasSgemm(hb, HIPBLAS_OP_N, HIPBLAS_OP_N, 2, L, 2, &one, da.p, 2, db.p, 2, &zero, dc.p, 2);
+    CHECK_HIP(hipMemcpyAsync(hc.data(), dc.p, (size_t)L * 2 * 4, hipMemcpyDeviceToHost, stream));
+    CHECK_HIP(hipStreamSynchronize(stream));
+    num = den = 0;
+    for (int j = 0; j < L; j += 5)
+      for (int i = 0; i < 2; i++) {
+        const double ref = (double)ha[i] * hb_[2 * (size_t)j] + (double)ha[i + 2] * hb_[2 * (size_t)j + 1];
+        const double d = ref - (double)hc[i + 2 * (size_t)j];
+        num += d * d;
+        den += ref * ref;
+      }
+    report("sgemm_2xNx2", st, num, den);
+  }
+
   // ---- several host threads, each with its own hipBLAS handle and stream ----
   // (PROBE_THREADS=<count>: every thread repeats two products of different
   // shapes and compares each result with the one the main thread computed)

@@ -129,3 +129,18 @@ def test_complex_entry_points_reach_the_tcec_kernels():
     assert "hipblasCgemmStridedBatched op=(N, N), shape=(1100, 1100, 1100), batch=2, mode=FP16TCEC" in text
     assert text.count("hipblasGemmEx op=(N, N), shape=(1100, 1100, 1100), mode=FP16TCEC") == 1
     assert "hipblasGemmStridedBatchedEx op=(N, N), shape=(1100, 1100, 1100), batch=2, mode=FP16TCEC" in text
+
+
+def test_gate_shapes_take_the_streaming_kernels_when_enabled():
+    """M x 2 x 2 and 2 x N x 2 products (M, N powers of two) go to the dedicated streaming kernels
+    when CUMPSGEMM_CUSTOM_GEMM_MX2X2 is set (reference src/cumpsgemm_cublas.cu:269-338), whatever
+    the compute mode; otherwise the rule decides (small dimensions: hipBLAS)."""
+    res, logs = _probe({"CUMPSGEMM_CUSTOM_GEMM_MX2X2": "1", "CUMPSGEMM_INFO": "1", "PROBE_MX2X2": "1"})
+    text = "\n".join(logs)
+    assert res["cgemm_Mx2x2"][0] == 0 and res["cgemm_Mx2x2"][1] < 2e-7
+    assert res["sgemm_2xNx2"][0] == 0 and res["sgemm_2xNx2"][1] < 2e-7
+    assert " +---> gemm_Mx2x2" in text and " +---> gemm_2xNx2" in text
+    res, logs = _probe({"CUMPSGEMM_INFO": "1", "PROBE_MX2X2": "1"})
+    text = "\n".join(logs)
+    assert res["cgemm_Mx2x2"][0] == 0 and res["cgemm_Mx2x2"][1] < 2e-7 and res["sgemm_2xNx2"][1] < 2e-7
+    assert "gemm_Mx2x2" not in text and "shape=(262144, 2, 2), mode=CUBLAS_SIMT" in text
