@@ -78,6 +78,36 @@ torch.cuda.synchronize()
 print("RESULT ctl_small -", "%.3e" % rel(t, a[:256, :256].double() @ b[:256, :256].double()),
       ctl.get_last_called_function_str(), flush=True)
 ctl.unset_control_function()
+
+# statistics of the result of forwarded calls, switched on through the library's own handle
+# (reference src/cumpsgemm_cublas.cu:420-425; hijack_control.hpp get_internal_global_handle)
+import ctypes
+P = ctypes.CDLL(None)
+P.cuMpSGEMM_hijack_get_internal_global_handle.restype = ctypes.c_void_p
+hd = ctypes.c_void_p(P.cuMpSGEMM_hijack_get_internal_global_handle())
+P.cuMpSGEMM_enable_exp_stats.argtypes = [ctypes.c_void_p]
+P.cuMpSGEMM_disable_exp_stats.argtypes = [ctypes.c_void_p]
+P.cuMpSGEMM_get_current_exp_stats_buffer_id.argtypes = [ctypes.c_void_p]
+P.cuMpSGEMM_get_current_exp_stats_buffer_id.restype = ctypes.c_uint
+P.cuMpSGEMM_get_exp_stats.argtypes = [ctypes.c_void_p, ctypes.c_uint, ctypes.POINTER(ctypes.c_uint64),
+                                      ctypes.POINTER(ctypes.c_uint64)]
+P.cuMpSGEMM_get_max_exp.argtypes = [ctypes.c_void_p, ctypes.c_uint]
+P.cuMpSGEMM_get_max_exp.restype = ctypes.c_float
+P.cuMpSGEMM_enable_exp_stats(hd)
+ctl.set_compute_mode(ctl.CUMPSGEMM_CUBLAS)
+before = P.cuMpSGEMM_get_current_exp_stats_buffer_id(hd)
+c = a @ b
+torch.cuda.synchronize()
+after = P.cuMpSGEMM_get_current_exp_stats_buffer_id(hd)
+u, t = ctypes.c_uint64(0), ctypes.c_uint64(0)
+P.cuMpSGEMM_get_exp_stats(hd, after, ctypes.byref(u), ctypes.byref(t))
+mx = P.cuMpSGEMM_get_max_exp(hd, after)
+want_max = 2.0 ** torch.floor(torch.log2(c.abs().max())).item()
+small = int((c.abs() < 2.0 ** -15).sum().item())
+if small > 0:   # zero tolerance: the second pass recounts against 2^-16 x the maximum exponent
+    small = int((c.abs() < 2.0 ** -16 * want_max).sum().item())
+print("RESULT cstats -", "%.3e" % 0.0, "%d %d %d %d %d %g %g" % (before, after, u.value, t.value, small, mx, want_max), flush=True)
+P.cuMpSGEMM_disable_exp_stats(hd)
 '''
 
 
@@ -126,3 +156,8 @@ def test_torch_matmul_is_served_by_the_preloaded_library(cg, torch_gpu):
     err, last = res[("ctl_small", "-")]
     assert err < 3e-6 and last == "hipblasSgemm,N,N,256,256,256,1,CUBLAS", out
     assert "[cuMpSGEMM LOG] hipblasSgemm op=(N, N), shape=(1536, 1536, 1536), mode=FP16TCEC[static]" in out, out
+    # statistics of C after a forwarded call: one new slot, every element counted, the small ones found
+    before, after, under, total, small, mx, want_max = res[("cstats", "-")][1].split()
+    assert int(after) == int(before) + 1 and int(total) == 1536 * 1536 and int(under) == int(small)
+    assert float(mx) == float(want_max)
+    assert "mode=CUBLAS[static][exp_stats:1]" in out, out
