@@ -183,8 +183,10 @@ __global__ __launch_bounds__(kBlock) void exp_stats_kernel(const StatsJob job0, 
   if (!s_last) return;
 
   // last workgroup: fold all partials (device-scope loads, independent of each
-  // other so that they are all in flight together)
-  __threadfence();
+  // other so that they are all in flight together).  No fence is needed: every
+  // partial was acknowledged by memory before its workgroup took a ticket, the
+  // last ticket was taken before the barrier above, and device-scope loads do
+  // not look at this XCD's L2.
   unsigned mxb = 0;
   unsigned long long t = 0, u = 0;
   for (unsigned i = tid; i < nblocks; i += kBlock) {
@@ -246,8 +248,8 @@ __global__ __launch_bounds__(kBlock) void exp_stats_kernel(const StatsJob job0, 
       slot->max_exp_bits = mxb;
     }
     // ready for the next pass on this stream
+    // (the slot and the ticket become visible to later kernels at the end of this one)
     __hip_atomic_store(ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __threadfence();
   }
 }
 
