@@ -94,6 +94,10 @@ def _declare(L):
                                      sp, _ptr, _u64, _u64, _u64]
     L.cuMpSGEMM_get_workspace_size.argtypes = [_ptr]
     L.cuMpSGEMM_get_workspace_size.restype = ctypes.c_size_t
+    L.cuMpSGEMM_get_workspace_pointer.argtypes = [_ptr]
+    L.cuMpSGEMM_get_workspace_pointer.restype = _ptr
+    L.cuMpSGEMM_reload_tuning_env.argtypes = []
+    L.cuMpSGEMM_reload_tuning_env.restype = None
     L.cuMpSGEMM_describe_tile_config.argtypes = [_int, _int, _int, _int, _int, ctypes.c_char_p, ctypes.c_size_t]
     stats_args = [_ptr, _u32, _u32, _ptr, _u32, _u32, _u32]
     for name in ("cuMpSGEMM_exp_stats_ext_s", "cuMpSGEMM_exp_stats_ext_c",
@@ -207,6 +211,10 @@ class Handle:
     def workspace_size(self):
         """Bytes of device memory held for pre-split operands."""
         return self._L.cuMpSGEMM_get_workspace_size(self._h)
+
+    def workspace_pointer(self):
+        """Device address of that workspace (0 until it exists)."""
+        return self._L.cuMpSGEMM_get_workspace_pointer(self._h) or 0
 
     # ---- GEMM ----
     def gemm(self, op_a, op_b, m, n, k, alpha, a, lda, b, ldb, beta, c, ldc, mode, cplx=False,

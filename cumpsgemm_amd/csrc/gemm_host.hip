@@ -7,11 +7,42 @@
 #include "utils.hpp"
 #include <cumpsgemm/cumpsgemm.hpp>
 #include <cumpsgemm/cumpsgemm_ext.h>
+#include <mutex>
 #include <new>
 #include <stdexcept>
 #include <type_traits>
 
 namespace cumpsgemm_amd {
+
+namespace {
+Tuning read_tuning_env() {
+  Tuning t;
+  auto as_int = [](const char *name, int unset) {
+    const char *v = std::getenv(name);
+    return v != nullptr ? std::atoi(v) : unset;
+  };
+  if (const char *v = std::getenv("CUMPSGEMM_PACKED")) t.packed = v[0] == '0' ? 0 : (v[0] == '1' ? 1 : -1);
+  if (const char *v = std::getenv("CUMPSGEMM_PACKED_WALK")) t.packed_walk = v[0] == '1' ? 1 : 0;
+  const int rg = as_int("CUMPSGEMM_RASTER_GROUP", 0);
+  t.raster_group = (rg >= 1 && rg <= 64) ? rg : 0;
+  t.force_cls = as_int("CUMPSGEMM_FORCE_TILE_CLASS", -1);
+  if (t.force_cls < 0 || t.force_cls >= kNumTileClasses) t.force_cls = -1;
+  t.force_split = as_int("CUMPSGEMM_FORCE_KSPLIT", 0);
+  t.no_persistent = std::getenv("CUMPSGEMM_NO_PERSISTENT") != nullptr;
+  t.no_column_split = std::getenv("CUMPSGEMM_NO_COLUMN_SPLIT") != nullptr;
+  t.no_fused_scaling = std::getenv("CUMPSGEMM_NO_FUSED_SCALING") != nullptr;
+  if (const char *v = std::getenv("CUMPSGEMM_PERSISTENT_MAX_STEPS")) t.persistent_max_steps = (unsigned)std::atoi(v);
+  if (const char *v = std::getenv("CUMPSGEMM_MAX_WORKSPACE_BYTES")) t.max_workspace_bytes = std::strtoull(v, nullptr, 10);
+  return t;
+}
+Tuning g_tuning;
+std::once_flag g_tuning_once;
+} // namespace
+
+const Tuning &tuning() {
+  std::call_once(g_tuning_once, [] { g_tuning = read_tuning_env(); });
+  return g_tuning;
+}
 
 void check_hip(hipError_t err, const char *what) {
   if (err != hipSuccess) {
@@ -195,14 +226,8 @@ Plan make_plan(const cuMpSGEMM_handle *h, Prec p, bool cplx, bool a_kc, bool b_k
 // tile wide and high (edge tiles are computed from an origin moved inwards),
 // every K-chunk a multiple of the 32-wide step and at least four steps long,
 // and every per-thread offset must fit 31 bits.
-constexpr unsigned kPersistentMaxSteps = 32; // K-steps per tile up to which tiles are walked
-unsigned persistent_max_steps() {
-  static const unsigned max_steps = [] {
-    const char *e = std::getenv("CUMPSGEMM_PERSISTENT_MAX_STEPS");
-    return e != nullptr ? (unsigned)std::atoi(e) : kPersistentMaxSteps;
-  }();
-  return max_steps;
-}
+// (K-steps per tile up to which tiles are walked: Tuning::persistent_max_steps, 32)
+unsigned persistent_max_steps() { return tuning().persistent_max_steps; }
 
 template <class T>
 bool persistent_ok(const KernelEntry *e, bool a_kc, bool b_kc, uint64_t m, uint64_t n, uint64_t k,
@@ -266,8 +291,8 @@ PreSplitChoice choose_pre_split(const cuMpSGEMM_handle *h, bool a_kc, bool b_kc,
                                 int force_cls, int force_split, int depth) {
   PreSplitChoice ch;
   if (CPLX && mode != CUMPSGEMM_FP16TCEC) return ch; // (complex: FP16TCEC only, also under FP16TCEC_SCALING)
-  const char *fp = std::getenv("CUMPSGEMM_PACKED"); // "0" never, "1" whenever possible
-  const bool never = fp != nullptr && fp[0] == '0', always = fp != nullptr && fp[0] == '1';
+  // CUMPSGEMM_PACKED: "0" never, "1" whenever possible
+  const bool never = tuning().packed == 0, always = tuning().packed == 1;
   // bf16x3 (explicit TF32TCEC mode): its in-loop three-way split costs 5.4
   // vector instructions per MFMA, so the pre-pass pays for every layout
   ch.bf16 = (mode == CUMPSGEMM_TF32TCEC);
@@ -310,32 +335,45 @@ PreSplitChoice choose_pre_split(const cuMpSGEMM_handle *h, bool a_kc, bool b_kc,
   return ch;
 }
 
-// The handle's workspace only grows.  false: no memory (the caller falls back
-// to the in-loop kernels) or, with *failed set, the stream is broken.
-bool ensure_pack_workspace(cuMpSGEMM_handle *h, uint64_t bytes, bool *failed) {
+// The handle's workspace only grows.  Returns the buffer, or nullptr: no memory
+// or over the cap (the caller falls back to the in-loop kernels) or, with
+// *failed set, the stream is broken.
+void *ensure_pack_workspace(cuMpSGEMM_handle *h, uint64_t bytes, bool *failed) {
   *failed = false;
-  if (h->pack_ws_bytes >= bytes) return h->pack_ws != nullptr;
-  // no allocation or synchronisation while the stream is being captured into a
-  // graph: the call takes the path that needs no workspace instead
   hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
   if (hipStreamIsCapturing(h->stream, &cap) != hipSuccess) (void)hipGetLastError();
-  if (cap != hipStreamCaptureStatusNone) return false;
+  const bool capturing = cap != hipStreamCaptureStatusNone;
+  if (h->pack_ws_bytes >= bytes && h->pack_ws != nullptr) {
+    // a graph being captured now will hold this address for as long as it lives
+    if (capturing) h->pack_ws_captured = true;
+    return h->pack_ws;
+  }
+  if (bytes > tuning().max_workspace_bytes) return nullptr;
+  // no allocation or synchronisation while the stream is being captured into a
+  // graph: the call takes the path that needs no workspace instead
+  if (capturing) return nullptr;
   // the previous workspace may still be in use by work queued on the stream
   if (hipStreamSynchronize(h->stream) != hipSuccess) {
     log_error("stream synchronisation failed before growing the pack workspace");
     *failed = true;
-    return false;
+    return nullptr;
   }
-  if (h->pack_ws != nullptr) (void)hipFree(h->pack_ws);
+  if (h->pack_ws != nullptr) {
+    // a captured graph may replay at any time: its workspace stays until the
+    // handle is destroyed
+    if (h->pack_ws_captured) h->retired_ws.push_back(h->pack_ws);
+    else (void)hipFree(h->pack_ws);
+  }
+  h->pack_ws_captured = false;
   h->pack_ws = nullptr;
   h->pack_ws_bytes = 0;
   if (hipMalloc(&h->pack_ws, bytes) != hipSuccess) {
     (void)hipGetLastError();
     h->pack_ws = nullptr;
-    return false;
+    return nullptr;
   }
   h->pack_ws_bytes = bytes;
-  return true;
+  return h->pack_ws;
 }
 
 // `args`: the call's arguments (scalars, C, conj flags, launch flag); `accept_*`:
@@ -354,10 +392,10 @@ PreSplit run_pre_split(cuMpSGEMM_handle *h, const GemmArgs &args, bool a_kc, boo
   const uint64_t a3_bytes = ch.auto_bf16 ? packed_bytes(mp, k, 3) : 0;
   const uint64_t b3_bytes = ch.auto_bf16 ? packed_bytes(np, k, 3) : 0;
   const uint64_t ws_bytes = a_bytes + b_bytes + a3_bytes + b3_bytes;
-  if (ws_bytes > (16ull << 30) || mp * 64ull >= 0xffffffffull || np * 64ull >= 0xffffffffull)
-    return PreSplit::NOT_TAKEN;
+  if (mp * 64ull >= 0xffffffffull || np * 64ull >= 0xffffffffull) return PreSplit::NOT_TAKEN;
   bool failed = false;
-  if (!ensure_pack_workspace(h, ws_bytes, &failed)) return failed ? PreSplit::FAILED : PreSplit::NOT_TAKEN;
+  void *const ws = ensure_pack_workspace(h, ws_bytes, &failed);
+  if (ws == nullptr) return failed ? PreSplit::FAILED : PreSplit::NOT_TAKEN;
 
   const float *af = reinterpret_cast<const float *>(a), *bf = reinterpret_cast<const float *>(b);
   const int *gate = ch.auto_ok ? args.launch_flag : nullptr;
@@ -402,7 +440,7 @@ PreSplit run_pre_split(cuMpSGEMM_handle *h, const GemmArgs &args, bool a_kc, boo
     // (measured cross-over: 16 K-steps for the fp16 kernel, which gains 6 - 8 % from
     // the one-tile form at 8192^3, the usual 32 for bf16x3, which gains nothing)
     bool walk = walk_short_only ? pargs.k / 32 < 16 : pargs.k / 32 <= persistent_max_steps();
-    if (const char *w = std::getenv("CUMPSGEMM_PACKED_WALK")) walk = w[0] == '1';
+    if (tuning().packed_walk >= 0) walk = tuning().packed_walk == 1;
     const dim3 grid = walk ? dim3((unsigned)std::min<uint64_t>(total, h->num_cus), 1, 1)
                            : dim3((unsigned)total, 1, 1);
     launch_kernel(pargs, grid, walk);
@@ -414,7 +452,7 @@ PreSplit run_pre_split(cuMpSGEMM_handle *h, const GemmArgs &args, bool a_kc, boo
     return true;
   };
 
-  char *pa = static_cast<char *>(h->pack_ws), *pb = pa + a_bytes;
+  char *pa = static_cast<char *>(ws), *pb = pa + a_bytes;
   const uint32_t accept = ch.auto_ok ? accept_fp16 : 0u;
   bool ok;
   if constexpr (CPLX) {
@@ -487,10 +525,7 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
   scalar_parts<T>::get(beta, args.beta_re, args.beta_im);
   args.conj_a = (CPLX && op_A == HIPBLAS_OP_C) ? 1u : 0u;
   args.conj_b = (CPLX && op_B == HIPBLAS_OP_C) ? 1u : 0u;
-  if (const char *g = std::getenv("CUMPSGEMM_RASTER_GROUP")) { // experiments: tile order of the one-tile kernels
-    const int v = std::atoi(g);
-    if (v >= 1 && v <= 64) args.raster_group = (uint32_t)v;
-  }
+  args.raster_group = (uint32_t)tuning().raster_group; // experiments: tile order of the one-tile kernels
 
   // which kernels to launch: one for a fixed mode; for AUTO both candidates,
   // each gated on the device flag so that no host synchronisation is needed
@@ -512,15 +547,9 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
     args.launch_flag = nullptr;
   }
 
-  int force_cls = -1;
-  if (const char *f = std::getenv("CUMPSGEMM_FORCE_TILE_CLASS")) {
-    force_cls = std::atoi(f);
-    if (force_cls < 0 || force_cls >= kNumTileClasses) force_cls = -1;
-  }
-
-  int force_split = 0; // experiments: fix the split-K factor (a power of two)
-  if (const char *f = std::getenv("CUMPSGEMM_FORCE_KSPLIT")) force_split = std::atoi(f);
-  const bool no_persist = std::getenv("CUMPSGEMM_NO_PERSISTENT") != nullptr;
+  const int force_cls = tuning().force_cls;
+  const int force_split = tuning().force_split; // experiments: fix the split-K factor (a power of two)
+  const bool no_persist = tuning().no_persistent;
 
   // the two halves of a column split are timed as one call, by the outer level
   struct ProfilerPause {
@@ -567,7 +596,7 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
   // cut in two: a first part whose tiles fill whole rounds, and the remaining
   // columns, planned on their own (typically with K split to fill the chip).
   if (!split && batch == 1 && depth == 0 && !fp16_served && k >= 256 &&
-      std::getenv("CUMPSGEMM_NO_COLUMN_SPLIT") == nullptr) {
+      !tuning().no_column_split) {
     const KernelEntry *e0 = plan0.entry;
     const uint64_t slots = (uint64_t)h->num_cus * resident_groups(e0);
     const uint64_t tiles = (uint64_t)plan0.tiles_m * plan0.tiles_n;
@@ -674,9 +703,7 @@ hipblasStatus_t cumpsgemm::gemm_stridedBatch(
   if (handle != nullptr && batch_count > 1 && batch_count <= 1024 && m <= 0x7fffffffull && n <= 0x7fffffffull &&
       k <= 0x7fffffffull) {
     constexpr bool CPLX = std::is_same<T, hipComplex>::value;
-    int force_cls = -1, force_split = 0;
-    if (const char *f = std::getenv("CUMPSGEMM_FORCE_TILE_CLASS")) force_cls = std::atoi(f);
-    if (const char *f = std::getenv("CUMPSGEMM_FORCE_KSPLIT")) force_split = std::atoi(f);
+    const int force_cls = tuning().force_cls, force_split = tuning().force_split;
     const PreSplitChoice ch = choose_pre_split<CPLX>(handle, op_A != HIPBLAS_OP_N, op_B == HIPBLAS_OP_N, m, n, k, 1,
                                                      compute_mode, force_cls, force_split, 0);
     if (ch.take) {
@@ -768,6 +795,7 @@ hipblasStatus_t cuMpSGEMM_destroy(cuMpSGEMM_handle_t handle) {
   (void)hipFree(handle->stats_ticket);
   (void)hipFree(handle->flag_buffer);
   if (handle->pack_ws != nullptr) (void)hipFree(handle->pack_ws);
+  for (void *p : handle->retired_ws) (void)hipFree(p);
   if (handle->order_event != nullptr) (void)hipEventDestroy(handle->order_event);
   if (handle->host_scratch) (void)hipHostFree(handle->host_scratch);
   delete handle;
@@ -878,6 +906,13 @@ hipblasStatus_t cuMpSGEMM_cgemm_ex(cuMpSGEMM_handle_t handle, hipblasOperation_t
 
 size_t cuMpSGEMM_get_workspace_size(cuMpSGEMM_handle_t handle) {
   return handle != nullptr ? (size_t)handle->pack_ws_bytes : 0;
+}
+const void *cuMpSGEMM_get_workspace_pointer(cuMpSGEMM_handle_t handle) {
+  return handle != nullptr ? handle->pack_ws : nullptr;
+}
+void cuMpSGEMM_reload_tuning_env(void) {
+  (void)tuning();
+  g_tuning = read_tuning_env();
 }
 
 int cuMpSGEMM_describe_tile_config(int compute_mode, int is_complex, int op_A, int op_B,

@@ -6,6 +6,7 @@
 // src/instance_sm80.cu, src/cumpsgemm.cu:19-89).
 #pragma once
 #include "gemm_kernel.hpp"
+#include <atomic>
 
 namespace cumpsgemm_amd {
 
@@ -35,13 +36,15 @@ template <class Cfg>
 void launch_cfg(const GemmArgs &args, dim3 grid, hipStream_t stream) {
   if (Cfg::LDS_BYTES > 64 * 1024) {
     // more than 64 KiB of dynamic LDS must be allowed once per kernel and device
-    static bool attr_done[64] = {};
+    // (setting it twice is harmless, so threads that race here only need the
+    // flag itself to be free of a data race)
+    static std::atomic<bool> attr_done[64] = {};
     int dev = 0;
     (void)hipGetDevice(&dev);
-    if (dev < 0 || dev >= 64 || !attr_done[dev]) {
+    if (dev < 0 || dev >= 64 || !attr_done[dev].load(std::memory_order_acquire)) {
       (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_tcec_kernel<Cfg>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES);
-      if (dev >= 0 && dev < 64) attr_done[dev] = true;
+      if (dev >= 0 && dev < 64) attr_done[dev].store(true, std::memory_order_release);
     }
   }
   hipLaunchKernelGGL(gemm_tcec_kernel<Cfg>, grid, dim3(Cfg::NT), Cfg::LDS_BYTES, stream, args);

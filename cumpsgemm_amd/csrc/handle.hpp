@@ -10,6 +10,7 @@
 #include <cstdint>
 #include <string>
 #include <unordered_map>
+#include <vector>
 
 namespace cumpsgemm_amd {
 
@@ -43,6 +44,25 @@ struct Profiler {
 
 constexpr unsigned kRingLength = 10000;        // reference src/exp_stats.cu:574
 constexpr unsigned kMaxStatsBlocks = 4096;     // partial-result scratch entries
+
+// Tuning knobs of the GEMM path, read from the environment once per process
+// (cuMpSGEMM_reload_tuning_env() reads them again; it is meant for tests and
+// experiments and must not run while another thread is inside a GEMM call).
+struct Tuning {
+  int packed = -1;      // CUMPSGEMM_PACKED: 0 never / 1 whenever possible take the pre-split path
+  int packed_walk = -1; // CUMPSGEMM_PACKED_WALK: 0 / 1 force the one-tile / persistent pre-split kernel
+  int raster_group = 0; // CUMPSGEMM_RASTER_GROUP: tile rows per column group (0: built-in choice)
+  int force_cls = -1;   // CUMPSGEMM_FORCE_TILE_CLASS
+  int force_split = 0;  // CUMPSGEMM_FORCE_KSPLIT
+  bool no_persistent = false;    // CUMPSGEMM_NO_PERSISTENT
+  bool no_column_split = false;  // CUMPSGEMM_NO_COLUMN_SPLIT
+  bool no_fused_scaling = false; // CUMPSGEMM_NO_FUSED_SCALING
+  unsigned persistent_max_steps = 32; // CUMPSGEMM_PERSISTENT_MAX_STEPS
+  // CUMPSGEMM_MAX_WORKSPACE_BYTES: the pre-split path is not taken when its
+  // planes would need more than this (0 keeps the path from allocating at all)
+  unsigned long long max_workspace_bytes = 16ull << 30;
+};
+const Tuning &tuning();
 } // namespace cumpsgemm_amd
 
 struct cuMpSGEMM_handle {
@@ -78,6 +98,12 @@ struct cuMpSGEMM_handle {
   // the handle
   void *pack_ws = nullptr;
   unsigned long long pack_ws_bytes = 0;
+  // A HIP graph captured while the pre-split path ran holds the address of
+  // pack_ws: from then on that buffer is never freed before the handle is
+  // destroyed (a later, larger call gets a new one and the old one is parked
+  // here), so replays of the graph keep reading and writing memory they own.
+  bool pack_ws_captured = false;
+  std::vector<void *> retired_ws;
 
   // The rings, partials and workspaces above are shared by every call on the
   // handle, so work of the handle on two streams must not overlap: when the

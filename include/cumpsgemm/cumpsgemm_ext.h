@@ -38,6 +38,21 @@ int cuMpSGEMM_describe_tile_config(int compute_mode, int is_complex, int op_A, i
  * by cuMpSGEMM_destroy).  No counterpart in the reference, whose kernels need
  * no workspace beyond the fixed scratch of its handle. */
 size_t cuMpSGEMM_get_workspace_size(cuMpSGEMM_handle_t handle);
+/* Address of that workspace (NULL until it exists).  A buffer that was in use
+ * while the handle's stream was being captured into a HIP graph is never
+ * freed before cuMpSGEMM_destroy, so replays of the graph stay valid when a
+ * later, larger call makes the handle take a new buffer.  The pre-split path
+ * is skipped when its planes would exceed CUMPSGEMM_MAX_WORKSPACE_BYTES
+ * (environment, decimal bytes, default 16 GiB; 0 = never allocate). */
+const void *cuMpSGEMM_get_workspace_pointer(cuMpSGEMM_handle_t handle);
+
+/* The tuning variables of the GEMM path (CUMPSGEMM_PACKED, _PACKED_WALK,
+ * _RASTER_GROUP, _FORCE_TILE_CLASS, _FORCE_KSPLIT, _NO_PERSISTENT,
+ * _NO_COLUMN_SPLIT, _NO_FUSED_SCALING, _PERSISTENT_MAX_STEPS,
+ * _MAX_WORKSPACE_BYTES) are read from the environment once per process; this
+ * reads them again.  For tests and experiments: not to be called while another
+ * thread is inside a GEMM call.  The reference has no such variables. */
+void cuMpSGEMM_reload_tuning_env(void);
 
 /* The whole mode pipeline of an intercepted call, callable directly:
  *   FP16TCEC_SCALING: exp_max(A), exp_max(B) -> scale A, B in place -> FP16TCEC

@@ -28,6 +28,41 @@ def cg():
     return cumpsgemm_amd
 
 
+class _TuningEnv:
+    """monkeypatch whose environment changes reach the library: the GEMM path reads
+    its CUMPSGEMM_* tuning variables once per process, so after every change the
+    library is told to read them again."""
+
+    def __init__(self, mp):
+        self._mp = mp
+
+    def _reload(self):
+        import cumpsgemm_amd
+        cumpsgemm_amd.lib().cuMpSGEMM_reload_tuning_env()
+
+    def setenv(self, name, value, prepend=None):
+        self._mp.setenv(name, value, prepend)
+        self._reload()
+
+    def delenv(self, name, raising=True):
+        self._mp.delenv(name, raising)
+        self._reload()
+
+    def undo(self):
+        self._mp.undo()
+        self._reload()
+
+    def __getattr__(self, name):
+        return getattr(self._mp, name)
+
+
+@pytest.fixture
+def monkeypatch(monkeypatch):
+    mp = _TuningEnv(monkeypatch)
+    yield mp
+    mp.undo()
+
+
 @pytest.fixture(scope="session")
 def torch_gpu():
     import torch

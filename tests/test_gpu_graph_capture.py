@@ -106,3 +106,60 @@ def test_capture_never_grows_the_workspace(cg, torch_gpu, monkeypatch):
     finally:
         torch.cuda.synchronize()
         h.close()
+
+
+def test_captured_workspace_outlives_a_larger_eager_call(cg, torch_gpu):
+    """A graph captured on the pre-split path holds the address of the handle's workspace.  A
+    later, larger eager call makes the handle take a new workspace; the captured one must stay
+    allocated so that replays of the graph keep working on memory they own."""
+    torch = torch_gpu
+    m, n, k = 4096, 3840, 768
+    dev = torch.device("cuda:0")
+    h = cg.Handle()
+    side = torch.cuda.Stream()
+    a = torch.from_numpy(inputs.uniform(41, m * k)).to(dev)
+    b = torch.from_numpy(inputs.uniform(42, k * n)).to(dev)
+    c_graph = torch.zeros(m * n, device=dev)
+    c_eager = torch.zeros(m * n, device=dev)
+
+    def call(c_out):
+        return h.gemm(N_OP, 112, m, n, k, 1.0, a, m, b, n, 0.0, c_out, m, FP16TCEC, want_module_id=True)
+
+    try:
+        h.set_stream(side)
+        with torch.cuda.stream(side):
+            st, mid = call(c_eager)             # outside the capture: allocates the workspace
+        torch.cuda.synchronize()
+        assert st == 0 and mid == 200
+        ws_captured, size_captured = h.workspace_pointer(), h.workspace_size()
+        assert ws_captured != 0
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=side):
+            h.set_stream(torch.cuda.current_stream())
+            st, mid = call(c_graph)
+        assert st == 0 and mid == 200 and h.workspace_pointer() == ws_captured
+        # a larger eager call on the same handle: new workspace, the old one is kept
+        m2 = n2 = 4096
+        k2 = 2048
+        a2 = torch.from_numpy(inputs.uniform(43, m2 * k2)).to(dev)
+        b2 = torch.from_numpy(inputs.uniform(44, k2 * n2)).to(dev)
+        c2 = torch.zeros(m2 * n2, device=dev)
+        h.set_stream(torch.cuda.current_stream())
+        st, mid = h.gemm(N_OP, 112, m2, n2, k2, 1.0, a2, m2, b2, n2, 0.0, c2, m2, FP16TCEC, want_module_id=True)
+        torch.cuda.synchronize()
+        assert st == 0 and mid == 200 and h.workspace_size() > size_captured
+        ws_new = h.workspace_pointer()
+        assert ws_new != ws_captured
+        # memory allocated now must not land on the captured workspace (it would if it had been freed)
+        filler = torch.full((size_captured // 4,), 7.0, device=dev)
+        assert not (ws_captured <= filler.data_ptr() < ws_captured + size_captured)
+        for _ in range(2):
+            c_graph.zero_()
+            torch.cuda.synchronize()
+            g.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(c_graph, c_eager)
+            assert float(filler.min()) == 7.0 and float(filler.max()) == 7.0
+    finally:
+        torch.cuda.synchronize()
+        h.close()
