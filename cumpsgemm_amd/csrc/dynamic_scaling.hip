@@ -20,21 +20,27 @@ constexpr int kBlock = 256;
 constexpr float kHalfExpMax = 16384.0f; // 2^14
 constexpr int kScaleABit = 0x40, kScaleBBit = 0x20, kModeMask = 0x1f;
 
-enum ScaleKind : int { SCALE_A = 0, SCALE_B = 1, SCALE_C = 2, RESET_A = 3, RESET_B = 4 };
+// UNSCALE_C: the inverse of SCALE_C's coefficient (see unscale_C below)
+enum ScaleKind : int { SCALE_A = 0, SCALE_B = 1, SCALE_C = 2, RESET_A = 3, RESET_B = 4, UNSCALE_C = 5 };
 
 // Coefficient for one scaling launch, or 0 to skip (flag bit clear / max == 0).
 __device__ inline float scaling_coef(int kind, const int *flag_ptr, const StatsSlot *slot_a,
                                      const StatsSlot *slot_b) {
   const int flag = *flag_ptr;
   const float ma = __uint_as_float(slot_a->max_exp_bits);
-  if (kind == SCALE_C) {
+  if (kind == SCALE_C || kind == UNSCALE_C) {
     const float mb = __uint_as_float(slot_b->max_exp_bits);
     if (ma == 0.0f || mb == 0.0f) return 0.0f;
     const bool sa = flag & kScaleABit, sb = flag & kScaleBBit;
     if (!sa && !sb) return 0.0f;
     float coef = 1.0f;
-    if (sa) coef *= ma / kHalfExpMax;
-    if (sb) coef *= mb / kHalfExpMax;
+    if (kind == SCALE_C) {
+      if (sa) coef *= ma / kHalfExpMax;
+      if (sb) coef *= mb / kHalfExpMax;
+    } else {
+      if (sa) coef *= kHalfExpMax / ma;
+      if (sb) coef *= kHalfExpMax / mb;
+    }
     return coef;
   }
   const bool is_a = (kind == SCALE_A || kind == RESET_A);
@@ -139,6 +145,23 @@ int read_flag(cuMpSGEMM_handle *h, unsigned id) {
   return v;
 }
 } // namespace
+} // namespace cumpsgemm_amd
+
+namespace cumpsgemm_amd {
+// C *= 1 / (scale_C's coefficient).  The stand-alone form of the scaled
+// pipelines runs this on C before a GEMM with beta != 0, so that the scale_C
+// pass that follows the GEMM -- which multiplies all of C, beta * C_old
+// included -- leaves beta * C_old as it was: every factor is a power of two,
+// hence exact unless C_old / coefficient leaves FP32's range.
+template <class T>
+void unscale_C(cuMpSGEMM_handle *h, unsigned slot_a, unsigned slot_b, unsigned flag_id, unsigned m, unsigned n,
+               T *ptr, unsigned ld, unsigned batch, unsigned stride) {
+  launch_scaling<T>(h, UNSCALE_C, slot_a, slot_b, flag_id, m, n, ptr, ld, batch, stride, "scaling_C");
+}
+template void unscale_C<float>(cuMpSGEMM_handle *, unsigned, unsigned, unsigned, unsigned, unsigned, float *,
+                               unsigned, unsigned, unsigned);
+template void unscale_C<hipComplex>(cuMpSGEMM_handle *, unsigned, unsigned, unsigned, unsigned, unsigned,
+                                    hipComplex *, unsigned, unsigned, unsigned);
 } // namespace cumpsgemm_amd
 
 using namespace cumpsgemm_amd;

@@ -5,6 +5,7 @@
 // src/cumpsgemm_cublas.cu:446-577 (single) and :836-960 (strided batch).
 #include "pipeline.hpp"
 #include <cstdlib>
+#include <type_traits>
 #include "handle.hpp"
 #include "utils.hpp"
 #include <cumpsgemm/cumpsgemm_ext.h>
@@ -49,9 +50,11 @@ hipblasStatus_t gemm_pipeline(cuMpSGEMM_handle_t h, hipblasOperation_t op_A,
   // A and B in place through a const_cast and undoes it afterwards
   // (src/cumpsgemm_cublas.cu:511-518, :562-573); that form is kept for callers
   // that ask for the scaled operands to be left behind (restore_AB == false).
-  // One deliberate difference: with beta != 0 the fused form computes
-  // alpha*A*B + beta*C, while rescaling the finished C also rescales beta*C.
-  const bool fused = scaled && restore_AB && std::getenv("CUMPSGEMM_NO_FUSED_SCALING") == nullptr;
+  // Both forms compute alpha*op(A)*op(B) + beta*C.  (The reference's sequence
+  // GEMM-with-beta, then scale_C over all of C also rescales beta*C_old,
+  // src/cumpsgemm_cublas.cu:549-559; the stand-alone form here divides C_old
+  // by that power of two first, which the final scale_C undoes exactly.)
+  const bool fused = scaled && restore_AB && !tuning().no_fused_scaling;
   if (mode == CUMPSGEMM_AUTO) {
     exp_stats_pair<T>(h, va, vb, a_id, b_id);
     flag_id = cumpsgemm::get_next_dynamic_launch_buffer_id(h);
@@ -68,6 +71,13 @@ hipblasStatus_t gemm_pipeline(cuMpSGEMM_handle_t h, hipblasOperation_t op_A,
       cumpsgemm::scale_A<T>(h, a_id, flag_id, a_rows, a_cols, a, (unsigned)lda, sb, sa_stride);
       cumpsgemm::scale_B<T>(h, b_id, flag_id, b_rows, b_cols, b, (unsigned)ldb, sb, sb_stride);
     }
+  }
+  if (scaled && !fused) {
+    bool beta_nonzero;
+    if constexpr (std::is_same<T, hipComplex>::value) beta_nonzero = beta != nullptr && (beta->x != 0.0f || beta->y != 0.0f);
+    else beta_nonzero = beta != nullptr && *beta != 0.0f;
+    if (beta_nonzero)
+      unscale_C<T>(h, a_id, b_id, flag_id, (unsigned)m, (unsigned)n, c, (unsigned)ldc, sb, sc_stride);
   }
   if (fused) {
     h->fused_scaling = true;

@@ -14,4 +14,8 @@ hipblasStatus_t gemm_pipeline(cuMpSGEMM_handle_t h, hipblasOperation_t op_A,
                               uint64_t ldb, uint64_t strideb, const T *beta, T *c, uint64_t ldc,
                               uint64_t stridec, uint64_t batch, bool batched,
                               cuMpSGEMM_compute_mode_t mode, bool restore_AB, PipelineIds *ids);
+// C *= 1 / (the coefficient scale_C applies), see dynamic_scaling.hip
+template <class T>
+void unscale_C(cuMpSGEMM_handle *h, unsigned slot_a, unsigned slot_b, unsigned flag_id, unsigned m, unsigned n,
+               T *ptr, unsigned ld, unsigned batch, unsigned stride);
 } // namespace cumpsgemm_amd

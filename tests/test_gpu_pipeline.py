@@ -266,3 +266,45 @@ def test_pipeline_rejects_what_the_statistics_cannot_address(handle, dev, mode):
     c = dev.up(np.zeros(16, np.float32))
     st, _ = handle.gemm_pipeline(N, N, 4, 4, 1, 1.0, x, big, x, 4, 0.0, c, 4, FP16TCEC)
     assert st == 0 and np.array_equal(dev.down(c), np.ones(16, np.float32))
+
+
+@pytest.mark.parametrize("mode", [SCALING, AUTO])
+@pytest.mark.parametrize("cplx", [False, True])
+@pytest.mark.parametrize("restore,fused", [(True, True), (True, False), (False, False)])
+def test_scaled_pipelines_with_beta(O, handle, dev, monkeypatch, mode, cplx, restore, fused):
+    """alpha * op(A) * op(B) + beta * C in the scaled modes, beta != 0, against FP64: the fused form
+    (A, B untouched), the stand-alone passes with restoration and the form that leaves A and B scaled
+    all keep beta * C_old out of the rescaling of C.  (Rescaling the finished C, as the reference's
+    sequence does, src/cumpsgemm_cublas.cu:549-559, would multiply beta * C_old by 2^-17 here.)"""
+    m, n, k = 200, 136, 160
+    dt = np.complex64 if cplx else np.float32
+    gen = (lambda s, c: inputs.complex_normal(s, c, 1.0)) if cplx else inputs.uniform
+    a = (gen(91, m * k) * np.float32(2.0 ** -21)).astype(dt)     # needs scaling (by 2^34 or so)
+    b = (gen(92, k * n) * np.float32(2.0 ** 3)).astype(dt)
+    c0 = (gen(93, (m + 5) * n) * np.float32(2.0 ** -16)).astype(dt)  # same magnitude as alpha*A*B
+    alpha, beta = ((0.75 - 0.5j), (-1.25 + 0.5j)) if cplx else (0.75, -1.25)
+    ldc = m + 5
+    if fused:
+        monkeypatch.delenv("CUMPSGEMM_NO_FUSED_SCALING", raising=False)
+    else:
+        monkeypatch.setenv("CUMPSGEMM_NO_FUSED_SCALING", "1")
+    if mode == AUTO:
+        handle.set_exp_stats_params(0.0, 2.0 ** -15, 0.1)
+    try:
+        da, db, dc = dev.up(a), dev.up(b), dev.up(c0)
+        st, ids = handle.gemm_pipeline(T, N, m, n, k, alpha, da, k, db, k, beta, dc, ldc, mode, cplx=cplx,
+                                       restore_ab=restore)
+        assert st == 0
+        c = dev.down(dc, dt)
+        a_after = dev.down(da, dt)
+    finally:
+        handle.set_exp_stats_params(0.0, 2.0 ** -15, 0.0)
+    if mode == AUTO:
+        assert handle.get_dynamic_launch_flag(ids[2]) == (FP16TCEC | 0x40)
+    assert np.array_equal(a_after, a) == restore
+    ref = O.gemm_fp64(T, N, m, n, k, alpha, a, k, b, k, beta, c0, ldc)
+    cf = oracle_gemm(O, FP32, T, N, m, n, k, alpha, a, k, b, k, beta, c0, ldc)
+    r, r32 = O.residual(ref, c, m, n, ldc), O.residual(ref, cf, m, n, ldc)
+    assert r <= 2.0 * r32 + 2.0 ** -24, (r, r32)
+    # rows m .. ldc of every column are not part of C
+    assert np.array_equal(c.reshape(n, ldc)[:, m:], c0.reshape(n, ldc)[:, m:])
