@@ -103,6 +103,18 @@ hipStream_t caller_stream(hipblasHandle_t hb) {
   return s;
 }
 
+// Whether the caller's hipBLAS handle takes alpha and beta from device memory.
+// This library's entry points read them on the host (as the reference does,
+// src/cumpsgemm.cu:266, with no cublasGetPointerMode anywhere in
+// src/cumpsgemm_cublas.cu), so such calls are left to hipBLAS.
+bool device_pointer_mode(hipblasHandle_t hb) {
+  using fn_t = hipblasStatus_t (*)(hipblasHandle_t, hipblasPointerMode_t *);
+  static fn_t fn = reinterpret_cast<fn_t>(real_symbol("hipblasGetPointerMode"));
+  hipblasPointerMode_t pm = HIPBLAS_POINTER_MODE_HOST;
+  if (fn == nullptr || hb == nullptr || fn(hb, &pm) != HIPBLAS_STATUS_SUCCESS) return false;
+  return pm == HIPBLAS_POINTER_MODE_DEVICE;
+}
+
 bool mx2x2_enabled() {
   if (g_mx2x2_enabled) return true;
   return env_flag("CUMPSGEMM_CUSTOM_GEMM_MX2X2", false);
@@ -272,15 +284,23 @@ hipblasStatus_t hijack_core(const char *func_name, hipblasHandle_t hb, hipblasOp
     return HIPBLAS_STATUS_INVALID_VALUE;
   }
   const cuMpSGEMM_compute_mode_t mode = query_mode(func_name, hb, op_A, op_B, m, n, k);
+  // scalars in device memory: nothing here can read them, the call goes to hipBLAS
+  const bool device_scalars = mode != CUMPSGEMM_DRY_RUN && device_pointer_mode(hb);
+  const bool gate_shape = mx2x2_enabled() && !device_scalars && k == 2 &&
+                          ((n == 2 && is_pow2((uint64_t)m)) || (m == 2 && is_pow2((uint64_t)n)));
+  const bool forward = mode != CUMPSGEMM_DRY_RUN && !gate_shape && (forwards_to_hipblas(mode) || device_scalars);
   // One intercepted call at a time from here on: the process-wide handle, the
   // record of the last call and the stream it runs on are shared by all host
   // threads.  (The rule hook above runs outside the lock: it may call back
   // into user code.  Recursive, in case the vendor library's own GEMM entry
   // points call each other through the dynamic symbol table.)
   static std::recursive_mutex call_mutex;
-  const std::lock_guard<std::recursive_mutex> lock(call_mutex);
-  // a dry run only logs: it must not need a device, so the handle is created after it
-  cuMpSGEMM_handle_t h = (mode == CUMPSGEMM_DRY_RUN) ? g_handles[current_device()] : global_handle();
+  std::unique_lock<std::recursive_mutex> lock(call_mutex);
+  // a dry run only logs: it must not need a device, so the handle is created
+  // after it; a forwarded call uses the handle only if there is one already
+  // (statistics of C are switched on through a handle)
+  cuMpSGEMM_handle_t h =
+      (mode == CUMPSGEMM_DRY_RUN || forward) ? g_handles[current_device()] : global_handle();
 
   if (env_flag("CUMPSGEMM_INFO", false)) {
     log_info(std::string(func_name) + " op=(" + op_str(op_A) + ", " + op_str(op_B) + "), shape=(" +
@@ -301,6 +321,34 @@ hipblasStatus_t hijack_core(const char *func_name, hipblasHandle_t hb, hipblasOp
   g_last.mode = mode;
 
   if (mode == CUMPSGEMM_DRY_RUN) return HIPBLAS_STATUS_SUCCESS;
+
+  if (forward) {
+    // The vendor library does this call; unless statistics of C are wanted
+    // nothing of this library is involved, so other threads' calls need not wait.
+    const bool stats_of_c = h != nullptr && h->exp_stats_enabled;
+    if (!stats_of_c) lock.unlock();
+    if (device_scalars && !forwards_to_hipblas(mode)) {
+      log_warning("alpha / beta are in device memory (HIPBLAS_POINTER_MODE_DEVICE): forwarding to hipBLAS");
+      log_info(" +---> forwarded to hipBLAS (device pointer mode)");
+    }
+    CulipScope prof(culip_enabled(), caller_stream(hb), func_name, op_A, op_B, m, n, k, batched, batch);
+    const hipblasStatus_t st =
+        batched ? forward_gemm_sb<T>(hb, op_A, op_B, m, n, k, alpha, a, lda, sa, b, ldb, sb, beta,
+                                     c, ldc, sc, batch)
+                : forward_gemm<T>(hb, op_A, op_B, m, n, k, alpha, a, lda, b, ldb, beta, c, ldc);
+    if (stats_of_c) {
+      // statistics of the result, as the reference does for forwarded calls
+      // (src/cumpsgemm_cublas.cu:420-425); the statistics take a 32-bit stride
+      if (batched && (sc < 0 || sc > 0xffffffffll)) {
+        log_warning("exp_stats of C skipped: the batch stride does not fit 32 bits");
+      } else {
+        cuMpSGEMM_set_stream(h, caller_stream(hb));
+        cumpsgemm::exp_stats_ext<T>(h, (unsigned)m, (unsigned)n, c, (unsigned)ldc,
+                                    batched ? (unsigned)batch : 1u, batched ? (unsigned)sc : 0u);
+      }
+    }
+    return st;
+  }
   if (h == nullptr) return HIPBLAS_STATUS_NOT_INITIALIZED;
 
   if (batched && (sa < 0 || sb < 0 || sc < 0)) {
@@ -342,24 +390,6 @@ hipblasStatus_t hijack_core(const char *func_name, hipblasHandle_t hb, hipblasOp
                                    usc, nb);
   }
 
-  if (forwards_to_hipblas(mode)) {
-    CulipScope prof(culip, cstream, func_name, op_A, op_B, m, n, k, batched, batch);
-    const hipblasStatus_t st =
-        batched ? forward_gemm_sb<T>(hb, op_A, op_B, m, n, k, alpha, a, lda, sa, b, ldb, sb, beta,
-                                     c, ldc, sc, batch)
-                : forward_gemm<T>(hb, op_A, op_B, m, n, k, alpha, a, lda, b, ldb, beta, c, ldc);
-    if (h->exp_stats_enabled) {
-      // statistics of the result, as the reference does for forwarded calls
-      // (src/cumpsgemm_cublas.cu:420-425); the statistics take a 32-bit stride
-      if (batched && (sc < 0 || sc > 0xffffffffll)) {
-        log_warning("exp_stats of C skipped: the batch stride does not fit 32 bits");
-      } else {
-        cumpsgemm::exp_stats_ext<T>(h, (unsigned)m, (unsigned)n, c, (unsigned)ldc,
-                                    batched ? (unsigned)batch : 1u, batched ? (unsigned)sc : 0u);
-      }
-    }
-    return st;
-  }
   if (mode == CUMPSGEMM_FP32_SIMT || mode == CUMPSGEMM_UNDEFINED) {
     log_error(std::string("mode ") + cuMpSGEMM_get_compute_mode_string(mode) +
               " is not executable; forwarding to hipBLAS");

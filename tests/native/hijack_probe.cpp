@@ -118,6 +118,19 @@ int main(int argc, char **argv) {
   st = hipblasSgemm(hb, HIPBLAS_OP_N, HIPBLAS_OP_N, 0, n, n, &one, da.p, n, db.p, n, &zero, dc.p, n);
   std::printf("RESULT zero_m status=%d relerr=0\n", (int)st);
 
+  // alpha and beta in device memory: the interposer cannot read them on the host and must
+  // leave the call to hipBLAS whatever the mode
+  {
+    dev_buf<float> dscal(2);
+    const float hs[2] = {1.0f, 0.0f};
+    CHECK_HIP(hipMemcpyAsync(dscal.p, hs, sizeof(hs), hipMemcpyHostToDevice, stream));
+    CHECK_HIP(hipMemsetAsync(dc.p, 0, e * batch * 4, stream));
+    hipblasSetPointerMode(hb, HIPBLAS_POINTER_MODE_DEVICE);
+    st = hipblasSgemm(hb, HIPBLAS_OP_N, HIPBLAS_OP_N, n, n, n, dscal.p, da.p, n, db.p, n, dscal.p + 1, dc.p, n);
+    hipblasSetPointerMode(hb, HIPBLAS_POINTER_MODE_HOST);
+    check_real("hipblasSgemm_device_scalars", st, 1, false);
+  }
+
   // complex: the float buffers reinterpreted as n/2-column complex matrices
   {
     const int nc = n / 2; // complex matrices are n x nc? keep them square: nc x nc

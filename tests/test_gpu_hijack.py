@@ -76,6 +76,18 @@ def test_preload_other_modes(mode):
     assert any(f"mode={mode}" in l for l in logs)
 
 
+def test_device_pointer_mode_calls_are_forwarded():
+    """alpha / beta in device memory (HIPBLAS_POINTER_MODE_DEVICE): the TCEC entry points read
+    them on the host, so the interposer hands such a call to hipBLAS instead of faulting."""
+    res, logs = _probe({"CUMPSGEMM_COMPUTE_MODE": "FP16TC", "CUMPSGEMM_INFO": "1", "CUMPSGEMM_ERROR_LOG": "1"})
+    assert res["hipblasSgemm"][0] == 0 and res["hipblasSgemm"][1] > 1e-5       # our fp16 kernel
+    st, err = res["hipblasSgemm_device_scalars"]
+    assert st == 0 and err < 2e-6                                               # hipBLAS FP32
+    text = "\n".join(logs)
+    assert "[cuMpSGEMM WARNING] alpha / beta are in device memory" in text
+    assert "forwarded to hipBLAS (device pointer mode)" in text
+
+
 def test_preload_dry_run_leaves_c_untouched():
     res, logs = _probe({"CUMPSGEMM_COMPUTE_MODE": "DRY_RUN", "CUMPSGEMM_INFO": "1"})
     assert res["hipblasSgemm"] == (0, 1.0)  # C stayed zero: relative error exactly 1
