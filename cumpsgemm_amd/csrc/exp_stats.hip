@@ -62,6 +62,30 @@ struct StatsJob {
 // two saves a kernel boundary, which costs about as much as scanning 30 MB):
 // workgroups [0, job0.blocks) take job0, the rest job1, each job with its own
 // partials and arrival counter.
+// Ordering of the hand-over from the publishing workgroups to the folding one.
+// CUMPSGEMM_STATS_STRICT_ORDER = 1 makes the ticket an acquire-release atomic
+// at device scope, which is all the HIP memory model asks for; on gfx950 that
+// costs an L2 write-back and invalidate per workgroup, serialised behind one
+// another (64 MiB scan: 77 us against 17 us).  The default form relies on three
+// properties of gfx950 instead, and refuses to compile for anything else:
+//  - an atomic store or load at device scope is performed at the memory side of
+//    the fabric (it bypasses the issuing XCD's L2 and the vector L1), so a
+//    partial record needs no cache write-back to become visible to another XCD
+//    and no invalidate to be read fresh;
+//  - s_waitcnt vmcnt(0) / lgkmcnt(0) returns only when those stores have been
+//    acknowledged, so every record is in memory before its workgroup's ticket
+//    increment is issued;
+//  - the compiler keeps relaxed atomics to different addresses in program
+//    order around the explicit waitcnt (they are volatile-like memory
+//    operations to it).
+// A soak test (thousands of launches of every size against an independent
+// count) guards the default form.
+#ifndef CUMPSGEMM_STATS_STRICT_ORDER
+#define CUMPSGEMM_STATS_STRICT_ORDER 0
+#endif
+#if !CUMPSGEMM_STATS_STRICT_ORDER && defined(__HIP_DEVICE_COMPILE__) && !defined(__gfx950__)
+#error "the fence-free hand-over of exp_stats_kernel is written for gfx950; build with -DCUMPSGEMM_STATS_STRICT_ORDER=1"
+#endif
 template <int MODE>
 __global__ __launch_bounds__(kBlock) void exp_stats_kernel(const StatsJob job0, const StatsJob job1,
                                                            float ignore_thr, float under_thr,
@@ -172,10 +196,16 @@ __global__ __launch_bounds__(kBlock) void exp_stats_kernel(const StatsJob job0, 
                          __HIP_MEMORY_SCOPE_AGENT);
       __hip_atomic_store(&p->total, t, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       __hip_atomic_store(&p->underflow, u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#if CUMPSGEMM_STATS_STRICT_ORDER
+      // the portable form: the ticket is a release / acquire operation at device scope
+      const unsigned arrived =
+          __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+#else
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
       __builtin_amdgcn_s_waitcnt(0);
       const unsigned arrived =
           __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#endif
       s_last = (arrived == nblocks - 1);
     }
   }
