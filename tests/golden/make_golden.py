@@ -85,6 +85,68 @@ def make_exact_gemm():
             "cases": cases}
 
 
+def make_exact_cgemm():
+    """Gaussian-integer CGEMMs: every real product and partial sum is a small integer, so the
+    result is exact in every emulation mode and in any order.  All nine (op A, op B) pairs,
+    complex alpha and beta, leading dimensions larger than the matrices (and odd).  Computed
+    with Python integers: re/im parts are kept apart, no floating point is involved."""
+    rng = np.random.default_rng(11)
+    shapes = [(5, 4, 7), (33, 17, 40), (64, 32, 64), (19, 70, 129), (40, 3, 33), (7, 9, 16), (65, 66, 35),
+              (12, 12, 200), (31, 2, 64)]
+    cases = []
+    idx = 0
+    for opa in "NTC":
+        for opb in "NTC":
+            m, n, k = shapes[idx]
+            idx += 1
+            Ar, Ai = rng.integers(-8, 9, (m, k)), rng.integers(-8, 9, (m, k))
+            Br, Bi = rng.integers(-8, 9, (k, n)), rng.integers(-8, 9, (k, n))
+            Cr, Ci = rng.integers(-4, 5, (m, n)), rng.integers(-4, 5, (m, n))
+            (ar, ai), (br, bi) = [(2, -1), (-1, 2), (0, 3)][idx % 3], [(-1, 2), (3, 0), (1, 1)][idx % 3]
+            # logical product with Python integers
+            Pr = [[sum(int(Ar[i, p]) * int(Br[p, j]) - int(Ai[i, p]) * int(Bi[p, j]) for p in range(k))
+                   for j in range(n)] for i in range(m)]
+            Pi = [[sum(int(Ar[i, p]) * int(Bi[p, j]) + int(Ai[i, p]) * int(Br[p, j]) for p in range(k))
+                   for j in range(n)] for i in range(m)]
+            Er = [[ar * Pr[i][j] - ai * Pi[i][j] + br * int(Cr[i, j]) - bi * int(Ci[i, j]) for j in range(n)]
+                  for i in range(m)]
+            Ei = [[ar * Pi[i][j] + ai * Pr[i][j] + br * int(Ci[i, j]) + bi * int(Cr[i, j]) for j in range(n)]
+                  for i in range(m)]
+
+            def stored(Xr, Xi, op):
+                # what sits in memory so that op(stored) is the logical operand
+                if op == "N":
+                    return Xr, Xi
+                if op == "T":
+                    return Xr.T, Xi.T
+                return Xr.T, -Xi.T      # C: conjugate transpose
+
+            def flat(Xr, Xi, ld):
+                rows, cols = Xr.shape
+                out = [0] * (2 * ld * cols)
+                for j in range(cols):
+                    for i in range(ld):
+                        if i < rows:
+                            out[2 * (i + j * ld)] = int(Xr[i, j])
+                            out[2 * (i + j * ld) + 1] = int(Xi[i, j])
+                        else:               # padding rows: a value that must never be used
+                            out[2 * (i + j * ld)] = 99
+                            out[2 * (i + j * ld) + 1] = -99
+                return out
+            sar, sai = stored(Ar, Ai, opa)
+            sbr, sbi = stored(Br, Bi, opb)
+            lda, ldb, ldc = sar.shape[0] + 3, sbr.shape[0] + 1, m + 1 + 2 * (m % 2)
+            c0 = flat(Cr, Ci, ldc)
+            c = flat(np.array(Er), np.array(Ei), ldc)
+            cases.append({"m": m, "n": n, "k": k, "opa": opa, "opb": opb, "alpha": [ar, ai], "beta": [br, bi],
+                          "a": flat(sar, sai, lda), "lda": lda, "b": flat(sbr, sbi, ldb), "ldb": ldb,
+                          "c0": c0, "c": c, "ldc": ldc})
+    return {"comment": "Gaussian-integer CGEMMs, column-major interleaved (re, im) flat buffers with padded leading "
+                       "dimensions (padding rows hold 99 - 99i and must come back untouched in C); exact expected "
+                       "C = alpha*op(A)*op(B) + beta*C0 from Python integer arithmetic",
+            "cases": cases}
+
+
 def stats_bruteforce(bits, ignore_thr, under_thr, tol):
     """Scalar restatement over bit patterns; returns the record a statistics
     pass leaves behind."""
@@ -144,7 +206,8 @@ def make_stats():
 
 def main():
     for name, fn in (("fp16_convert_kat.json", make_convert), ("fp16_split_kat.json", make_split),
-                     ("gemm_exact_kat.json", make_exact_gemm), ("exp_stats_kat.json", make_stats)):
+                     ("gemm_exact_kat.json", make_exact_gemm), ("cgemm_exact_kat.json", make_exact_cgemm),
+                     ("exp_stats_kat.json", make_stats)):
         with open(os.path.join(HERE, name), "w") as f:
             json.dump(fn(), f, separators=(",", ":"))
         print("wrote", name, os.path.getsize(os.path.join(HERE, name)), "bytes")

@@ -55,6 +55,28 @@ def test_oracle_exact_gemms(O, mode):
         assert np.array_equal(c, want)
 
 
+_OPS = {"N": 111, "T": 112, "C": 113}
+
+
+def _exact_ccase_arrays(case):
+    f = lambda v: np.array(v, dtype=np.float32).view(np.complex64)
+    return f(case["a"]), f(case["b"]), f(case["c0"]), f(case["c"])
+
+
+@pytest.mark.parametrize("mode", ALL_GEMM_MODES + [12])
+def test_oracle_exact_complex_gemms(O, mode):
+    """All nine op pairs with complex alpha and beta and padded leading dimensions: pins the
+    oracle's complex epilogue (reference src/device_common.hpp:47-67) and its conjugation."""
+    cases = _load("cgemm_exact_kat.json")["cases"]
+    assert sorted(c["opa"] + c["opb"] for c in cases) == sorted(x + y for x in "NTC" for y in "NTC")
+    for case in cases:
+        a, b, c0, want = _exact_ccase_arrays(case)
+        c = c0.copy()
+        O.gemm(mode, _OPS[case["opa"]], _OPS[case["opb"]], case["m"], case["n"], case["k"], complex(*case["alpha"]),
+               a, case["lda"], b, case["ldb"], complex(*case["beta"]), c, case["ldc"])
+        assert np.array_equal(c.view(np.float32), want.view(np.float32)), (case["opa"], case["opb"])
+
+
 def test_oracle_exp_stats_known_answers(O):
     for case in _load("exp_stats_kat.json")["cases"]:
         x = np.array(case["bits"], dtype=np.uint32).view(np.float32)
@@ -78,6 +100,20 @@ def test_gpu_exact_gemms(handle, dev, mode):
                          case["ldb"], float(case["beta"]), dc, case["m"], mode)
         assert st == 0
         assert np.array_equal(dev.down(dc), want)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("mode", ALL_GEMM_MODES)
+def test_gpu_exact_complex_gemms(handle, dev, mode):
+    for case in _load("cgemm_exact_kat.json")["cases"]:
+        a, b, c0, want = _exact_ccase_arrays(case)
+        da, db, dc = dev.up(a), dev.up(b), dev.up(c0)
+        st = handle.gemm(_OPS[case["opa"]], _OPS[case["opb"]], case["m"], case["n"], case["k"],
+                         complex(*case["alpha"]), da, case["lda"], db, case["ldb"], complex(*case["beta"]), dc,
+                         case["ldc"], mode, cplx=True)
+        assert st == 0
+        got = dev.down(dc, np.complex64)
+        assert np.array_equal(got.view(np.float32), want.view(np.float32)), (case["opa"], case["opb"])
 
 
 @pytest.mark.gpu
