@@ -4,12 +4,14 @@ M=N=K=8192 (NN, uniform[-1,1], alpha=1, beta=0) on one MI355X, with the relative
 Frobenius error against an FP64 GEMM of the same inputs, next to hipBLAS native
 FP32 SGEMM on the same GPU and to the split-and-correct algorithm on host cores.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--full]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--headline-only]
 
 One "step" is one GEMM call through the C ABI (cuMpSGEMM_sgemm) with operands
-resident in HBM.  Prints ONE JSON line.  --full adds the other benchmark
-configurations (layouts, bf16x3, batched CGEMM, scaling pipeline, tall-skinny,
-Mx2x2) under "extra".
+resident in HBM.  Prints ONE JSON line.  After the headline's timed region the
+other benchmark configurations run as well (C1 on the host cores, C2 layouts and
+bf16x3, C3 batched CGEMM, C4 scaling pipeline, C5a tall-skinny, C5b Mx2x2) and
+are reported under "extra", each with its own roofline, its error against FP64
+and the vendor FP32 routine on the same inputs; --headline-only skips them.
 """
 import argparse
 import ctypes
@@ -43,7 +45,8 @@ def main():
     ap.add_argument("--steps", type=int, default=32)   # the reference times 32 calls (test/main.cu:15)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--size", type=int, default=8192)
-    ap.add_argument("--full", action="store_true")
+    ap.add_argument("--full", action="store_true", help="(default now: kept so that old command lines work)")
+    ap.add_argument("--headline-only", action="store_true", help="skip the other configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the host-core baseline")
     ap.add_argument("--kernel-only", action="store_true",
                     help="time the FP16TCEC GEMM only (no FP64 check, hipBLAS or CPU legs): for profilers")
@@ -172,8 +175,10 @@ def main():
         log(f"[bench] hipBLAS comparison unavailable: {e}")
 
     extra = {}
-    if args.full:
-        extra = full_suite(torch, cg, inputs, h, dev, stream, timed, log)
+    if not args.headline_only and n == 8192:
+        del ref, A64, B64
+        torch.cuda.empty_cache()
+        extra = full_suite(torch, cg, inputs, h, dev, stream, timed, log, a, b, c, not args.no_cpu)
 
     # ---- CPU baseline: the same algorithm on the host cores (oracle, bounded sample) ----
     cpu = None
@@ -232,6 +237,8 @@ def main():
             "unit": "TFLOP/s",
             "frac": round(kernel_tflops / FP16_MFMA_PEAK_TFLOPS, 4),
             "traffic": GEMM_TRAFFIC_BYTES if n == 8192 else None,
+            "traffic_source": "constant from the committed rocprofv3 counter runs "
+                              "(profiles/gemm_fp16tcec_8192_nn.md), not measured in this run",
             # one call = two pre-split passes (about 0.2 ms) + the GEMM kernel: all inside
             "kernel_ms": round(ev_ms, 4),
             "kernels_per_step": "pack_split_pair_kernel + gemm_tcec_kernel (packed)" if module_id == 200 else
@@ -293,28 +300,81 @@ def hbm_kernel_only(args, torch, cg, inputs, h, dev, stream):
                       "ms_per_call": round(ms, 5), "GBs": round(nbytes / ms / 1e6, 1)}), flush=True)
 
 
-def full_suite(torch, cg, inputs, h, dev, stream, timed, log):
-    """The other benchmark configurations (C2 layouts, C3, C4, C5a, C5b), reported under "extra"."""
+def mfma_roofline(flops, ev_ms, products, kernels):
+    """Roofline entry of an MFMA-bound configuration: algorithmic flops of one call over its
+    duration between HIP events on the launch stream, against the dense fp16 / bf16 MFMA peak;
+    `products` MFMA products are issued per real multiply-add of the algorithm."""
+    t = flops / (ev_ms * 1e-3) / 1e12
+    return {"bound": "mfma", "achieved": round(t, 2), "peak": FP16_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+            "frac": round(t / FP16_MFMA_PEAK_TFLOPS, 4), "kernel_ms": round(ev_ms, 4),
+            "mfma_products_per_real_mac": products,
+            "frac_of_emulation_peak": round(products * t / FP16_MFMA_PEAK_TFLOPS, 4), "kernels": kernels}
+
+
+def hbm_roofline(nbytes, ev_ms, kernels):
+    g = nbytes / (ev_ms * 1e-3) / 1e9
+    return {"bound": "hbm", "achieved": round(g, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": round(g / HBM_PEAK_GBS, 4), "kernel_ms": round(ev_ms, 5), "bytes_per_call": nbytes,
+            "kernels": kernels}
+
+
+def full_suite(torch, cg, inputs, h, dev, stream, timed, log, a, b, c, with_cpu):
+    """The other benchmark configurations (C1, C2 layouts and bf16x3, C3, C4, C5a, C5b), reported
+    under "extra".  a, b, c: the headline's 8192^2 device buffers (uniform, seeds 1 and 2)."""
     res = {}
 
     def rel_err(got, ref):
         return (torch.linalg.norm(got - ref) / torch.linalg.norm(ref)).item()
 
-    # C2 layouts and modes at 8192^3
+    # C1: the split-and-correct arithmetic on the host cores at 1024^3 (oracle), against FP64
+    if with_cpu:
+        from oracle import oracle as O
+        O.lib()
+        cores = int(os.environ.get("OMP_NUM_THREADS", "0")) or min(os.cpu_count() or 1, 16)
+        s1 = 1024
+        ca, cb = inputs.uniform(1, s1 * s1), inputs.uniform(2, s1 * s1)
+        cc, c32 = np.zeros(s1 * s1, np.float32), np.zeros(s1 * s1, np.float32)
+        log("[bench] C1 host cores 1024^3")
+        O.gemm(O.MODE_FP16TCEC, O.OP_N, O.OP_N, s1, s1, s1, 1.0, ca, s1, cb, s1, 0.0, cc, s1)   # warm-up
+        t0 = time.perf_counter()
+        O.gemm(O.MODE_FP16TCEC, O.OP_N, O.OP_N, s1, s1, s1, 1.0, ca, s1, cb, s1, 0.0, cc, s1)
+        dt = time.perf_counter() - t0
+        O.gemm(O.MODE_FP32, O.OP_N, O.OP_N, s1, s1, s1, 1.0, ca, s1, cb, s1, 0.0, c32, s1)
+        ref1 = O.gemm_fp64(O.OP_N, O.OP_N, s1, s1, s1, 1.0, ca, s1, cb, s1)
+        # the same problem through the GPU library, for the record
+        da, db, dc = torch.from_numpy(ca).to(dev), torch.from_numpy(cb).to(dev), torch.zeros(s1 * s1, device=dev)
+        h.gemm(cg.OP_N, cg.OP_N, s1, s1, s1, 1.0, da, s1, db, s1, 0.0, dc, s1, cg.FP16TCEC)
+        _, gev = timed(lambda: h.gemm(cg.OP_N, cg.OP_N, s1, s1, s1, 1.0, da, s1, db, s1, 0.0, dc, s1, cg.FP16TCEC),
+                       20, 3)
+        res["C1_sgemm_NN_1024_host_cores"] = {
+            "host_gflops": round(2.0 * s1 ** 3 / dt / 1e9, 1), "cores": cores,
+            "rel_error_fp16tcec_cpu": O.residual(ref1, cc, s1, s1, s1),
+            "rel_error_fp32_cpu": O.residual(ref1, c32, s1, s1, s1),
+            "rel_error_fp16tcec_gpu": O.residual(ref1, dc.cpu().numpy(), s1, s1, s1),
+            "gpu_tflops": round(2.0 * s1 ** 3 / gev / 1e9, 2), "dtype": "f16 hi/lo split of f32 emulated in f32 on the host"}
+
+    # C2 layouts and modes at 8192^3 (the headline's buffers)
     n = 8192
-    a = torch.from_numpy(inputs.uniform(1, n * n)).to(dev)
-    b = torch.from_numpy(inputs.uniform(2, n * n)).to(dev)
-    c = torch.zeros(n * n, device=dev)
     A, B = a.view(n, n).t().double(), b.view(n, n).t().double()
-    refs = {"NN": A @ B, "TN": A.t() @ B, "NT": A @ B.t()}
+    A32, B32 = a.view(n, n).t(), b.view(n, n).t()
     for name, opa, opb in (("NN", cg.OP_N, cg.OP_N), ("TN", cg.OP_T, cg.OP_N), ("NT", cg.OP_N, cg.OP_T)):
-        for mode_name, mode in (("FP16TCEC", cg.FP16TCEC), ("bf16x3", cg.TF32TCEC)):
+        ref = (A.t() if opa == cg.OP_T else A) @ (B.t() if opb == cg.OP_T else B)
+        x32, y32 = (A32.t() if opa == cg.OP_T else A32), (B32.t() if opb == cg.OP_T else B32)
+        vwall, _ = timed(lambda: torch.matmul(x32, y32), 6, 2)
+        verr = rel_err(torch.matmul(x32, y32).double(), ref)
+        for mode_name, mode, prods in (("FP16TCEC", cg.FP16TCEC, 3), ("bf16x3", cg.TF32TCEC, 6)):
+            if name == "NN" and mode_name == "FP16TCEC":
+                continue                     # the headline itself
             log(f"[bench] C2 {name} {mode_name}")
             fn = lambda: h.gemm(opa, opb, n, n, n, 1.0, a, n, b, n, 0.0, c, n, mode)
             wall, ev = timed(fn, 10, 2)
-            res[f"C2_{name}_{mode_name}"] = {"tflops": round(2.0 * n ** 3 / wall / 1e9, 2),
-                                             "rel_error": rel_err(c.view(n, n).t().double(), refs[name])}
-    del refs, A, B, a, b, c
+            res[f"C2_{name}_{mode_name}"] = {
+                "tflops": round(2.0 * n ** 3 / wall / 1e9, 2), "rel_error": rel_err(c.view(n, n).t().double(), ref),
+                "vendor_fp32_matmul_tflops": round(2.0 * n ** 3 / vwall / 1e9, 2), "rel_error_vendor_fp32": verr,
+                "dtype": "f16 hi/lo" if prods == 3 else "bf16 three-term split (stands in for TF32TCEC)",
+                "roofline": mfma_roofline(2.0 * n ** 3, ev, prods, "pack_split_pair_kernel + gemm_tcec_kernel (packed)")}
+        del ref
+    del A, B, A32, B32
     torch.cuda.empty_cache()
 
     # C3: strided-batched CGEMM, batch 64 x 512^3
@@ -325,58 +385,78 @@ def full_suite(torch, cg, inputs, h, dev, stream, timed, log):
     fn = lambda: h.gemm_strided_batch(cg.OP_N, cg.OP_N, s, s, s, 1.0, za, s, s * s, zb, s, s * s, 0.0, zc, s, s * s,
                                       bs, cg.FP16TCEC, cplx=True)
     log("[bench] C3 batched CGEMM")
-    wall, ev = timed(fn, 20, 2)
+    wall, ev = timed(fn, 20, 3)
     ZA = torch.view_as_complex(za.view(bs, s, s, 2)).transpose(1, 2).to(torch.complex128)
     ZB = torch.view_as_complex(zb.view(bs, s, s, 2)).transpose(1, 2).to(torch.complex128)
     ZC = torch.view_as_complex(zc.view(bs, s, s, 2)).transpose(1, 2).to(torch.complex128)
     za32 = torch.view_as_complex(za.view(bs, s, s, 2)).transpose(1, 2)
     zb32 = torch.view_as_complex(zb.view(bs, s, s, 2)).transpose(1, 2)
     vwall, _ = timed(lambda: torch.matmul(za32, zb32), 20, 2)
-    res["C3_cgemm_batch64_512"] = {"tflops": round(8.0 * s ** 3 * bs / wall / 1e9, 2), "rel_error": rel_err(ZC, ZA @ ZB),
-                                   "vendor_complex64_matmul_tflops": round(8.0 * s ** 3 * bs / vwall / 1e9, 2)}
+    zref = ZA @ ZB
+    res["C3_cgemm_batch64_512"] = {
+        "tflops": round(8.0 * s ** 3 * bs / wall / 1e9, 2), "rel_error": rel_err(ZC, zref),
+        "vendor_complex64_matmul_tflops": round(8.0 * s ** 3 * bs / vwall / 1e9, 2),
+        "rel_error_vendor_complex64": rel_err(torch.matmul(za32, zb32).to(torch.complex128), zref),
+        "dtype": "f16 hi/lo, four real products per complex product (12 MFMA products per complex multiply-add)",
+        "roofline": mfma_roofline(8.0 * s ** 3 * bs, ev, 3, "gemm_tcec_kernel (complex)")}
+    del za, zb, zc, ZA, ZB, ZC, zref
+    torch.cuda.empty_cache()
 
     # C4: FP16TCEC_SCALING pipeline at 4096^3 with 2^{+-30} row/column exponents
     n = 4096
     ea = inputs.exponent_spread(3, n, n, per_row=True)
     eb = inputs.exponent_spread(4, n, n, per_row=False)
-    a, b = torch.from_numpy(ea).to(dev), torch.from_numpy(eb).to(dev)
-    c = torch.zeros(n * n, device=dev)
-    ref = a.view(n, n).t().double() @ b.view(n, n).t().double()
+    a4, b4 = torch.from_numpy(ea).to(dev), torch.from_numpy(eb).to(dev)
+    c4 = torch.zeros(n * n, device=dev)
+    ref = a4.view(n, n).t().double() @ b4.view(n, n).t().double()
     log("[bench] C4 scaling pipeline")
-    fn = lambda: h.gemm_pipeline(cg.OP_N, cg.OP_N, n, n, n, 1.0, a, n, b, n, 0.0, c, n, cg.FP16TCEC_SCALING)
+    fn = lambda: h.gemm_pipeline(cg.OP_N, cg.OP_N, n, n, n, 1.0, a4, n, b4, n, 0.0, c4, n, cg.FP16TCEC_SCALING)
     wall, ev = timed(fn, 10, 2)
-    err_scaled = rel_err(c.view(n, n).t().double(), ref)
-    h.gemm_pipeline(cg.OP_N, cg.OP_N, n, n, n, 1.0, a, n, b, n, 0.0, c, n, cg.AUTO)
-    err_auto = rel_err(c.view(n, n).t().double(), ref)
-    err_fp32 = rel_err((a.view(n, n).t() @ b.view(n, n).t()).double(), ref)
-    st_ms = timed(lambda: h.exp_stats_ext(n, n, a, n), 20, 3)[1]
-    mx_ms = timed(lambda: h.exp_max_ext(n, n, a, n), 20, 3)[1]
-    sid = h.exp_max_ext(n, n, a, n)
-    sc_ms = timed(lambda: (h.scale_A(sid, 1, n, n, a, n), h.reset_scale_A(sid, 1, n, n, a, n)), 20, 3)[1] / 2
+    err_scaled = rel_err(c4.view(n, n).t().double(), ref)
+    awall, aev = timed(lambda: h.gemm_pipeline(cg.OP_N, cg.OP_N, n, n, n, 1.0, a4, n, b4, n, 0.0, c4, n, cg.AUTO), 10, 2)
+    err_auto = rel_err(c4.view(n, n).t().double(), ref)
+    vwall, _ = timed(lambda: torch.matmul(a4.view(n, n).t(), b4.view(n, n).t()), 10, 2)
+    err_fp32 = rel_err((a4.view(n, n).t() @ b4.view(n, n).t()).double(), ref)
+    st_ms = timed(lambda: h.exp_stats_ext(n, n, a4, n), 20, 3)[1]
+    mx_ms = timed(lambda: h.exp_max_ext(n, n, a4, n), 20, 3)[1]
+    sid = h.exp_max_ext(n, n, a4, n)
+    sc_ms = timed(lambda: (h.scale_A(sid, 1, n, n, a4, n), h.reset_scale_A(sid, 1, n, n, a4, n)), 20, 3)[1] / 2
     nbytes = 4.0 * n * n
     res["C4_scaling_4096"] = {
-        "pipeline_tflops": round(2.0 * n ** 3 / wall / 1e9, 2), "rel_error_scaling": err_scaled,
-        "rel_error_auto": err_auto, "rel_error_fp32_matmul": err_fp32,
-        "exp_stats_GBs": round(nbytes * 2 / st_ms / 1e6, 1), "exp_max_GBs": round(nbytes / mx_ms / 1e6, 1),
-        "scaling_GBs": round(2 * nbytes / sc_ms / 1e6, 1), "hbm_peak_GBs": HBM_PEAK_GBS}
-    del a, b, c, ref
+        "pipeline_tflops": round(2.0 * n ** 3 / wall / 1e9, 2), "auto_pipeline_tflops": round(2.0 * n ** 3 / awall / 1e9, 2),
+        "rel_error_scaling": err_scaled, "rel_error_auto": err_auto, "rel_error_vendor_fp32": err_fp32,
+        "vendor_fp32_matmul_tflops": round(2.0 * n ** 3 / vwall / 1e9, 2),
+        "dtype": "f16 hi/lo after one power-of-two scaling per matrix (AUTO decides for bf16x3 on these inputs)",
+        # the whole pipeline of one call: exp_max of A and B (one launch), pre-split with scaling, GEMM
+        "roofline": mfma_roofline(2.0 * n ** 3, ev, 3, "exp_stats_kernel<max> + pack_split_pair_kernel + gemm_tcec_kernel (packed, scaled)"),
+        # two passes (stage 1 + stage 2) over one 64 MiB matrix / one pass / read + write
+        "roofline_exp_stats": hbm_roofline(2 * nbytes, st_ms, "exp_stats_kernel<0> + exp_stats_kernel<1>"),
+        "roofline_exp_max": hbm_roofline(nbytes, mx_ms, "exp_stats_kernel<2>"),
+        "roofline_scaling": hbm_roofline(2 * nbytes, sc_ms, "scaling_kernel")}
+    del a4, b4, c4, ref
     torch.cuda.empty_cache()
 
     # C5a: tall-skinny 16384 x 16384 x 256
     mm, kk = 16384, 256
-    a = torch.from_numpy(inputs.uniform(1, mm * kk)).to(dev)
-    b = torch.from_numpy(inputs.uniform(2, kk * mm)).to(dev)
-    c = torch.zeros(mm * mm, device=dev)
+    a5 = torch.from_numpy(inputs.uniform(1, mm * kk)).to(dev)
+    b5 = torch.from_numpy(inputs.uniform(2, kk * mm)).to(dev)
+    c5 = torch.zeros(mm * mm, device=dev)
     log("[bench] C5a tall-skinny")
-    fn = lambda: h.gemm(cg.OP_N, cg.OP_N, mm, mm, kk, 1.0, a, mm, b, kk, 0.0, c, mm, cg.FP16TCEC)
+    fn = lambda: h.gemm(cg.OP_N, cg.OP_N, mm, mm, kk, 1.0, a5, mm, b5, kk, 0.0, c5, mm, cg.FP16TCEC)
     wall, ev = timed(fn, 10, 2)
-    ref = a.view(kk, mm).t().double() @ b.view(mm, kk).t().double()
-    A32, B32 = a.view(kk, mm).t(), b.view(mm, kk).t()
+    _, mid5 = h.gemm(cg.OP_N, cg.OP_N, mm, mm, kk, 1.0, a5, mm, b5, kk, 0.0, c5, mm, cg.FP16TCEC, want_module_id=True)
+    ref = a5.view(kk, mm).t().double() @ b5.view(mm, kk).t().double()
+    A32, B32 = a5.view(kk, mm).t(), b5.view(mm, kk).t()
     vwall, _ = timed(lambda: torch.matmul(A32, B32), 10, 2)
-    res["C5a_16384x16384x256"] = {"tflops": round(2.0 * mm * mm * kk / wall / 1e9, 2),
-                                  "rel_error": rel_err(c.view(mm, mm).t().double(), ref),
-                                  "vendor_fp32_matmul_tflops": round(2.0 * mm * mm * kk / vwall / 1e9, 2)}
-    del a, b, c, ref
+    res["C5a_16384x16384x256"] = {
+        "tflops": round(2.0 * mm * mm * kk / wall / 1e9, 2), "rel_error": rel_err(c5.view(mm, mm).t().double(), ref),
+        "vendor_fp32_matmul_tflops": round(2.0 * mm * mm * kk / vwall / 1e9, 2),
+        "rel_error_vendor_fp32": rel_err(torch.matmul(A32, B32).double(), ref), "dtype": "f16 hi/lo",
+        "c_write_floor_ms": round(4.0 * mm * mm / (HBM_PEAK_GBS * 1e9) * 1e3, 4),
+        "roofline": mfma_roofline(2.0 * mm * mm * kk, ev, 3,
+                                  "pack_split_pair_kernel + gemm_tcec_kernel (packed)" if mid5 == 200
+                                  else "gemm_tcec_kernel (in-loop split, persistent)")}
+    del a5, b5, c5, ref
     torch.cuda.empty_cache()
 
     # C5b: Mx2x2 CGEMM, M = 2^27 (state vector x 2x2 unitary), HBM-bound
@@ -390,8 +470,10 @@ def full_suite(torch, cg, inputs, h, dev, stream, timed, log):
     X = torch.view_as_complex(x.view(2, M, 2)[:, : 1 << 20].contiguous()).t().to(torch.complex128)
     Y = torch.view_as_complex(y.view(2, M, 2)[:, : 1 << 20].contiguous()).t().to(torch.complex128)
     U = torch.view_as_complex(u.view(2, 2, 2)).t().to(torch.complex128)
-    res["C5b_cgemm_2^27x2x2"] = {"GBs": round(2.0 * M * 2 * 8 / ev / 1e6, 1), "hbm_peak_GBs": HBM_PEAK_GBS,
-                                 "rel_error_first_2^20_rows": rel_err(Y, X @ U)}
+    res["C5b_cgemm_2^27x2x2"] = {
+        "GBs": round(2.0 * M * 2 * 8 / ev / 1e6, 1), "rel_error_first_2^20_rows": rel_err(Y, X @ U),
+        "dtype": "f32 (plain FMA streaming kernel: wider than FP16TCEC, as the reference's external Mx2x2 kernels)",
+        "roofline": hbm_roofline(2.0 * M * 2 * 8, ev, "long2x2_kernel")}
     return res
 
 
