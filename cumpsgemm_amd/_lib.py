@@ -77,6 +77,9 @@ def _declare(L):
     L.cuMpSGEMM_sgemm.argtypes = [_ptr, _int, _int] + gemm_tail + [f32p, _ptr, _u64, _ptr, _u64, f32p, _ptr, _u64, _int]
     L.cuMpSGEMM_cgemm.argtypes = [_ptr, _int, _int] + gemm_tail + [c2p, _ptr, _u64, _ptr, _u64, c2p, _ptr, _u64, _int]
     L.cuMpSGEMM_sgemm_ex.argtypes = L.cuMpSGEMM_sgemm.argtypes + [ctypes.POINTER(_u32)]
+    L.cuMpSGEMM_sgemm_no_alloc.argtypes = L.cuMpSGEMM_sgemm.argtypes
+    L.cuMpSGEMM_get_static_scratch_size.argtypes = []
+    L.cuMpSGEMM_get_static_scratch_size.restype = ctypes.c_size_t
     L.cuMpSGEMM_cgemm_ex.argtypes = L.cuMpSGEMM_cgemm.argtypes + [ctypes.POINTER(_u32)]
     L.cuMpSGEMM_sgemm_strided_batch.argtypes = [_ptr, _int, _int] + gemm_tail + [
         f32p, _ptr, _u64, _u64, _ptr, _u64, _u64, f32p, _ptr, _u64, _u64, _u64, _int]
@@ -224,6 +227,12 @@ class Handle:
         st = fn(self._h, op_a, op_b, m, n, k, _scalar(alpha, cplx), _dptr(a), lda, _dptr(b), ldb,
                 _scalar(beta, cplx), _dptr(c), ldc, int(mode), ctypes.byref(mid))
         return (st, mid.value) if want_module_id else st
+
+    def gemm_no_alloc(self, op_a, op_b, m, n, k, alpha, a, lda, b, ldb, beta, c, ldc, mode):
+        """cuMpSGEMM_sgemm_no_alloc: the pre-split path over the library's static scratch."""
+        return self._L.cuMpSGEMM_sgemm_no_alloc(self._h, op_a, op_b, m, n, k, _scalar(alpha, False), _dptr(a),
+                                                lda, _dptr(b), ldb, _scalar(beta, False), _dptr(c), ldc,
+                                                int(mode))
 
     def gemm_strided_batch(self, op_a, op_b, m, n, k, alpha, a, lda, stridea, b, ldb, strideb, beta,
                            c, ldc, stridec, batch, mode, cplx=False):

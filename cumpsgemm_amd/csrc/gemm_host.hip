@@ -39,6 +39,43 @@ Tuning g_tuning;
 std::once_flag g_tuning_once;
 } // namespace
 
+// ---- home of the pre-split planes for the entry point that allocates nothing
+// One array per GPU, inside the library's code object, held until the process
+// ends.  In host code `scratch` is only a stand-in for the symbol: the device
+// address is asked for once per device (scratch_address) and that pointer is
+// what kernels and the planner get.
+constexpr unsigned long long kStaticScratchBytes = 64ull << 20;
+} // namespace cumpsgemm_amd
+static __device__ __align__(256) unsigned char scratch[cumpsgemm_amd::kStaticScratchBytes];
+namespace cumpsgemm_amd {
+namespace {
+constexpr int kMaxDevices = 64;
+void *g_scratch_ptr[kMaxDevices] = {};
+std::mutex g_scratch_mutex;
+// Device address of `scratch` on device `dev`, which must be the current
+// device; nullptr (logged) if the runtime cannot resolve it.
+void *scratch_address(int dev) {
+  if (dev < 0 || dev >= kMaxDevices) return nullptr;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void *ptr = nullptr;
+    const hipError_t err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (err != hipSuccess || ptr == nullptr) {
+      (void)hipGetLastError();
+      log_error(std::string("hipGetSymbolAddress(scratch) failed: ") + hipGetErrorString(err));
+      return nullptr;
+    }
+    g_scratch_ptr[dev] = ptr;
+    // the kernels that entry point launches are loaded now, so that its first
+    // call does not make the runtime allocate memory for their code either
+    prepare_pack_split_real();
+    prepare_packed_fp16tcec_s();
+    prepare_packed_bf16x3_s();
+  }
+  return g_scratch_ptr[dev];
+}
+} // namespace
+
 const Tuning &tuning() {
   std::call_once(g_tuning_once, [] { g_tuning = read_tuning_env(); });
   return g_tuning;
@@ -291,8 +328,10 @@ PreSplitChoice choose_pre_split(const cuMpSGEMM_handle *h, bool a_kc, bool b_kc,
                                 int force_cls, int force_split, int depth) {
   PreSplitChoice ch;
   if (CPLX && mode != CUMPSGEMM_FP16TCEC) return ch; // (complex: FP16TCEC only, also under FP16TCEC_SCALING)
-  // CUMPSGEMM_PACKED: "0" never, "1" whenever possible
-  const bool never = tuning().packed == 0, always = tuning().packed == 1;
+  // CUMPSGEMM_PACKED: "0" never, "1" whenever possible; the entry point that
+  // allocates nothing always goes this way (its planes have a home already)
+  const bool forced = h->ws_override != nullptr;
+  const bool never = tuning().packed == 0 && !forced, always = tuning().packed == 1 || forced;
   // bf16x3 (explicit TF32TCEC mode): its in-loop three-way split costs 5.4
   // vector instructions per MFMA, so the pre-pass pays for every layout
   ch.bf16 = (mode == CUMPSGEMM_TF32TCEC);
@@ -301,7 +340,7 @@ PreSplitChoice choose_pre_split(const cuMpSGEMM_handle *h, bool a_kc, bool b_kc,
   ch.planes = CPLX ? 4u : (ch.bf16 ? 3u : 2u);
   // (the pre-pass launches workgroups of 64 rows x 32 .. 256 K-values on a 2-D grid)
   const bool shape_ok = batch == 1 && k >= 128 &&
-                        (uint64_t)m * n >= (uint64_t)h->num_cus * ch.bm * ch.bn && k / 32 < 65535;
+                        (forced || (uint64_t)m * n >= (uint64_t)h->num_cus * ch.bm * ch.bn) && k / 32 < 65535;
   const double mn_ratio = (double)m * (double)n / ((double)m + (double)n);
   // (K = 256: 6144^2 + 8 %, 4096^2 - 4 %)
   const bool pays_nt = !a_kc && !b_kc && ((k >= 512 && mn_ratio >= 1800.0) || (k >= 256 && mn_ratio >= 2800.0));
@@ -340,6 +379,7 @@ PreSplitChoice choose_pre_split(const cuMpSGEMM_handle *h, bool a_kc, bool b_kc,
 // *failed set, the stream is broken.
 void *ensure_pack_workspace(cuMpSGEMM_handle *h, uint64_t bytes, bool *failed) {
   *failed = false;
+  if (h->ws_override != nullptr) return bytes <= h->ws_override_bytes ? h->ws_override : nullptr;
   hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
   if (hipStreamIsCapturing(h->stream, &cap) != hipSuccess) (void)hipGetLastError();
   const bool capturing = cap != hipStreamCaptureStatusNone;
@@ -764,6 +804,7 @@ hipblasStatus_t cuMpSGEMM_create(cuMpSGEMM_handle_t *handle) {
   }
   h->device = dev;
   h->num_cus = (unsigned)cus;
+  (void)scratch_address(dev); // set-up for cuMpSGEMM_sgemm_no_alloc, once per device
   bool ok = true;
   ok = ok && hipMalloc(&h->stats_slots, sizeof(StatsSlot) * h->stats_ring_length) == hipSuccess;
   ok = ok && hipMalloc(&h->stats_partials, sizeof(StatsPartial) * kMaxStatsBlocks) == hipSuccess;
@@ -903,6 +944,43 @@ hipblasStatus_t cuMpSGEMM_cgemm_ex(cuMpSGEMM_handle_t handle, hipblasOperation_t
   return cumpsgemm::gemm<hipComplex>(handle, op_A, op_B, m, n, k, alpha, a, lda, b, ldb, beta, c,
                                      ldc, mode, used_kernel_module_id);
 }
+
+hipblasStatus_t cuMpSGEMM_sgemm_no_alloc(cuMpSGEMM_handle_t handle, hipblasOperation_t op_A,
+                                         hipblasOperation_t op_B, uint64_t m, uint64_t n, uint64_t k,
+                                         const float *alpha, const float *a, uint64_t lda, const float *b,
+                                         uint64_t ldb, const float *beta, float *c, uint64_t ldc,
+                                         cuMpSGEMM_compute_mode_t mode) {
+  if (handle == nullptr) return HIPBLAS_STATUS_INVALID_VALUE;
+  if (mode != CUMPSGEMM_FP16TCEC && mode != CUMPSGEMM_TF32TCEC) {
+    log_error("cuMpSGEMM_sgemm_no_alloc serves FP16TCEC and TF32TCEC only");
+    return HIPBLAS_STATUS_INVALID_VALUE;
+  }
+  if (m == 0 || n == 0) return HIPBLAS_STATUS_SUCCESS;
+  if (k < 128 || m > 0x7fffffffull || n > 0x7fffffffull || k > 0x7fffffffull) {
+    log_error("cuMpSGEMM_sgemm_no_alloc needs 128 <= k and sizes below 2^31");
+    return HIPBLAS_STATUS_INVALID_VALUE;
+  }
+  const unsigned planes = mode == CUMPSGEMM_TF32TCEC ? 3u : 2u;
+  const unsigned long long need =
+      packed_bytes(packed_rows(m), k, planes) + packed_bytes(packed_rows(n), k, planes);
+  if (need > kStaticScratchBytes) {
+    log_error("cuMpSGEMM_sgemm_no_alloc: the split operands need " + std::to_string(need) +
+              " bytes, the static scratch holds " + std::to_string(kStaticScratchBytes) +
+              " ((m + n rounded up to 256) * (k rounded up to 32) * " + std::to_string(2 * planes) + " bytes)");
+    return HIPBLAS_STATUS_INVALID_VALUE;
+  }
+  void *const ptr = scratch_address(handle->device);
+  if (ptr == nullptr) return HIPBLAS_STATUS_NOT_INITIALIZED;
+  handle->ws_override = ptr;
+  handle->ws_override_bytes = kStaticScratchBytes;
+  const hipblasStatus_t st = cumpsgemm::gemm<float>(handle, op_A, op_B, m, n, k, alpha, a, lda, b, ldb, beta, c,
+                                                    ldc, mode, nullptr);
+  handle->ws_override = nullptr;
+  handle->ws_override_bytes = 0;
+  return st;
+}
+
+size_t cuMpSGEMM_get_static_scratch_size(void) { return (size_t)kStaticScratchBytes; }
 
 size_t cuMpSGEMM_get_workspace_size(cuMpSGEMM_handle_t handle) {
   return handle != nullptr ? (size_t)handle->pack_ws_bytes : 0;

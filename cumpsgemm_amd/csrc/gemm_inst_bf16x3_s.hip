@@ -18,5 +18,9 @@ void launch_packed_bf16x3_s(const GemmArgs &args, dim3 grid, hipStream_t stream,
         args, grid, stream);
   }
 }
+void prepare_packed_bf16x3_s() {
+  prepare_cfg<GemmCfg<Prec::BF16X3, false, true, true, 128, 128, 64, 32, 2, true, true, false, true>>();
+  prepare_cfg<GemmCfg<Prec::BF16X3, false, true, true, 128, 128, 64, 32, 2, true, false, false, true>>();
+}
 #undef ROW
 } // namespace cumpsgemm_amd

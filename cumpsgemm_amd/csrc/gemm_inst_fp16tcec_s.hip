@@ -18,6 +18,10 @@ void launch_packed_fp16tcec_s(const GemmArgs &args, dim3 grid, hipStream_t strea
         args, grid, stream);
   }
 }
+void prepare_packed_fp16tcec_s() {
+  prepare_cfg<GemmCfg<Prec::FP16TCEC, false, true, true, 256, 128, 64, 64, 2, true, true, false, true>>();
+  prepare_cfg<GemmCfg<Prec::FP16TCEC, false, true, true, 256, 128, 64, 64, 2, true, false, false, true>>();
+}
 void launch_packed_scaled_fp16tcec_s(const GemmArgs &args, dim3 grid, hipStream_t stream, bool walk) {
   if (walk) {
     launch_cfg<GemmCfg<Prec::FP16TCEC, false, true, true, 256, 128, 64, 64, 2, true, true, true, true>>(

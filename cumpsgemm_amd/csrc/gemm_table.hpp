@@ -32,6 +32,19 @@ constexpr int kNumTileClasses = 3; // 0 = large ... 2 = small
 // layout index = (a_kc ? 1 : 0) + (b_kc ? 2 : 0)
 const KernelEntry *lookup_kernel(Prec p, bool cplx, bool a_kc, bool b_kc, int cls);
 
+// Everything a first launch of this kernel would set up behind the caller's
+// back -- loading its code object onto the current device (which allocates
+// device memory) and lifting the dynamic-LDS limit -- done ahead of time.
+template <class Cfg>
+void prepare_cfg() {
+  hipFuncAttributes attr;
+  (void)hipFuncGetAttributes(&attr, reinterpret_cast<const void *>(&gemm_tcec_kernel<Cfg>));
+  if (Cfg::LDS_BYTES > 64 * 1024)
+    (void)hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_tcec_kernel<Cfg>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::LDS_BYTES);
+  (void)hipGetLastError();
+}
+
 template <class Cfg>
 void launch_cfg(const GemmArgs &args, dim3 grid, hipStream_t stream) {
   if (Cfg::LDS_BYTES > 64 * 1024) {
@@ -87,6 +100,10 @@ CUMPSGEMM_DECLARE_TABLE(g_tab_bf16x2_c)
 void launch_packed_fp16tcec_s(const GemmArgs &args, dim3 grid, hipStream_t stream, bool walk);
 void launch_packed_scaled_fp16tcec_s(const GemmArgs &args, dim3 grid, hipStream_t stream, bool walk);
 void launch_packed_bf16x3_s(const GemmArgs &args, dim3 grid, hipStream_t stream, bool walk);
+// load the real pre-split kernels (GEMM and pre-pass) onto the current device
+void prepare_packed_fp16tcec_s();
+void prepare_packed_bf16x3_s();
+void prepare_pack_split_real();
 constexpr int kPackedBM = 256, kPackedBN = 128;             // FP16TCEC
 constexpr int kPackedBf16BM = 128, kPackedBf16BN = 128;     // bf16x3
 void launch_packed_fp16tcec_c(const GemmArgs &args, dim3 grid, hipStream_t stream, bool walk, bool scaled);

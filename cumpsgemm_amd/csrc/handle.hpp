@@ -104,6 +104,12 @@ struct cuMpSGEMM_handle {
   // here), so replays of the graph keep reading and writing memory they own.
   bool pack_ws_captured = false;
   std::vector<void *> retired_ws;
+  // Set for the duration of one call by the entry point that allocates
+  // nothing: the planes go to this caller-independent buffer (a static device
+  // array), the pre-split path is taken whatever the shape rules say, and no
+  // allocation, free or synchronisation happens.
+  void *ws_override = nullptr;
+  unsigned long long ws_override_bytes = 0;
 
   // The rings, partials and workspaces above are shared by every call on the
   // handle, so work of the handle on two streams must not overlap: when the

@@ -241,6 +241,22 @@ void launch_pair_of(hipStream_t stream, const PackJob &ja, bool a_kc, const Pack
 }
 } // namespace
 
+// Loads the real pre-pass kernels onto the current device (a first launch would
+// otherwise do that, allocating device memory for the code).
+void prepare_pack_split_real() {
+  hipFuncAttributes attr;
+  auto touch = [&](auto kernel) { (void)hipFuncGetAttributes(&attr, reinterpret_cast<const void *>(kernel)); };
+  touch(pack_split_pair_kernel<true, true, Prec::FP16TCEC, false>);
+  touch(pack_split_pair_kernel<true, false, Prec::FP16TCEC, false>);
+  touch(pack_split_pair_kernel<false, true, Prec::FP16TCEC, false>);
+  touch(pack_split_pair_kernel<false, false, Prec::FP16TCEC, false>);
+  touch(pack_split_pair_kernel<true, true, Prec::BF16X3, false>);
+  touch(pack_split_pair_kernel<true, false, Prec::BF16X3, false>);
+  touch(pack_split_pair_kernel<false, true, Prec::BF16X3, false>);
+  touch(pack_split_pair_kernel<false, false, Prec::BF16X3, false>);
+  (void)hipGetLastError();
+}
+
 void launch_pack_split_pair(hipStream_t stream, const PackOperand &a, const PackOperand &b, uint32_t k,
                             PackKind kind, const int *scale_flag, const int *launch_flag,
                             uint32_t flag_accept_mask) {

@@ -24,6 +24,7 @@ struct PackOperand {
   uint32_t rows_pad;
   const uint32_t *scale_max; // nullptr: no scaling
 };
+void prepare_pack_split_real();
 void launch_pack_split_pair(hipStream_t stream, const PackOperand &a, const PackOperand &b, uint32_t k,
                             PackKind kind, const int *scale_flag = nullptr, const int *launch_flag = nullptr,
                             uint32_t flag_accept_mask = 0);

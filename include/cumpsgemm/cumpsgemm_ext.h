@@ -29,6 +29,28 @@ hipblasStatus_t cuMpSGEMM_cgemm_ex(cuMpSGEMM_handle_t handle, hipblasOperation_t
                                    hipComplex *c, uint64_t ldc, cuMpSGEMM_compute_mode_t mode,
                                    unsigned *used_kernel_module_id);
 
+/* cuMpSGEMM_sgemm for callers that cannot allocate device memory (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).
+ * No counterpart in the reference.  Same arguments and result as
+ * cuMpSGEMM_sgemm for compute_mode FP16TCEC or TF32TCEC, but the call always
+ * takes the pre-split path and keeps the fp16 / bf16 planes of A and B in a
+ * static device array inside the library instead of the handle's grow-on-demand
+ * workspace: it calls no hipMalloc / hipFree and does not synchronise.
+ * Limits: k >= 128 and
+ *   (roundup(m, 256) + roundup(n, 256)) * roundup(k, 32) * 4 bytes (6 for
+ *   TF32TCEC) <= cuMpSGEMM_get_static_scratch_size() (64 MiB);
+ * anything else returns HIPBLAS_STATUS_INVALID_VALUE with an error line.
+ * Every call on a GPU shares that GPU's array: calls that may overlap on one
+ * GPU (two streams, two handles, two threads) race and must be ordered by the
+ * caller.  Nothing in the array needs clearing between calls: the pre-pass
+ * writes every byte the GEMM kernel reads, padding included. */
+hipblasStatus_t cuMpSGEMM_sgemm_no_alloc(cuMpSGEMM_handle_t handle, hipblasOperation_t op_A,
+                                         hipblasOperation_t op_B, uint64_t m, uint64_t n, uint64_t k,
+                                         const float *alpha, const float *a, uint64_t lda,
+                                         const float *b, uint64_t ldb, const float *beta, float *c,
+                                         uint64_t ldc, cuMpSGEMM_compute_mode_t compute_mode);
+size_t cuMpSGEMM_get_static_scratch_size(void);
+
 /* Human-readable description of one tile-config table entry; 0 on success. */
 int cuMpSGEMM_describe_tile_config(int compute_mode, int is_complex, int op_A, int op_B,
                                    int tile_class, char *buf, size_t buf_len);
