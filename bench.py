@@ -53,6 +53,9 @@ def main():
     ap.add_argument("--kernel", default="gemm", choices=["gemm", "copy", "exp_stats", "exp_max", "scale", "mx2x2"],
                     help="with --kernel-only: which kernel to run (copy = a plain device copy of the "
                          "same bytes, the reference point for the HBM traffic counters)")
+    ap.add_argument("--tile-sweep", action="store_true",
+                    help="time every tile class of the table for each layout over a list of shapes (split in the "
+                         "K loop, no workspace) next to the planner's own choice; prints a table")
     ap.add_argument("--op", default="NN", choices=["NN", "TN", "NT", "TT"])
     ap.add_argument("--data", default="uniform", choices=["uniform", "zeros", "ones", "ints", "fp16"],
                     help="with --kernel-only: operand values (the part is power-limited and the MFMAs' "
@@ -76,6 +79,10 @@ def main():
 
     n = args.size
     m = k = n
+    if args.tile_sweep:
+        tile_sweep(args, torch, cg, h, dev, stream)
+        h.close()
+        return
     if args.kernel_only and args.kernel != "gemm":
         hbm_kernel_only(args, torch, cg, inputs, h, dev, stream)
         h.close()
@@ -254,6 +261,65 @@ def main():
         out["extra"] = extra
     print(json.dumps(out), flush=True)
     h.close()
+
+
+def tile_sweep(args, torch, cg, h, dev, stream):
+    """Effective TFLOP/s of each tile class (CUMPSGEMM_FORCE_TILE_CLASS) for the four layouts, with the
+    split in the K loop (CUMPSGEMM_PACKED=0), then what the planner picks on its own (same restriction)
+    and the default path (pre-split operands where the rules allow: module id 200)."""
+    L = cg.lib()
+    mode = getattr(cg, args.mode)
+
+    def setenv(**kw):
+        for key in ("CUMPSGEMM_PACKED", "CUMPSGEMM_FORCE_TILE_CLASS"):
+            os.environ.pop(key, None)
+        for key, v in kw.items():
+            os.environ["CUMPSGEMM_" + key] = v
+        L.cuMpSGEMM_reload_tuning_env()
+
+    def bench(fn, steps=6, warm=2):
+        best = None
+        for _ in range(2):
+            for _ in range(warm):
+                fn()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            for _ in range(steps):
+                fn()
+            e1.record(stream)
+            torch.cuda.synchronize()
+            t = e0.elapsed_time(e1) / steps
+            best = t if best is None else min(best, t)
+        return best
+
+    squares = [512, 768, 1024, 1280, 1536, 1792, 2048, 2560, 3072, 3584, 4096, 5120, 6144, 8192]
+    shapes = [(s, s, s) for s in squares] + [(4096, 4096, 1024), (8192, 8192, 1024), (2048, 8192, 2048),
+                                             (8192, 2048, 2048), (16384, 16384, 256), (1024, 1024, 8192),
+                                             (4096, 1024, 4096)]
+    print("| shape | layout | class 0 | class 1 | class 2 | best | planner, in-loop | default path (module id) |")
+    print("|---|---|---|---|---|---|---|---|")
+    for (m, n, k) in shapes:
+        a = torch.rand(m * k, device=dev) * 2 - 1
+        b = torch.rand(k * n, device=dev) * 2 - 1
+        c = torch.zeros(m * n, device=dev)
+        for lay, opa, opb, lda, ldb in (("NN", 111, 111, m, k), ("TN", 112, 111, k, k), ("NT", 111, 112, m, n),
+                                        ("TT", 112, 112, k, n)):
+            fn = lambda: h.gemm(opa, opb, m, n, k, 1.0, a, lda, b, ldb, 0.0, c, m, mode)
+            gf = 2.0 * m * n * k / 1e9
+            tf = []
+            for cl in range(3):
+                setenv(PACKED="0", FORCE_TILE_CLASS=str(cl))
+                tf.append(gf / bench(fn))
+            setenv(PACKED="0")
+            auto = gf / bench(fn)
+            setenv()
+            dflt = gf / bench(fn)
+            _, mid = h.gemm(opa, opb, m, n, k, 1.0, a, lda, b, ldb, 0.0, c, m, mode, want_module_id=True)
+            print(f"| {m}x{n}x{k} | {lay} | " + " | ".join(f"{x:.0f}" for x in tf) +
+                  f" | {max(range(3), key=lambda i: tf[i])} | {auto:.0f} | {dflt:.0f} ({mid}) |", flush=True)
+        del a, b, c
+    setenv()
 
 
 def hbm_kernel_only(args, torch, cg, inputs, h, dev, stream):

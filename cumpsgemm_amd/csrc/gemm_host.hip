@@ -343,7 +343,7 @@ PreSplitChoice choose_pre_split(const cuMpSGEMM_handle *h, bool a_kc, bool b_kc,
                         (forced || (uint64_t)m * n >= (uint64_t)h->num_cus * ch.bm * ch.bn) && k / 32 < 65535;
   const double mn_ratio = (double)m * (double)n / ((double)m + (double)n);
   // (K = 256: 6144^2 + 8 %, 4096^2 - 4 %)
-  const bool pays_nt = !a_kc && !b_kc && ((k >= 512 && mn_ratio >= 1800.0) || (k >= 256 && mn_ratio >= 2800.0));
+  const bool pays_nt_shape = !a_kc && !b_kc && ((k >= 512 && mn_ratio >= 1800.0) || (k >= 256 && mn_ratio >= 2800.0));
   // Every other layout: the pre-split kernel, freed of the split arithmetic,
   // outruns the in-loop one by more than the pre-pass costs once the problem
   // is large (8192^3: 381 vs 361 - 372 TFLOP/s; 8192^2 x 1024: 351 vs 318 -
@@ -353,7 +353,15 @@ PreSplitChoice choose_pre_split(const cuMpSGEMM_handle *h, bool a_kc, bool b_kc,
   const uint64_t last_round = ptiles % h->num_cus;
   const bool rounds_ok = last_round == 0 || 2 * last_round >= h->num_cus || ptiles >= 6ull * h->num_cus;
   // (complex: four times the MFMA work per element split, so the pre-pass weighs less)
-  const bool pays = pays_nt || (k >= 1024 && mn_ratio >= (CPLX ? 1500.0 : 3000.0) && rounds_ok);
+  // (5120^3, 800 tiles = 3.1 rounds: 329 TFLOP/s this way, 356 in-loop, whose planner cuts C in two)
+  const bool pays_nt = pays_nt_shape && rounds_ok;
+  // Short K, operands read through the scalar-offset loader (op_A = N) or a very
+  // large C: per tile the in-loop kernels lose more to the split than the
+  // pre-pass costs (16384^2 x 256 NN 574 -> 536 us, 12288^2 x 768 NN 739 -> 681,
+  // TN 703 -> 674; 8192^2 x 256 .. 768 and smaller: no gain).
+  const bool pays_short = !CPLX && rounds_ok &&
+                          ((k >= 256 && mn_ratio >= 8000.0 && !a_kc && b_kc) || (k >= 768 && mn_ratio >= 6000.0));
+  const bool pays = pays_nt || pays_short || (k >= 1024 && mn_ratio >= (CPLX ? 1500.0 : 3000.0) && rounds_ok);
   // With fused scaling the in-loop split costs one more instruction per pair
   // and those kernels run 8 - 25 % below the plain ones, so the pre-pass (which
   // scales as it splits) pays for every layout.
@@ -637,24 +645,41 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
   // columns, planned on their own (typically with K split to fill the chip).
   if (!split && batch == 1 && depth == 0 && !fp16_served && k >= 256 &&
       !tuning().no_column_split) {
+    // (C's rows are independent as well: the cut that leaves the cheaper pair of
+    // problems wins -- which one that is depends on the tile's aspect ratio)
     const KernelEntry *e0 = plan0.entry;
     const uint64_t slots = (uint64_t)h->num_cus * resident_groups(e0);
     const uint64_t tiles = (uint64_t)plan0.tiles_m * plan0.tiles_n;
     const uint64_t full = tiles / slots;
     const uint64_t cols1 = (full * slots) / plan0.tiles_m; // tile columns of the first part
-    if (full >= 1 && tiles % slots != 0 && cols1 >= 1 && cols1 < plan0.tiles_n) {
-      const uint64_t n1 = cols1 * (uint64_t)e0->bn, n2 = n - n1;
-      const double c1 = make_plan(h, launches[0].p, CPLX, a_kc, b_kc, m, n1, k, 1, force_cls, force_split).cost;
-      const double c2 = make_plan(h, launches[0].p, CPLX, a_kc, b_kc, m, n2, k, 1, force_cls, force_split).cost;
-      const double extra_launch = 3.0 * 256.0 * 128.0;
-      if (c1 + c2 + extra_launch < 0.93 * plan0.cost) {
-        const T *b2 = b_kc ? b + n1 * ldb : b + n1; // op(B) = N: columns of B; else rows of B^T
-        hipblasStatus_t st = run_gemm<T>(h, op_A, op_B, m, n1, k, alpha, a, lda, stridea, b, ldb, strideb,
+    const uint64_t rows1 = (full * slots) / plan0.tiles_n; // or its tile rows
+    const double extra_launch = 3.0 * 256.0 * 128.0;
+    auto cost_of = [&](uint64_t mm, uint64_t nn) {
+      return make_plan(h, launches[0].p, CPLX, a_kc, b_kc, mm, nn, k, 1, force_cls, force_split).cost;
+    };
+    double cost_cols = -1.0, cost_rows = -1.0;
+    const uint64_t n1 = cols1 * (uint64_t)e0->bn, m1 = rows1 * (uint64_t)e0->bm;
+    if (full >= 1 && tiles % slots != 0) {
+      if (cols1 >= 1 && cols1 < plan0.tiles_n) cost_cols = cost_of(m, n1) + cost_of(m, n - n1) + extra_launch;
+      if (rows1 >= 1 && rows1 < plan0.tiles_m) cost_rows = cost_of(m1, n) + cost_of(m - m1, n) + extra_launch;
+    }
+    const bool by_rows = cost_rows >= 0.0 && (cost_cols < 0.0 || cost_rows < cost_cols);
+    const double cost_cut = by_rows ? cost_rows : cost_cols;
+    if (cost_cut >= 0.0 && cost_cut < 0.93 * plan0.cost) {
+      if (by_rows) {
+        const T *a2 = a_kc ? a + m1 * lda : a + m1; // op(A) = T: columns of A^T; else rows of A
+        hipblasStatus_t st = run_gemm<T>(h, op_A, op_B, m1, n, k, alpha, a, lda, stridea, b, ldb, strideb,
                                          beta, c, ldc, stridec, 1, mode, used_id, label, 1);
         if (st != HIPBLAS_STATUS_SUCCESS) return st;
-        return run_gemm<T>(h, op_A, op_B, m, n2, k, alpha, a, lda, stridea, b2, ldb, strideb, beta,
-                           c + n1 * ldc, ldc, stridec, 1, mode, nullptr, label, 1);
+        return run_gemm<T>(h, op_A, op_B, m - m1, n, k, alpha, a2, lda, stridea, b, ldb, strideb, beta,
+                           c + m1, ldc, stridec, 1, mode, nullptr, label, 1);
       }
+      const T *b2 = b_kc ? b + n1 * ldb : b + n1; // op(B) = N: columns of B; else rows of B^T
+      hipblasStatus_t st = run_gemm<T>(h, op_A, op_B, m, n1, k, alpha, a, lda, stridea, b, ldb, strideb,
+                                       beta, c, ldc, stridec, 1, mode, used_id, label, 1);
+      if (st != HIPBLAS_STATUS_SUCCESS) return st;
+      return run_gemm<T>(h, op_A, op_B, m, n - n1, k, alpha, a, lda, stridea, b2, ldb, strideb, beta,
+                         c + n1 * ldc, ldc, stridec, 1, mode, nullptr, label, 1);
     }
   }
 
