@@ -264,7 +264,7 @@ def main():
 
 
 def tile_sweep(args, torch, cg, h, dev, stream):
-    """Effective TFLOP/s of each tile class (CUMPSGEMM_FORCE_TILE_CLASS) for the four layouts, with the
+    """Effective TFLOP/s of each tile class (CUMPSGEMM_FORCE_TILE_CLASS, 0 - 4) for the four layouts, with the
     split in the K loop (CUMPSGEMM_PACKED=0), then what the planner picks on its own (same restriction)
     and the default path (pre-split operands where the rules allow: module id 200)."""
     L = cg.lib()
@@ -296,9 +296,15 @@ def tile_sweep(args, torch, cg, h, dev, stream):
     squares = [512, 768, 1024, 1280, 1536, 1792, 2048, 2560, 3072, 3584, 4096, 5120, 6144, 8192]
     shapes = [(s, s, s) for s in squares] + [(4096, 4096, 1024), (8192, 8192, 1024), (2048, 8192, 2048),
                                              (8192, 2048, 2048), (16384, 16384, 256), (1024, 1024, 8192),
-                                             (4096, 1024, 4096)]
-    print("| shape | layout | class 0 | class 1 | class 2 | best | planner, in-loop | default path (module id) |")
-    print("|---|---|---|---|---|---|---|---|")
+                                             (4096, 1024, 4096),
+                                             # C with a few columns / rows: classes 3 and 4 (memory-bound: the
+                                             # vendor FP32 routine is the yardstick)
+                                             (8192, 8, 8192), (8192, 32, 8192), (8, 8192, 8192), (32, 8192, 8192),
+                                             (65536, 16, 1024), (16384, 4, 16384), (8192, 1, 8192)]
+    ncls = 5
+    print("| shape | layout | " + " | ".join(f"class {c}" for c in range(ncls)) +
+          " | best | planner, in-loop | default path (module id) | vendor FP32 |")
+    print("|---|---|" + "---|" * (ncls + 4))
     for (m, n, k) in shapes:
         a = torch.rand(m * k, device=dev) * 2 - 1
         b = torch.rand(k * n, device=dev) * 2 - 1
@@ -308,7 +314,7 @@ def tile_sweep(args, torch, cg, h, dev, stream):
             fn = lambda: h.gemm(opa, opb, m, n, k, 1.0, a, lda, b, ldb, 0.0, c, m, mode)
             gf = 2.0 * m * n * k / 1e9
             tf = []
-            for cl in range(3):
+            for cl in range(ncls):
                 setenv(PACKED="0", FORCE_TILE_CLASS=str(cl))
                 tf.append(gf / bench(fn))
             setenv(PACKED="0")
@@ -316,8 +322,12 @@ def tile_sweep(args, torch, cg, h, dev, stream):
             setenv()
             dflt = gf / bench(fn)
             _, mid = h.gemm(opa, opb, m, n, k, 1.0, a, lda, b, ldb, 0.0, c, m, mode, want_module_id=True)
-            print(f"| {m}x{n}x{k} | {lay} | " + " | ".join(f"{x:.0f}" for x in tf) +
-                  f" | {max(range(3), key=lambda i: tf[i])} | {auto:.0f} | {dflt:.0f} ({mid}) |", flush=True)
+            am = a.view(k, m).t() if opa == 111 else a.view(m, k)      # logical m x k over the same memory
+            bm = b.view(n, k).t() if opb == 111 else b.view(k, n)
+            vend = gf / bench(lambda: torch.matmul(am, bm))
+            print(f"| {m}x{n}x{k} | {lay} | " + " | ".join(f"{x:.1f}" if x < 10 else f"{x:.0f}" for x in tf) +
+                  f" | {max(range(ncls), key=lambda i: tf[i])} | {auto:.1f} | {dflt:.1f} ({mid}) | {vend:.1f} |",
+                  flush=True)
         del a, b, c
     setenv()
 

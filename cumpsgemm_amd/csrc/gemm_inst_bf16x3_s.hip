@@ -5,7 +5,9 @@ namespace cumpsgemm_amd {
 #define ROW(AKC, BKC) \
   { CUMPSGEMM_ENTRY(Prec::BF16X3, false, AKC, BKC, 128, 128, 64, 32, 2, true, "128x128x32_w64x32_deep"), \
     CUMPSGEMM_ENTRY(Prec::BF16X3, false, AKC, BKC, 128, 128, 64, 32, 2, true, "128x128x32_w64x32_deep"), \
-    CUMPSGEMM_ENTRY(Prec::BF16X3, false, AKC, BKC, 64, 64, 32, 32, 2, false, "64x64x32_w32x32") }
+    CUMPSGEMM_ENTRY(Prec::BF16X3, false, AKC, BKC, 64, 64, 32, 32, 2, false, "64x64x32_w32x32"), \
+    CUMPSGEMM_ENTRY(Prec::BF16X3, false, AKC, BKC, 128, 32, 32, 32, 2, true, "128x32x32_w32x32_deep"), \
+    CUMPSGEMM_ENTRY(Prec::BF16X3, false, AKC, BKC, 32, 128, 32, 32, 2, true, "32x128x32_w32x32_deep") }
 CUMPSGEMM_DEFINE_TABLE(g_tab_bf16x3_s, ROW)
 // the large tile over pre-split operands (three bf16 planes, K-contiguous);
 // `walk`: persistent form (short tiles) or one tile per workgroup

@@ -5,6 +5,8 @@ namespace cumpsgemm_amd {
 #define ROW(AKC, BKC) \
   { CUMPSGEMM_ENTRY(Prec::FP16TC, true, AKC, BKC, 128, 64, 32, 32, 2, true, "c128x64x32_w32x32_deep"), \
     CUMPSGEMM_ENTRY(Prec::FP16TC, true, AKC, BKC, 64, 64, 32, 32, 2, false, "c64x64x32_w32x32"), \
+    CUMPSGEMM_ENTRY(Prec::FP16TC, true, AKC, BKC, 64, 32, 32, 32, 1, false, "c64x32x32_w32x32"), \
+    CUMPSGEMM_ENTRY(Prec::FP16TC, true, AKC, BKC, 64, 32, 32, 32, 1, false, "c64x32x32_w32x32"), \
     CUMPSGEMM_ENTRY(Prec::FP16TC, true, AKC, BKC, 64, 32, 32, 32, 1, false, "c64x32x32_w32x32") }
 CUMPSGEMM_DEFINE_TABLE(g_tab_fp16tc_c, ROW)
 #undef ROW

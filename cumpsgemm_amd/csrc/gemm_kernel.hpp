@@ -529,6 +529,28 @@ struct tile_loader {
       int row, chunk;
       unit_coords(u, tid, row, chunk);
       const int k0 = chunk * 8;
+      if constexpr (KC) {
+        // a unit that lies inside the matrix is 8 (complex: 16) consecutive
+        // floats: wide loads, like an interior tile (a narrow operand next to a
+        // long one -- C with a few columns -- sends both through this loader)
+        if (row < rows_left && k0 + 8 <= k_left) {
+          typedef float f4u_t __attribute__((ext_vector_type(4), aligned(4)));
+          const f4u_t *p = reinterpret_cast<const f4u_t *>(base + ((uint64_t)row * ld + k0) * ES);
+          if constexpr (!CPLX) {
+            const f4u_t lo = p[0], hi = p[1];
+            reg.v[u][0][0] = lo.x; reg.v[u][0][1] = lo.y; reg.v[u][0][2] = lo.z; reg.v[u][0][3] = lo.w;
+            reg.v[u][0][4] = hi.x; reg.v[u][0][5] = hi.y; reg.v[u][0][6] = hi.z; reg.v[u][0][7] = hi.w;
+          } else {
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+              const f4u_t t = p[q];
+              reg.v[u][0][2 * q] = t.x; reg.v[u][1][2 * q] = t.y;
+              reg.v[u][0][2 * q + 1] = t.z; reg.v[u][1][2 * q + 1] = t.w;
+            }
+          }
+          continue;
+        }
+      }
 #pragma unroll
       for (int j = 0; j < 8; j++) {
         const uint64_t idx = KC ? (uint64_t)row * ld + (k0 + j) : (uint64_t)(k0 + j) * ld + row;

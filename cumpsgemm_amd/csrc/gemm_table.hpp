@@ -27,7 +27,7 @@ struct KernelEntry {
   const char *name;
 };
 
-constexpr int kNumTileClasses = 3; // 0 = large ... 2 = small
+constexpr int kNumTileClasses = 5; // 0 = large ... 2 = small, 3 = tall-skinny C, 4 = short-wide C
 
 // layout index = (a_kc ? 1 : 0) + (b_kc ? 2 : 0)
 const KernelEntry *lookup_kernel(Prec p, bool cplx, bool a_kc, bool b_kc, int cls);

@@ -265,7 +265,7 @@ def test_persistent_split_k(O, handle, dev, monkeypatch):
 # the overhang; the rows / columns it shares with its neighbour must not be updated
 # twice (beta != 0, split-K accumulation).  Forced tile classes make sure that large
 # tiles meet small overhangs.
-@pytest.mark.parametrize("cls", [0, 1, 2])
+@pytest.mark.parametrize("cls", [0, 1, 2, 3, 4])
 @pytest.mark.parametrize("cplx,opa,opb,m,n,k,alpha,beta", [
     (False, N, N, 300, 200, 160, 1.5, -0.5),     # K a multiple of 32: persistent kernels
     (False, T, N, 257, 129, 96, 1.0, 1.0),
@@ -293,6 +293,34 @@ def test_edge_tiles_split_k(O, handle, dev, monkeypatch, cls):
     ref = O.gemm_fp64(N, N, m, n, k, 1.0, a, m, b, k, 0.5, c0, m)
     cf = oracle_gemm(O, FP32, N, N, m, n, k, 1.0, a, m, b, k, 0.5, c0, m)
     assert O.residual(ref, c, m, n, m) <= 2.0 * O.residual(ref, cf, m, n, m)
+
+
+# ---- C with a few columns, or a few rows -------------------------------------------
+# Tile classes 3 (256 x 32) and 4 (32 x 256) serve products whose result is at most 32 wide or high:
+# the long operand is streamed once, K is split so that every CU has a share, the narrow operand goes
+# through the guarded loader (wide loads where a unit lies inside the matrix).
+@pytest.mark.parametrize("mode", [FP16TCEC, TF32TCEC])
+@pytest.mark.parametrize("opa,opb", [(N, N), (T, N), (N, T), (T, T)])
+@pytest.mark.parametrize("m,n,k,want_cls", [
+    (4096, 8, 4096, 3), (4100, 1, 1000, 3), (2048, 17, 515, 3), (8192, 32, 1024, 3),
+    (8, 4096, 4096, 4), (5, 3000, 777, 4), (32, 8192, 1024, 4),
+])
+def test_narrow_results_on_the_streaming_tile_classes(O, handle, dev, monkeypatch, mode, opa, opb, m, n, k, want_cls):
+    if m * n * k < 8 * 4096 * 4096:     # (the planner takes these classes on its own from about this size on)
+        monkeypatch.setenv("CUMPSGEMM_FORCE_TILE_CLASS", str(want_cls))
+    a, lda = make_operand(inputs.uniform, 61, opa, m, k, 1)
+    b, ldb = make_operand(inputs.uniform, 62, opb, k, n, 2)
+    ldc = m + 3
+    c0 = inputs.uniform(63, ldc * n)
+    c, st, mid = run_gemm(handle, dev, mode, opa, opb, m, n, k, 0.75, a, lda, b, ldb, -0.5, c0, ldc, False,
+                          want_module_id=True)
+    assert st == 0 and mid % 100 == want_cls, mid
+    ref = O.gemm_fp64(opa, opb, m, n, k, 0.75, a, lda, b, ldb, -0.5, c0, ldc)
+    cf = oracle_gemm(O, FP32, opa, opb, m, n, k, 0.75, a, lda, b, ldb, -0.5, c0, ldc)
+    co = oracle_gemm(O, mode, opa, opb, m, n, k, 0.75, a, lda, b, ldb, -0.5, c0, ldc)
+    assert O.residual(ref, c, m, n, ldc) <= 2.0 * O.residual(ref, cf, m, n, ldc) + 2.0 ** -24
+    assert rel_diff(c, co, m, n, ldc) <= 4 * 2.0 ** -24 * np.sqrt(k)
+    assert np.array_equal(c.reshape(n, ldc)[:, m:], c0.reshape(n, ldc)[:, m:])
 
 
 # ---- pre-split (packed) path ------------------------------------------------------
