@@ -495,6 +495,28 @@ struct tile_loader {
         reg.third[u] = *reinterpret_cast<const u4_t *>(p + 2u * plane_bytes + off);
     }
   }
+  // The same copy without the round trip through registers: 16-byte global ->
+  // LDS loads (gfx950).  The 64 lanes of a wave fill 1 KiB of contiguous LDS,
+  // which is what the planes' layout (the linear LDS image) asks for.  Returns
+  // nothing; completion is tracked by the wave's vector-memory counter.
+  template <int NPL>
+  __device__ static inline void dma_packed(const float *__restrict__ base, uint32_t plane_bytes, char *lds_op,
+                                           int wave) {
+    typedef const void __attribute__((address_space(1))) *gptr_t;
+    typedef void __attribute__((address_space(3))) *lptr_t;
+    constexpr int PLANE = ROWS * 64;
+    if (!active(threadIdx.x)) return;
+    const char *p = reinterpret_cast<const char *>(base);
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      const uint32_t off = (uint32_t)(threadIdx.x + u * NT) * 16u;
+#pragma unroll
+      for (int pl = 0; pl < NPL; pl++) {
+        __builtin_amdgcn_global_load_lds((gptr_t)(p + (uint32_t)pl * plane_bytes + off),
+                                         (lptr_t)(lds_op + pl * PLANE + (wave * 64 + u * NT) * 16), 16, 0, 0);
+      }
+    }
+  }
   template <int NPL>
   __device__ static inline void store_packed(Regs &reg, char *lds_op, int tid) {
     constexpr int PLANE = ROWS * 64;
@@ -1099,6 +1121,70 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
     }
   };
 
+  if constexpr (Cfg::PACKED && !Cfg::PERSIST) {
+    // ---- pre-split operands, one tile per workgroup: global -> LDS loads ------
+    // The planes go from memory straight into the LDS buffers: no staging
+    // registers, no ds_write.  In step t a wave
+    //   - asks for its share of tile t + 2 (into the buffer that tile t - 1 was
+    //     read from, free since the barrier that ended step t - 1),
+    //   - multiplies tile t (first K-slice from fragments fetched right after
+    //     that barrier, second fetched now),
+    //   - waits until its share of tile t + 1 -- asked for a whole step ago -- has
+    //     landed, then at the barrier for everybody else's.
+    // Same arithmetic in the same order as the register-staged pipeline
+    // (bit-identical results); measured against it at 8192^3: + 2 % for the
+    // fp16 kernel, + 0.5 % for bf16x3.
+    const int nk = klen / BK; // (pre-split operands are padded to whole K-steps)
+    const int last = nk - 1;
+    auto dma = [&](int kt, int stage) {
+      const int kc = kt < last ? kt : last;
+      char *sa = lds + stage * Cfg::STAGE_BYTES;
+      char *sb = sa + Cfg::A_STAGE_BYTES;
+      LA::template dma_packed<NP * NCOMP>(a_tile + (uint64_t)kc * a_kstep, (uint32_t)args.lda * 64u, sa, wave);
+      LB::template dma_packed<NP * NCOMP>(b_tile + (uint64_t)kc * b_kstep, (uint32_t)args.ldb * 64u, sb, wave);
+    };
+    // loads this wave issues per step (waves beyond the units of a small operand issue none for it)
+    constexpr int NDMA_A = Cfg::UA * NP * NCOMP, NDMA_B = Cfg::UB * NP * NCOMP;
+    static_assert(NDMA_A + NDMA_B <= 15, "vmcnt immediate");
+    const bool loads_a = LA::active(tid), loads_b = LB::active(tid); // wave-uniform
+    auto wait_previous_step = [&]() {
+      // at most this step's loads still in flight <=> the previous step's have landed
+      constexpr int KEEP = (7 << 4) | (15 << 8); // leave the other counters alone
+      if (loads_a && loads_b) __builtin_amdgcn_s_waitcnt((NDMA_A + NDMA_B) | KEEP);
+      else if (loads_a) __builtin_amdgcn_s_waitcnt(NDMA_A | KEEP);
+      else if (loads_b) __builtin_amdgcn_s_waitcnt(NDMA_B | KEEP);
+    };
+    Frags f0, f1;
+    dma(0, 0);
+    dma(1, 1);
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    int b0 = 0, b1 = 1, b2 = 2;
+    frag_load(f0, 0, 0);
+    for (int t = 0; t < nk; t++) {
+      frag_load(f1, b0, 1);
+      dma(t + 2, b2);
+      frag_mma(f0);
+      frag_mma(f1);
+      wait_previous_step();
+      // (a plain barrier: a workgroup-scope fence on LDS would make the compiler
+      // wait for the loads just issued as well; the "memory" clobber keeps it
+      // from moving the fragment reads below to this side)
+      asm volatile("s_barrier" ::: "memory");
+      const int tmp = b0;
+      b0 = b1;
+      b1 = b2;
+      b2 = tmp;
+      frag_load(f0, b0, 0); // first K-slice of the next tile (past the end: a re-read, unused)
+    }
+    __builtin_amdgcn_s_waitcnt(0);
+    if (ml0 == m0 && nl0 == n0 && rows_a == BM && rows_b == BN) {
+      epilogue(c, ml0, nl0, m0, n0, std::true_type{});
+    } else {
+      epilogue(c, ml0, nl0, m0, n0, std::false_type{});
+    }
+    return;
+  }
   if (a_full && b_full) {
     const int nk_full = klen / BK;
     if (nk_full > 0) pipeline(nk_full, std::true_type{});

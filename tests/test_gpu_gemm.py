@@ -306,8 +306,8 @@ def test_edge_tiles_split_k(O, handle, dev, monkeypatch, cls):
     (8, 4096, 4096, 4), (5, 3000, 777, 4), (32, 8192, 1024, 4),
 ])
 def test_narrow_results_on_the_streaming_tile_classes(O, handle, dev, monkeypatch, mode, opa, opb, m, n, k, want_cls):
-    if m * n * k < 8 * 4096 * 4096:     # (the planner takes these classes on its own from about this size on)
-        monkeypatch.setenv("CUMPSGEMM_FORCE_TILE_CLASS", str(want_cls))
+    # (the planner takes these classes on its own for the large ones; forced, so that the small ones run them too)
+    monkeypatch.setenv("CUMPSGEMM_FORCE_TILE_CLASS", str(want_cls))
     a, lda = make_operand(inputs.uniform, 61, opa, m, k, 1)
     b, ldb = make_operand(inputs.uniform, 62, opb, k, n, 2)
     ldc = m + 3
