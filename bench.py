@@ -56,6 +56,9 @@ def main():
     ap.add_argument("--tile-sweep", action="store_true",
                     help="time every tile class of the table for each layout over a list of shapes (split in the "
                          "K loop, no workspace) next to the planner's own choice; prints a table")
+    ap.add_argument("--shape", default=None,
+                    help="with --kernel-only: M,N,K[,BATCH] instead of a square --size (BATCH > 1: strided batch)")
+    ap.add_argument("--cplx", action="store_true", help="with --kernel-only --shape: complex64 operands (CGEMM)")
     ap.add_argument("--op", default="NN", choices=["NN", "TN", "NT", "TT"])
     ap.add_argument("--data", default="uniform", choices=["uniform", "zeros", "ones", "ints", "fp16"],
                     help="with --kernel-only: operand values (the part is power-limited and the MFMAs' "
@@ -85,6 +88,10 @@ def main():
         return
     if args.kernel_only and args.kernel != "gemm":
         hbm_kernel_only(args, torch, cg, inputs, h, dev, stream)
+        h.close()
+        return
+    if args.kernel_only and args.shape:
+        shape_kernel_only(args, torch, cg, h, dev, stream)
         h.close()
         return
     log(f"[bench] generating {n}x{n} inputs (seeds 1, 2)")
@@ -342,6 +349,44 @@ def tile_sweep(args, torch, cg, h, dev, stream):
                   flush=True)
         del a, b, c
     setenv()
+
+
+def shape_kernel_only(args, torch, cg, h, dev, stream):
+    """One GEMM call of any shape in a loop, for profilers (uniform[-1,1) operands made on the device)."""
+    dims = [int(x) for x in args.shape.split(",")]
+    m, n, k = dims[:3]
+    batch = dims[3] if len(dims) > 3 else 1
+    es = 2 if args.cplx else 1
+    opa = cg.OP_T if args.op[0] == "T" else cg.OP_N
+    opb = cg.OP_T if args.op[1] == "T" else cg.OP_N
+    lda, ldb = (m if opa == cg.OP_N else k), (k if opb == cg.OP_N else n)
+    a = torch.rand(batch * m * k * es, device=dev) * 2 - 1
+    b = torch.rand(batch * k * n * es, device=dev) * 2 - 1
+    c = torch.zeros(batch * m * n * es, device=dev)
+    mode = getattr(cg, args.mode)
+    if batch > 1:
+        fn = lambda: h.gemm_strided_batch(opa, opb, m, n, k, 1.0, a, lda, m * k, b, ldb, k * n, 0.0, c, m, m * n, batch,
+                                          mode, cplx=args.cplx)
+    else:
+        fn = lambda: h.gemm(opa, opb, m, n, k, 1.0, a, lda, b, ldb, 0.0, c, m, mode, cplx=args.cplx)
+    settle = float(os.environ.get("BENCH_SETTLE_MS", "100"))
+    t0 = time.perf_counter()
+    while (time.perf_counter() - t0) * 1e3 < settle:
+        fn()
+        torch.cuda.synchronize()
+    for _ in range(args.warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record(stream)
+    for _ in range(args.steps):
+        fn()
+    e1.record(stream)
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / args.steps
+    flops = (8.0 if args.cplx else 2.0) * m * n * k * batch
+    print(json.dumps({"kernel_only": True, "shape": [m, n, k, batch], "cplx": args.cplx, "op": args.op, "mode": args.mode,
+                      "kernel_ms": round(ms, 4), "tflops": round(flops / ms / 1e9, 2)}), flush=True)
 
 
 def hbm_kernel_only(args, torch, cg, inputs, h, dev, stream):
