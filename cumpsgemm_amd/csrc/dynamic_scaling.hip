@@ -18,7 +18,6 @@ namespace cumpsgemm_amd {
 namespace {
 constexpr int kBlock = 256;
 constexpr float kHalfExpMax = 16384.0f; // 2^14
-constexpr int kScaleABit = 0x40, kScaleBBit = 0x20, kModeMask = 0x1f;
 
 // UNSCALE_C: the inverse of SCALE_C's coefficient (see unscale_C below)
 enum ScaleKind : int { SCALE_A = 0, SCALE_B = 1, SCALE_C = 2, RESET_A = 3, RESET_B = 4, UNSCALE_C = 5 };
@@ -126,15 +125,7 @@ void launch_scaling(cuMpSGEMM_handle *h, int kind, unsigned slot_a, unsigned slo
 }
 
 __global__ void combine_flag_kernel(int *flag, const StatsSlot *a, const StatsSlot *b) {
-  const int pa = a->mode, pb = b->mode;
-  if (pa == CUMPSGEMM_TF32TCEC || pb == CUMPSGEMM_TF32TCEC) {
-    *flag = CUMPSGEMM_TF32TCEC;
-    return;
-  }
-  int f = CUMPSGEMM_FP16TCEC;
-  if (pa == CUMPSGEMM_FP16TCEC_SCALING) f |= kScaleABit;
-  if (pb == CUMPSGEMM_FP16TCEC_SCALING) f |= kScaleBBit;
-  *flag = f;
+  *flag = combine_launch_flag(a->mode, b->mode);
 }
 
 int read_flag(cuMpSGEMM_handle *h, unsigned id) {

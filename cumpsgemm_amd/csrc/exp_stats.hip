@@ -86,10 +86,38 @@ struct StatsJob {
 #if !CUMPSGEMM_STATS_STRICT_ORDER && defined(__HIP_DEVICE_COMPILE__) && !defined(__gfx950__)
 #error "the fence-free hand-over of exp_stats_kernel is written for gfx950; build with -DCUMPSGEMM_STATS_STRICT_ORDER=1"
 #endif
+// Stage 2 of a pair can also write the launch flag that the two decisions
+// give (flag_out != nullptr; the combination of src/dynamic_scaling.cu:364-385),
+// which saves the one-thread kernel that would otherwise follow, i.e. one more
+// kernel boundary per AUTO call.  Each job has one finishing thread -- thread 0
+// of its first workgroup when stage 1 has already decided and the job's
+// workgroups leave at once, thread 0 of its folding workgroup otherwise --
+// which takes a ticket of the pair once its job's slot is final; the second of
+// the two reads both decisions and writes the flag.  The hand-over between the
+// two finishing threads follows the same ordering rules as the partials.
+__device__ inline void finish_pair_job(int *flag_out, unsigned *pair_ticket, StatsSlot *slot_a,
+                                       StatsSlot *slot_b) {
+#if CUMPSGEMM_STATS_STRICT_ORDER
+  const unsigned arrived =
+      __hip_atomic_fetch_add(pair_ticket, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+#else
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  __builtin_amdgcn_s_waitcnt(0);
+  const unsigned arrived =
+      __hip_atomic_fetch_add(pair_ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#endif
+  if (arrived != 1u) return;
+  const int pa = __hip_atomic_load(&slot_a->mode, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  const int pb = __hip_atomic_load(&slot_b->mode, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  *flag_out = combine_launch_flag(pa, pb);
+  __hip_atomic_store(pair_ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 template <int MODE>
 __global__ __launch_bounds__(kBlock) void exp_stats_kernel(const StatsJob job0, const StatsJob job1,
                                                            float ignore_thr, float under_thr,
-                                                           float tolerance) {
+                                                           float tolerance, int *flag_out,
+                                                           unsigned *pair_ticket) {
   const bool second = blockIdx.x >= job0.blocks; // uniform
   const StatsJob &job = second ? job1 : job0;
   StatsSlot *const slot = job.slot;
@@ -100,7 +128,11 @@ __global__ __launch_bounds__(kBlock) void exp_stats_kernel(const StatsJob job0, 
   const unsigned m_f = job.m_f, n = job.n, nbatch = job.nbatch;
   const unsigned nblocks = job.blocks, bid = blockIdx.x - (second ? job0.blocks : 0u);
   if (MODE == 1) {
-    if (slot->mode != CUMPSGEMM_UNDEFINED) return; // uniform across the job's workgroups
+    if (slot->mode != CUMPSGEMM_UNDEFINED) { // uniform across the job's workgroups
+      if (flag_out != nullptr && bid == 0 && threadIdx.x == 0)
+        finish_pair_job(flag_out, pair_ticket, job0.slot, job1.slot);
+      return;
+    }
     const float max_exp = __uint_as_float(slot->max_exp_bits);
     ignore_thr *= max_exp;
     under_thr *= max_exp;
@@ -272,14 +304,17 @@ __global__ __launch_bounds__(kBlock) void exp_stats_kernel(const StatsJob job0, 
     } else if (MODE == 1) {
       slot->total = t;
       slot->underflow = u;
-      slot->mode = ((float)u <= (float)t * tolerance) ? CUMPSGEMM_FP16TCEC_SCALING
-                                                      : CUMPSGEMM_TF32TCEC;
+      const int decided = ((float)u <= (float)t * tolerance) ? CUMPSGEMM_FP16TCEC_SCALING
+                                                             : CUMPSGEMM_TF32TCEC;
+      // (a device-scope store: the other job's finishing thread may read it in this launch)
+      __hip_atomic_store(&slot->mode, decided, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     } else {
       slot->max_exp_bits = mxb;
     }
     // ready for the next pass on this stream
     // (the slot and the ticket become visible to later kernels at the end of this one)
     __hip_atomic_store(ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (MODE == 1 && flag_out != nullptr) finish_pair_job(flag_out, pair_ticket, job0.slot, job1.slot);
   }
 }
 
@@ -347,7 +382,7 @@ StatsJob make_job(cuMpSGEMM_handle *h, const View &v, const T *ptr, unsigned slo
 
 // MODE 0 + 1 (full statistics) or 2 (maximum only) over one job or two
 template <bool FULL>
-void launch_stats(cuMpSGEMM_handle *h, const StatsJob &j0, const StatsJob &j1) {
+void launch_stats(cuMpSGEMM_handle *h, const StatsJob &j0, const StatsJob &j1, int *flag_out = nullptr) {
   // (a null matrix would fault on the device; an empty one has nothing to read)
   const bool bad0 = j0.ptr == nullptr && j0.m_f != 0 && j0.n != 0;
   const bool bad1 = j1.blocks != 0 && j1.ptr == nullptr && j1.m_f != 0 && j1.n != 0;
@@ -360,18 +395,23 @@ void launch_stats(cuMpSGEMM_handle *h, const StatsJob &j0, const StatsJob &j1) {
     {
       ProfileScope prof(h, "exp_stats_1");
       hipLaunchKernelGGL(exp_stats_kernel<0>, grid, dim3(kBlock), 0, h->stream, j0, j1, h->ignore_threshold,
-                         h->underflow_threshold, h->underflow_tolerance_rate);
+                         h->underflow_threshold, h->underflow_tolerance_rate, (int *)nullptr,
+                         (unsigned *)nullptr);
     }
     {
       ProfileScope prof(h, "exp_stats_2");
       // stage-2 thresholds are half the stage-1 ones, times the max exponent
       // (reference src/exp_stats.cu:360-361, :205-206)
+      // (the launch flag of a pair is written by this launch when the caller asks for it)
+      const bool with_flag = flag_out != nullptr && j0.blocks != 0 && j1.blocks != 0;
       hipLaunchKernelGGL(exp_stats_kernel<1>, grid, dim3(kBlock), 0, h->stream, j0, j1, h->ignore_threshold / 2,
-                         h->underflow_threshold / 2, h->underflow_tolerance_rate);
+                         h->underflow_threshold / 2, h->underflow_tolerance_rate,
+                         with_flag ? flag_out : (int *)nullptr, h->stats_ticket + 2);
     }
   } else {
     ProfileScope prof(h, "exp_max");
-    hipLaunchKernelGGL(exp_stats_kernel<2>, grid, dim3(kBlock), 0, h->stream, j0, j1, 0.0f, 0.0f, 0.0f);
+    hipLaunchKernelGGL(exp_stats_kernel<2>, grid, dim3(kBlock), 0, h->stream, j0, j1, 0.0f, 0.0f, 0.0f,
+                       (int *)nullptr, (unsigned *)nullptr);
   }
 }
 
@@ -393,7 +433,7 @@ void run_exp_max(cuMpSGEMM_handle *h, unsigned m, unsigned n, const T *ptr, unsi
 // proportion to the sizes.
 template <class T, bool FULL>
 void run_pair(cuMpSGEMM_handle *h, const MatrixView<T> &a, unsigned slot_a, const MatrixView<T> &b,
-              unsigned slot_b) {
+              unsigned slot_b, int *flag_out = nullptr) {
   View va = make_view<T>(h, a.m, a.n, a.ld, a.batch, a.stride);
   View vb = make_view<T>(h, b.m, b.n, b.ld, b.batch, b.stride);
   const unsigned long long cap = std::min<unsigned long long>((unsigned long long)h->num_cus, kMaxStatsBlocks);
@@ -404,7 +444,8 @@ void run_pair(cuMpSGEMM_handle *h, const MatrixView<T> &a, unsigned slot_a, cons
     va.grid = std::min(va.grid, ga);
     vb.grid = std::min(vb.grid, (unsigned)cap - va.grid);
   }
-  launch_stats<FULL>(h, make_job<T>(h, va, a.ptr, slot_a, 0, 0), make_job<T>(h, vb, b.ptr, slot_b, 1, va.grid));
+  launch_stats<FULL>(h, make_job<T>(h, va, a.ptr, slot_a, 0, 0), make_job<T>(h, vb, b.ptr, slot_b, 1, va.grid),
+                     flag_out);
 }
 
 void read_slot(cuMpSGEMM_handle *h, unsigned id, StatsSlot &out) {
@@ -417,10 +458,10 @@ void read_slot(cuMpSGEMM_handle *h, unsigned id, StatsSlot &out) {
 
 template <class T>
 void exp_stats_pair(cuMpSGEMM_handle *h, const MatrixView<T> &a, const MatrixView<T> &b, unsigned &a_id,
-                    unsigned &b_id) {
+                    unsigned &b_id, int flag_id) {
   a_id = next_slot(h);
   b_id = next_slot(h);
-  run_pair<T, true>(h, a, a_id, b, b_id);
+  run_pair<T, true>(h, a, a_id, b, b_id, flag_id >= 0 ? h->flag_buffer + flag_id : nullptr);
 }
 template <class T>
 void exp_max_pair(cuMpSGEMM_handle *h, const MatrixView<T> &a, const MatrixView<T> &b, unsigned &a_id,
@@ -430,9 +471,9 @@ void exp_max_pair(cuMpSGEMM_handle *h, const MatrixView<T> &a, const MatrixView<
   run_pair<T, false>(h, a, a_id, b, b_id);
 }
 template void exp_stats_pair<float>(cuMpSGEMM_handle *, const MatrixView<float> &, const MatrixView<float> &,
-                                    unsigned &, unsigned &);
+                                    unsigned &, unsigned &, int);
 template void exp_stats_pair<hipComplex>(cuMpSGEMM_handle *, const MatrixView<hipComplex> &,
-                                         const MatrixView<hipComplex> &, unsigned &, unsigned &);
+                                         const MatrixView<hipComplex> &, unsigned &, unsigned &, int);
 template void exp_max_pair<float>(cuMpSGEMM_handle *, const MatrixView<float> &, const MatrixView<float> &,
                                   unsigned &, unsigned &);
 template void exp_max_pair<hipComplex>(cuMpSGEMM_handle *, const MatrixView<hipComplex> &,

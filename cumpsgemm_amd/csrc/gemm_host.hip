@@ -133,6 +133,7 @@ __global__ void init_rings_kernel(StatsSlot *slots, int *flags, unsigned *ticket
     flags[1] = (3 << 5) | CUMPSGEMM_FP16TCEC;
     ticket[0] = 0;
     ticket[1] = 0;
+    ticket[2] = 0;
   }
 }
 
@@ -833,7 +834,7 @@ hipblasStatus_t cuMpSGEMM_create(cuMpSGEMM_handle_t *handle) {
   bool ok = true;
   ok = ok && hipMalloc(&h->stats_slots, sizeof(StatsSlot) * h->stats_ring_length) == hipSuccess;
   ok = ok && hipMalloc(&h->stats_partials, sizeof(StatsPartial) * kMaxStatsBlocks) == hipSuccess;
-  ok = ok && hipMalloc(&h->stats_ticket, 2 * sizeof(unsigned)) == hipSuccess;
+  ok = ok && hipMalloc(&h->stats_ticket, 3 * sizeof(unsigned)) == hipSuccess;
   ok = ok && hipMalloc(&h->flag_buffer, sizeof(int) * h->flag_ring_length) == hipSuccess;
   ok = ok && hipHostMalloc(&h->host_scratch, sizeof(unsigned long long) * 4, hipHostMallocDefault) ==
                  hipSuccess;

@@ -24,6 +24,20 @@ struct StatsSlot {
 };
 static_assert(sizeof(StatsSlot) == 32, "slot layout");
 
+// Launch flag = compute mode (bits 0-4) + "scale B" (bit 5) + "scale A" (bit 6)
+// (reference src/dynamic_launch_utils.hpp:10-41), and the flag that the
+// decisions for A and B give (src/dynamic_scaling.cu:364-385): bf16x3 if
+// either matrix needs it, else FP16TCEC with a scale bit per matrix that asked
+// for scaling.
+constexpr int kScaleABit = 0x40, kScaleBBit = 0x20, kModeMask = 0x1f;
+__host__ __device__ inline int combine_launch_flag(int mode_a, int mode_b) {
+  if (mode_a == CUMPSGEMM_TF32TCEC || mode_b == CUMPSGEMM_TF32TCEC) return CUMPSGEMM_TF32TCEC;
+  int f = CUMPSGEMM_FP16TCEC;
+  if (mode_a == CUMPSGEMM_FP16TCEC_SCALING) f |= kScaleABit;
+  if (mode_b == CUMPSGEMM_FP16TCEC_SCALING) f |= kScaleBBit;
+  return f;
+}
+
 // Per-workgroup partial result of a statistics pass (device scratch).
 struct StatsPartial {
   uint32_t max_bits;
@@ -74,7 +88,7 @@ struct cuMpSGEMM_handle {
   bool exp_stats_enabled = false;
   cumpsgemm_amd::StatsSlot *stats_slots = nullptr;       // [ring_length]
   cumpsgemm_amd::StatsPartial *stats_partials = nullptr; // [kMaxStatsBlocks]
-  unsigned *stats_ticket = nullptr;                      // [2] self-resetting arrival counters
+  unsigned *stats_ticket = nullptr;                      // [3] self-resetting arrival counters (job 0, job 1, the pair)
   unsigned stats_ring_length = cumpsgemm_amd::kRingLength;
   unsigned stats_current_id = 1; // slots 0 / 1 are reserved presets
   float ignore_threshold = 0.0f;
@@ -142,9 +156,12 @@ template <class T> struct MatrixView {
   const T *ptr;
   unsigned m, n, ld, batch, stride;
 };
+// flag_id >= 0: the second pass also writes launch flag flag_id from the two
+// decisions (what set_dynamic_launch_buffer_by_exp_stats would do in a launch
+// of its own).
 template <class T>
 void exp_stats_pair(cuMpSGEMM_handle *h, const MatrixView<T> &a, const MatrixView<T> &b, unsigned &a_id,
-                    unsigned &b_id);
+                    unsigned &b_id, int flag_id = -1);
 template <class T>
 void exp_max_pair(cuMpSGEMM_handle *h, const MatrixView<T> &a, const MatrixView<T> &b, unsigned &a_id,
                   unsigned &b_id);

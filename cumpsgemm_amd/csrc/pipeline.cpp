@@ -56,9 +56,11 @@ hipblasStatus_t gemm_pipeline(cuMpSGEMM_handle_t h, hipblasOperation_t op_A,
   // by that power of two first, which the final scale_C undoes exactly.)
   const bool fused = scaled && restore_AB && !tuning().no_fused_scaling;
   if (mode == CUMPSGEMM_AUTO) {
-    exp_stats_pair<T>(h, va, vb, a_id, b_id);
+    // (the second statistics pass also writes the launch flag: the reference's
+    // set_dynamic_launch_buffer_by_exp_stats, src/cumpsgemm_cublas.cu:463-466,
+    // without a launch of its own)
     flag_id = cumpsgemm::get_next_dynamic_launch_buffer_id(h);
-    cumpsgemm::set_dynamic_launch_buffer_by_exp_stats(h, flag_id, a_id, b_id);
+    exp_stats_pair<T>(h, va, vb, a_id, b_id, (int)flag_id);
     if (!fused) {
       cumpsgemm::scale_A<T>(h, a_id, flag_id, a_rows, a_cols, a, (unsigned)lda, sb, sa_stride);
       cumpsgemm::scale_B<T>(h, b_id, flag_id, b_rows, b_cols, b, (unsigned)ldb, sb, sb_stride);

@@ -91,6 +91,35 @@ def test_auto_mode_decision_and_accuracy(O, handle, dev, case):
     assert O.residual(ref, c, m, n, m) <= 2.0 * r_fp32
 
 
+def _auto_operand(kind, seed, rows, cols, per_row):
+    if kind == "unit":      # decided by the first statistics pass: FP16TCEC
+        return inputs.uniform(seed, rows * cols, 0.25, 1.0)
+    if kind == "tiny":      # second pass: FP16TCEC with scaling
+        return (inputs.uniform(seed, rows * cols, 0.5, 1.0) * np.float32(2.0 ** -20)).astype(np.float32)
+    return inputs.exponent_spread(seed, rows, cols, per_row=per_row)  # second pass: TF32TCEC
+
+
+@pytest.mark.parametrize("size", [96, 1024])
+def test_auto_launch_flag_for_every_pair_of_decisions(O, handle, dev, size):
+    """The launch flag is written by the second statistics pass itself, by
+    whichever of the two matrices' scans finishes last -- or leaves at once
+    because the first pass had already decided.  All nine pairs of decisions,
+    with one and with many workgroups per matrix, twice on the same handle (the
+    arrival counter of the pair resets itself)."""
+    m = n = k = size
+    want = {"unit": FP16TCEC, "tiny": SCALING, "wide": TF32TCEC}
+    for rep in range(2):
+        for ka in ("unit", "tiny", "wide"):
+            for kb in ("unit", "tiny", "wide"):
+                a = _auto_operand(ka, 21 + rep, m, k, True)
+                b = _auto_operand(kb, 31 + rep, k, n, False)
+                _, _, _, ids = _pipeline(handle, dev, AUTO, N, N, m, n, k, a, b)
+                assert handle.get_exp_stats_compute_mode_level(ids[0]) == want[ka], (ka, kb, rep)
+                assert handle.get_exp_stats_compute_mode_level(ids[1]) == want[kb], (ka, kb, rep)
+                flag = handle.get_dynamic_launch_flag(ids[2])
+                assert flag == O.lib().oracle_combine_flag(want[ka], want[kb]), (ka, kb, rep)
+
+
 def test_auto_complex_batched(O, handle, dev):
     m, n, k, batch = 64, 48, 80, 3
     a = inputs.complex_normal(7, m * k * batch, 2.0 ** -19)
