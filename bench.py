@@ -352,7 +352,7 @@ def tile_sweep(args, torch, cg, h, dev, stream):
 
 
 def shape_kernel_only(args, torch, cg, h, dev, stream):
-    """One GEMM call of any shape in a loop, for profilers (uniform[-1,1) operands made on the device)."""
+    """One GEMM call of any shape in a loop, for profilers (operands made on the device: uniform[-1,1) or --data)."""
     dims = [int(x) for x in args.shape.split(",")]
     m, n, k = dims[:3]
     batch = dims[3] if len(dims) > 3 else 1
@@ -362,6 +362,14 @@ def shape_kernel_only(args, torch, cg, h, dev, stream):
     lda, ldb = (m if opa == cg.OP_N else k), (k if opb == cg.OP_N else n)
     a = torch.rand(batch * m * k * es, device=dev) * 2 - 1
     b = torch.rand(batch * k * n * es, device=dev) * 2 - 1
+    if args.data == "zeros":
+        a.zero_(), b.zero_()
+    elif args.data == "ones":
+        a.fill_(1.0), b.fill_(1.0)
+    elif args.data == "ints":
+        a, b = torch.round(a * 8), torch.round(b * 8)
+    elif args.data == "fp16":
+        a, b = a.half().float(), b.half().float()
     c = torch.zeros(batch * m * n * es, device=dev)
     mode = getattr(cg, args.mode)
     if batch > 1:
@@ -386,7 +394,7 @@ def shape_kernel_only(args, torch, cg, h, dev, stream):
     ms = e0.elapsed_time(e1) / args.steps
     flops = (8.0 if args.cplx else 2.0) * m * n * k * batch
     print(json.dumps({"kernel_only": True, "shape": [m, n, k, batch], "cplx": args.cplx, "op": args.op, "mode": args.mode,
-                      "kernel_ms": round(ms, 4), "tflops": round(flops / ms / 1e9, 2)}), flush=True)
+                      "data": args.data, "kernel_ms": round(ms, 4), "tflops": round(flops / ms / 1e9, 2)}), flush=True)
 
 
 def hbm_kernel_only(args, torch, cg, inputs, h, dev, stream):
