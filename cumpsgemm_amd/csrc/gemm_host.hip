@@ -299,7 +299,7 @@ template <> struct scalar_parts<hipComplex> {
 };
 
 // ---------------------------------------------------------------------------
-// Pre-split path (FP16TCEC real and complex, bf16x3 real): split A and B once,
+// Pre-split path (FP16TCEC real and complex; bf16x3, FP16TC and bf16x2 real): split A and B once,
 // up front, into fp16 / bf16 planes held in the handle's workspace, and run the
 // kernel that only copies them into LDS.  Results are bit-identical to the
 // in-loop split (same split, same order of accumulation).  The pre-pass is one
@@ -317,6 +317,7 @@ enum class PreSplit {
 struct PreSplitChoice {
   bool take = false;
   bool bf16 = false;      // explicit TF32TCEC: three bf16 planes
+  bool tc_only = false;   // FP16TC / TF32TC (no correction terms): one fp16 plane / two bf16 planes
   bool auto_ok = false;   // AUTO: the gated FP16TCEC candidate goes this way
   bool auto_bf16 = false; // AUTO: and so does the gated bf16x3 candidate
   int bm = 0, bn = 0;     // tile of the kernel that reads the planes
@@ -329,6 +330,7 @@ PreSplitChoice choose_pre_split(const cuMpSGEMM_handle *h, bool a_kc, bool b_kc,
                                 int force_cls, int force_split, int depth) {
   PreSplitChoice ch;
   if (CPLX && mode != CUMPSGEMM_FP16TCEC) return ch; // (complex: FP16TCEC only, also under FP16TCEC_SCALING)
+  ch.tc_only = !CPLX && (mode == CUMPSGEMM_FP16TC || mode == CUMPSGEMM_TF32TC);
   // CUMPSGEMM_PACKED: "0" never, "1" whenever possible; the entry point that
   // allocates nothing always goes this way (its planes have a home already)
   const bool forced = h->ws_override != nullptr;
@@ -338,7 +340,7 @@ PreSplitChoice choose_pre_split(const cuMpSGEMM_handle *h, bool a_kc, bool b_kc,
   ch.bf16 = (mode == CUMPSGEMM_TF32TCEC);
   ch.bm = CPLX ? kPackedCplxBM : (ch.bf16 ? kPackedBf16BM : kPackedBM);
   ch.bn = CPLX ? kPackedCplxBN : (ch.bf16 ? kPackedBf16BN : kPackedBN);
-  ch.planes = CPLX ? 4u : (ch.bf16 ? 3u : 2u);
+  ch.planes = CPLX ? 4u : (ch.bf16 ? 3u : (mode == CUMPSGEMM_FP16TC ? 1u : 2u));
   // (the pre-pass launches workgroups of 64 rows x 32 .. 256 K-values on a 2-D grid)
   const bool shape_ok = batch == 1 && k >= 128 &&
                         (forced || (uint64_t)m * n >= (uint64_t)h->num_cus * ch.bm * ch.bn) && k / 32 < 65535;
@@ -375,8 +377,19 @@ PreSplitChoice choose_pre_split(const cuMpSGEMM_handle *h, bool a_kc, bool b_kc,
   }
   // (measured: - 4 % at 3072^3, + 5 % at 4096^3, + 8 % at 6144^3, + 10 % from 8192^2 on)
   const bool pays_bf16 = k >= 512 && mn_ratio >= 2000.0;
-  const bool mode_ok = mode == CUMPSGEMM_FP16TCEC || ch.bf16 || ch.auto_ok;
-  const bool worth = ch.bf16 ? (pays_bf16 || always) : (pays || pays_scaled || always);
+  // The uncorrected modes issue a third (FP16TC) or as many (bf16x2) MFMAs per
+  // element as FP16TCEC, so the same pre-pass weighs three times as much for
+  // the former: it is taken for large square-ish problems only.
+  // Measured (in-loop -> pre-split, TFLOP/s): FP16TC 8192^3 580 - 624 -> 930 - 940, 4096^3 586 - 706 ->
+  // 852 - 870, 4096^2 x 1024 505 - 566 -> 634 - 654, 8192^2 x 512 482 - 520 -> 579 - 601, 16384^2 x 256
+  // 390 - 407 -> 461 - 480, 4096^2 x 512 level; bf16x2 8192^3 320 - 377 -> 394 - 396, 4096^2 x 1024
+  // 304 - 337 -> 348 - 355, 8192^2 x 512 275 - 308 -> 318 - 327, 4096^2 x 512 level except NT.
+  const bool pays_tc = rounds_ok && ((k >= 1024 && mn_ratio >= (mode == CUMPSGEMM_FP16TC ? 1500.0 : 2000.0)) ||
+                                     (k >= 512 && mn_ratio >= 4000.0) || (k >= 256 && mn_ratio >= 8000.0) ||
+                                     (mode == CUMPSGEMM_TF32TC && pays_nt_shape));
+  const bool mode_ok = mode == CUMPSGEMM_FP16TCEC || ch.bf16 || ch.auto_ok || ch.tc_only;
+  const bool worth = ch.bf16 ? (pays_bf16 || always)
+                             : (ch.tc_only ? (pays_tc || always) : (pays || pays_scaled || always));
   ch.take = mode_ok && !never && shape_ok && worth && force_cls <= 0 && force_split <= 1;
   // AUTO: the bf16x3 candidate gets its own (gated) pre-pass and planes behind the fp16 ones
   ch.auto_bf16 = ch.take && ch.auto_ok && pays_bf16;
@@ -513,6 +526,13 @@ PreSplit run_pre_split(cuMpSGEMM_handle *h, const GemmArgs &args, bool a_kc, boo
     ok = run(PackKind::BF16X3_REAL, pa, pb, ch.bm, ch.bn, accept, false,
              [&](const GemmArgs &g, dim3 grid, bool walk) { launch_packed_bf16x3_s(g, grid, h->stream, walk); },
              false);
+  } else if (ch.tc_only) {
+    const bool fp16 = mode == CUMPSGEMM_FP16TC;
+    ok = run(fp16 ? PackKind::FP16TC_REAL : PackKind::BF16X2_REAL, pa, pb, ch.bm, ch.bn, 0u, false,
+             [&](const GemmArgs &g, dim3 grid, bool walk) {
+               if (fp16) launch_packed_fp16tc_s(g, grid, h->stream, walk);
+               else launch_packed_bf16x2_s(g, grid, h->stream, walk);
+             }, true);
   } else {
     ok = run(PackKind::FP16_REAL, pa, pb, ch.bm, ch.bn, accept, h->fused_scaling,
              [&](const GemmArgs &g, dim3 grid, bool walk) {

@@ -10,4 +10,15 @@ namespace cumpsgemm_amd {
     CUMPSGEMM_ENTRY(Prec::BF16X2, false, AKC, BKC, 64, 64, 32, 32, 2, false, "64x64x32_w32x32") }
 CUMPSGEMM_DEFINE_TABLE(g_tab_bf16x2_s, ROW)
 #undef ROW
+// the large tile over pre-split operands (two bf16 planes, K-contiguous);
+// `walk`: persistent form (short tiles) or one tile per workgroup
+void launch_packed_bf16x2_s(const GemmArgs &args, dim3 grid, hipStream_t stream, bool walk) {
+  if (walk) {
+    launch_cfg<GemmCfg<Prec::BF16X2, false, true, true, 256, 128, 64, 64, 2, true, true, false, true>>(
+        args, grid, stream);
+  } else {
+    launch_cfg<GemmCfg<Prec::BF16X2, false, true, true, 256, 128, 64, 64, 2, true, false, false, true>>(
+        args, grid, stream);
+  }
+}
 } // namespace cumpsgemm_amd

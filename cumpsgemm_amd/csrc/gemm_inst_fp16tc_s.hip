@@ -10,4 +10,15 @@ namespace cumpsgemm_amd {
     CUMPSGEMM_ENTRY(Prec::FP16TC, false, AKC, BKC, 64, 64, 32, 32, 2, false, "64x64x32_w32x32") }
 CUMPSGEMM_DEFINE_TABLE(g_tab_fp16tc_s, ROW)
 #undef ROW
+// the large tile over pre-split operands (one fp16 plane, K-contiguous);
+// `walk`: persistent form (short tiles) or one tile per workgroup
+void launch_packed_fp16tc_s(const GemmArgs &args, dim3 grid, hipStream_t stream, bool walk) {
+  if (walk) {
+    launch_cfg<GemmCfg<Prec::FP16TC, false, true, true, 256, 128, 64, 64, 2, true, true, false, true>>(
+        args, grid, stream);
+  } else {
+    launch_cfg<GemmCfg<Prec::FP16TC, false, true, true, 256, 128, 64, 64, 2, true, false, false, true>>(
+        args, grid, stream);
+  }
+}
 } // namespace cumpsgemm_amd

@@ -237,7 +237,7 @@ template <Prec P_, bool CPLX_, bool A_KC_, bool B_KC_, int BM_, int BN_, int WM_
 struct GemmCfg {
   // (PACKED + SCALED: the operands were scaled when they were pre-split; the
   // kernel only folds the inverse scaling of C into alpha)
-  static_assert(!PACKED_ || (DEEP_ && (P_ == Prec::FP16TCEC || (P_ == Prec::BF16X3 && !CPLX_))),
+  static_assert(!PACKED_ || (DEEP_ && (P_ == Prec::FP16TCEC || !CPLX_)),
                 "packed form");
   static constexpr bool PACKED = PACKED_;
   static_assert(!PERSIST_ || DEEP_, "persistent kernels use the three-buffer pipeline");
@@ -478,7 +478,7 @@ struct tile_loader {
   template <int NPL>
   __device__ static inline void load_packed(Regs &reg, const float *__restrict__ base,
                                             uint32_t plane_bytes) {
-    static_assert(NPL == 2 || NPL == 3 || (NPL == 4 && NC == 2), "2, 3 or (complex) 2 x 2 planes");
+    static_assert((NPL >= 1 && NPL <= 3) || (NPL == 4 && NC == 2), "1, 2, 3 or (complex) 2 x 2 planes");
     if (!active(threadIdx.x)) return;
     const char *p = reinterpret_cast<const char *>(base);
 #pragma unroll
@@ -487,9 +487,11 @@ struct tile_loader {
 #pragma unroll
       for (int q = 0; q < (NPL == 4 ? 2 : 1); q++) { // complex: (re hi, re lo), (im hi, im lo)
         const float4 hi = *reinterpret_cast<const float4 *>(p + (2u * q) * plane_bytes + off);
-        const float4 lo = *reinterpret_cast<const float4 *>(p + (2u * q + 1u) * plane_bytes + off);
         reg.v[u][q][0] = hi.x; reg.v[u][q][1] = hi.y; reg.v[u][q][2] = hi.z; reg.v[u][q][3] = hi.w;
-        reg.v[u][q][4] = lo.x; reg.v[u][q][5] = lo.y; reg.v[u][q][6] = lo.z; reg.v[u][q][7] = lo.w;
+        if constexpr (NPL >= 2) {
+          const float4 lo = *reinterpret_cast<const float4 *>(p + (2u * q + 1u) * plane_bytes + off);
+          reg.v[u][q][4] = lo.x; reg.v[u][q][5] = lo.y; reg.v[u][q][6] = lo.z; reg.v[u][q][7] = lo.w;
+        }
       }
       if constexpr (NPL == 3)
         reg.third[u] = *reinterpret_cast<const u4_t *>(p + 2u * plane_bytes + off);
@@ -528,7 +530,8 @@ struct tile_loader {
       for (int q = 0; q < (NPL == 4 ? 2 : 1); q++) {
         const f8_t v = reg.v[u][q];
         *reinterpret_cast<float4 *>(lds_op + 2 * q * PLANE + off) = make_float4(v[0], v[1], v[2], v[3]);
-        *reinterpret_cast<float4 *>(lds_op + (2 * q + 1) * PLANE + off) = make_float4(v[4], v[5], v[6], v[7]);
+        if constexpr (NPL >= 2)
+          *reinterpret_cast<float4 *>(lds_op + (2 * q + 1) * PLANE + off) = make_float4(v[4], v[5], v[6], v[7]);
       }
       if constexpr (NPL == 3) *reinterpret_cast<u4_t *>(lds_op + 2 * PLANE + off) = reg.third[u];
     }

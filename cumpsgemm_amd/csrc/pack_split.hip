@@ -1,5 +1,6 @@
 // Pre-split of a whole FP32 / complex64 operand into fp16 hi / lo planes
-// (FP16TCEC) or three bf16 planes (bf16x3) for the packed kernels.  For large problems every element of A is otherwise split
+// (FP16TCEC), three or two bf16 planes (bf16x3, bf16x2) or one fp16 plane
+// (FP16TC) for the packed kernels.  For large problems every element of A is otherwise split
 // once per column of tiles (and B once per row of tiles) inside the GEMM's K
 // loop; doing it once up front takes the vector arithmetic out of that loop.
 //
@@ -10,7 +11,7 @@
 //   row < rows_pad (a multiple of 256, rows >= `rows` and K-values >= `k` are
 //   zero), and inside a row the 16-byte chunk c (8 K-values) sits at position
 //   c ^ lds_swizzle(row).
-// HBM-bound: reads 4 bytes and writes 4 (6) bytes per element.
+// HBM-bound: reads 4 bytes and writes 2 bytes per plane and element.
 #include "gemm_kernel.hpp"
 #include <algorithm>
 #include "pack_split.hpp"
@@ -265,6 +266,14 @@ void launch_pack_split_pair(hipStream_t stream, const PackOperand &a, const Pack
   switch (kind) {
   case PackKind::BF16X3_REAL:
     launch_pair_of<Prec::BF16X3, false>(stream, ja, a.k_contiguous, jb, b.k_contiguous, scale_flag, launch_flag,
+                                        flag_accept_mask);
+    break;
+  case PackKind::FP16TC_REAL:
+    launch_pair_of<Prec::FP16TC, false>(stream, ja, a.k_contiguous, jb, b.k_contiguous, scale_flag, launch_flag,
+                                        flag_accept_mask);
+    break;
+  case PackKind::BF16X2_REAL:
+    launch_pair_of<Prec::BF16X2, false>(stream, ja, a.k_contiguous, jb, b.k_contiguous, scale_flag, launch_flag,
                                         flag_accept_mask);
     break;
   case PackKind::FP16_COMPLEX:

@@ -333,7 +333,7 @@ def test_narrow_results_on_the_streaming_tile_classes(O, handle, dev, monkeypatc
     (N, T, 2304, 4100, 1000, (0, 5, 0), 1.0, 1.0),
     (T, T, 3333, 2777, 129, (2, 0, 1), -1.0, 0.25),
 ])
-@pytest.mark.parametrize("mode", [FP16TCEC, TF32TCEC])
+@pytest.mark.parametrize("mode", [FP16TCEC, TF32TCEC, FP16TC, TF32TC])
 def test_packed_path_matches_in_loop_split(O, handle, dev, monkeypatch, mode, opa, opb, m, n, k, pads, alpha, beta):
     a, lda = make_operand(inputs.uniform, 61, opa, m, k, pads[0])
     b, ldb = make_operand(inputs.uniform, 62, opb, k, n, pads[1])
@@ -348,8 +348,11 @@ def test_packed_path_matches_in_loop_split(O, handle, dev, monkeypatch, mode, op
         outs.append(c)
     assert np.array_equal(outs[0].view(np.uint32), outs[1].view(np.uint32))
     ref = O.gemm_fp64(opa, opb, m, n, k, alpha, a, lda, b, ldb, beta, c0, ldc)
-    cf = oracle_gemm(O, FP32, opa, opb, m, n, k, alpha, a, lda, b, ldb, beta, c0, ldc)
-    assert O.residual(ref, outs[0], m, n, ldc) <= 2.0 * O.residual(ref, cf, m, n, ldc)
+    if mode in (FP16TCEC, TF32TCEC):
+        cf = oracle_gemm(O, FP32, opa, opb, m, n, k, alpha, a, lda, b, ldb, beta, c0, ldc)
+        assert O.residual(ref, outs[0], m, n, ldc) <= 2.0 * O.residual(ref, cf, m, n, ldc)
+    else:  # the uncorrected modes: as accurate as one rounding of the operands to fp16 / two bf16 terms allows
+        assert O.residual(ref, outs[0], m, n, ldc) <= (2.0 ** -10 if mode == FP16TC else 2.0 ** -14)
     if pads[2]:
         assert np.array_equal(outs[0].reshape(n, ldc)[:, m:], c0.reshape(n, ldc)[:, m:])
 
@@ -433,7 +436,8 @@ def test_batch_of_large_matrices_takes_the_pre_split_path_one_by_one(cg, torch_g
         h.close()
 
 
-@pytest.mark.parametrize("mode,cplx", [(FP16TCEC, False), (TF32TCEC, False), (FP16TCEC, True)])
+@pytest.mark.parametrize("mode,cplx", [(FP16TCEC, False), (TF32TCEC, False), (FP16TCEC, True), (FP16TC, False),
+                                       (TF32TC, False)])
 def test_packed_kernels_walk_and_one_tile_forms_agree(handle, dev, monkeypatch, mode, cplx):
     """The pre-split kernels exist as persistent (tile-walking) and one-tile-per-workgroup
     forms, chosen by K; both do the same arithmetic in the same order."""
