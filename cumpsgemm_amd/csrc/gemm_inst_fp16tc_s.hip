@@ -11,13 +11,16 @@ namespace cumpsgemm_amd {
 CUMPSGEMM_DEFINE_TABLE(g_tab_fp16tc_s, ROW)
 #undef ROW
 // the large tile over pre-split operands (one fp16 plane, K-contiguous);
-// `walk`: persistent form (short tiles) or one tile per workgroup
+// `walk`: persistent form (short tiles) or one tile per workgroup.  The one-tile
+// form has a single accumulator set and no staging registers: built for four
+// waves per SIMD (96 registers), so that two workgroups share a CU and one of
+// them multiplies while the other waits at its K-step barrier.
 void launch_packed_fp16tc_s(const GemmArgs &args, dim3 grid, hipStream_t stream, bool walk) {
   if (walk) {
     launch_cfg<GemmCfg<Prec::FP16TC, false, true, true, 256, 128, 64, 64, 2, true, true, false, true>>(
         args, grid, stream);
   } else {
-    launch_cfg<GemmCfg<Prec::FP16TC, false, true, true, 256, 128, 64, 64, 2, true, false, false, true>>(
+    launch_cfg<GemmCfg<Prec::FP16TC, false, true, true, 256, 128, 64, 64, 4, true, false, false, true>>(
         args, grid, stream);
   }
 }
