@@ -329,8 +329,8 @@ PreSplitChoice choose_pre_split(const cuMpSGEMM_handle *h, bool a_kc, bool b_kc,
                                 uint64_t k, uint64_t batch, cuMpSGEMM_compute_mode_t mode,
                                 int force_cls, int force_split, int depth) {
   PreSplitChoice ch;
-  if (CPLX && mode != CUMPSGEMM_FP16TCEC) return ch; // (complex: FP16TCEC only, also under FP16TCEC_SCALING)
-  ch.tc_only = !CPLX && (mode == CUMPSGEMM_FP16TC || mode == CUMPSGEMM_TF32TC);
+  ch.tc_only = mode == CUMPSGEMM_FP16TC || mode == CUMPSGEMM_TF32TC;
+  if (CPLX && mode != CUMPSGEMM_FP16TCEC && !ch.tc_only) return ch; // (complex bf16x3 has no pre-split form)
   // CUMPSGEMM_PACKED: "0" never, "1" whenever possible; the entry point that
   // allocates nothing always goes this way (its planes have a home already)
   const bool forced = h->ws_override != nullptr;
@@ -340,7 +340,7 @@ PreSplitChoice choose_pre_split(const cuMpSGEMM_handle *h, bool a_kc, bool b_kc,
   ch.bf16 = (mode == CUMPSGEMM_TF32TCEC);
   ch.bm = CPLX ? kPackedCplxBM : (ch.bf16 ? kPackedBf16BM : kPackedBM);
   ch.bn = CPLX ? kPackedCplxBN : (ch.bf16 ? kPackedBf16BN : kPackedBN);
-  ch.planes = CPLX ? 4u : (ch.bf16 ? 3u : (mode == CUMPSGEMM_FP16TC ? 1u : 2u));
+  ch.planes = (CPLX ? 2u : 1u) * (ch.bf16 ? 3u : (mode == CUMPSGEMM_FP16TC ? 1u : 2u));
   // (the pre-pass launches workgroups of 64 rows x 32 .. 256 K-values on a 2-D grid)
   const bool shape_ok = batch == 1 && k >= 128 &&
                         (forced || (uint64_t)m * n >= (uint64_t)h->num_cus * ch.bm * ch.bn) && k / 32 < 65535;
@@ -384,9 +384,16 @@ PreSplitChoice choose_pre_split(const cuMpSGEMM_handle *h, bool a_kc, bool b_kc,
   // 852 - 870, 4096^2 x 1024 505 - 566 -> 634 - 654, 8192^2 x 512 482 - 520 -> 579 - 601, 16384^2 x 256
   // 390 - 407 -> 461 - 480, 4096^2 x 512 level; bf16x2 8192^3 320 - 377 -> 394 - 396, 4096^2 x 1024
   // 304 - 337 -> 348 - 355, 8192^2 x 512 275 - 308 -> 318 - 327, 4096^2 x 512 level except NT.
-  const bool pays_tc = rounds_ok && ((k >= 1024 && mn_ratio >= (mode == CUMPSGEMM_FP16TC ? 1500.0 : 2000.0)) ||
-                                     (k >= 512 && mn_ratio >= 4000.0) || (k >= 256 && mn_ratio >= 8000.0) ||
-                                     (mode == CUMPSGEMM_TF32TC && pays_nt_shape));
+  // Complex (the 128x64 kernels): FP16TC 4096^3 560 - 678 -> 872 - 891, 2048^3 525 - 640 -> 760 - 779,
+  // 8192^2 x 256 477 - 543 -> 624 - 643; bf16x2 4096^3 350 -> 375, 4096^2 x 1024 333 - 339 -> 365,
+  // 4096^2 x 512 303 - 326 -> 336 - 347.
+  const bool pays_tc =
+      rounds_ok &&
+      (CPLX ? (mode == CUMPSGEMM_FP16TC ? (k >= 256 && mn_ratio >= 1000.0)
+                                        : ((k >= 512 && mn_ratio >= 1500.0) || (k >= 256 && mn_ratio >= 4000.0)))
+            : ((k >= 1024 && mn_ratio >= (mode == CUMPSGEMM_FP16TC ? 1500.0 : 2000.0)) ||
+               (k >= 512 && mn_ratio >= 4000.0) || (k >= 256 && mn_ratio >= 8000.0) ||
+               (mode == CUMPSGEMM_TF32TC && pays_nt_shape)));
   const bool mode_ok = mode == CUMPSGEMM_FP16TCEC || ch.bf16 || ch.auto_ok || ch.tc_only;
   const bool worth = ch.bf16 ? (pays_bf16 || always)
                              : (ch.tc_only ? (pays_tc || always) : (pays || pays_scaled || always));
@@ -461,9 +468,10 @@ PreSplit run_pre_split(cuMpSGEMM_handle *h, const GemmArgs &args, bool a_kc, boo
 
   const float *af = reinterpret_cast<const float *>(a), *bf = reinterpret_cast<const float *>(b);
   const int *gate = ch.auto_ok ? args.launch_flag : nullptr;
+  constexpr int kWalkDefault = 0, kWalkShort = 1, kWalkAlways = 2; // which K ranges the persistent form serves
   // one candidate: pre-pass of both operands, then the kernel over their planes
   auto run = [&](PackKind kind, char *pa, char *pb, int bm, int bn, uint32_t accept, bool scaled,
-                 auto launch_kernel, bool walk_short_only) -> bool {
+                 auto launch_kernel, int walk_rule) -> bool {
     GemmArgs pargs = args;
     const uint32_t *max_a = nullptr, *max_b = nullptr;
     const int *sflag = nullptr;
@@ -501,7 +509,10 @@ PreSplit run_pre_split(cuMpSGEMM_handle *h, const GemmArgs &args, bool a_kc, boo
     // short tiles are walked by persistent workgroups, long ones get a workgroup each
     // (measured cross-over: 16 K-steps for the fp16 kernel, which gains 6 - 8 % from
     // the one-tile form at 8192^3, the usual 32 for bf16x3, which gains nothing)
-    bool walk = walk_short_only ? pargs.k / 32 < 16 : pargs.k / 32 <= persistent_max_steps();
+    // (the complex 128x64 kernels with four accumulator sets: the walking form at every K -- 4096^3
+    // 350 against 308 TFLOP/s for FP16TCEC, 375 against 311 for bf16x2 in the one-tile form)
+    bool walk = walk_rule == kWalkAlways ? true
+                : (walk_rule == kWalkShort ? pargs.k / 32 < 16 : pargs.k / 32 <= persistent_max_steps());
     if (tuning().packed_walk >= 0) walk = tuning().packed_walk == 1;
     const dim3 grid = walk ? dim3((unsigned)std::min<uint64_t>(total, h->num_cus), 1, 1)
                            : dim3((unsigned)total, 1, 1);
@@ -518,27 +529,36 @@ PreSplit run_pre_split(cuMpSGEMM_handle *h, const GemmArgs &args, bool a_kc, boo
   const uint32_t accept = ch.auto_ok ? accept_fp16 : 0u;
   bool ok;
   if constexpr (CPLX) {
-    ok = run(PackKind::FP16_COMPLEX, pa, pb, ch.bm, ch.bn, accept, h->fused_scaling,
-             [&](const GemmArgs &g, dim3 grid, bool walk) {
-               launch_packed_fp16tcec_c(g, grid, h->stream, walk, h->fused_scaling);
-             }, false);
+    if (ch.tc_only) {
+      const bool fp16 = mode == CUMPSGEMM_FP16TC;
+      ok = run(fp16 ? PackKind::FP16TC_COMPLEX : PackKind::BF16X2_COMPLEX, pa, pb, ch.bm, ch.bn, 0u, false,
+               [&](const GemmArgs &g, dim3 grid, bool walk) {
+                 if (fp16) launch_packed_fp16tc_c(g, grid, h->stream, walk);
+                 else launch_packed_bf16x2_c(g, grid, h->stream, walk);
+               }, fp16 ? kWalkShort : kWalkAlways);
+    } else {
+      ok = run(PackKind::FP16_COMPLEX, pa, pb, ch.bm, ch.bn, accept, h->fused_scaling,
+               [&](const GemmArgs &g, dim3 grid, bool walk) {
+                 launch_packed_fp16tcec_c(g, grid, h->stream, walk, h->fused_scaling);
+               }, kWalkAlways);
+    }
   } else if (ch.bf16) {
     ok = run(PackKind::BF16X3_REAL, pa, pb, ch.bm, ch.bn, accept, false,
              [&](const GemmArgs &g, dim3 grid, bool walk) { launch_packed_bf16x3_s(g, grid, h->stream, walk); },
-             false);
+             kWalkDefault);
   } else if (ch.tc_only) {
     const bool fp16 = mode == CUMPSGEMM_FP16TC;
     ok = run(fp16 ? PackKind::FP16TC_REAL : PackKind::BF16X2_REAL, pa, pb, ch.bm, ch.bn, 0u, false,
              [&](const GemmArgs &g, dim3 grid, bool walk) {
                if (fp16) launch_packed_fp16tc_s(g, grid, h->stream, walk);
                else launch_packed_bf16x2_s(g, grid, h->stream, walk);
-             }, true);
+             }, kWalkShort);
   } else {
     ok = run(PackKind::FP16_REAL, pa, pb, ch.bm, ch.bn, accept, h->fused_scaling,
              [&](const GemmArgs &g, dim3 grid, bool walk) {
                if (h->fused_scaling) launch_packed_scaled_fp16tcec_s(g, grid, h->stream, walk);
                else launch_packed_fp16tcec_s(g, grid, h->stream, walk);
-             }, true);
+             }, kWalkShort);
   }
   if (!ok) return PreSplit::FAILED;
   if (used_id != nullptr) *used_id = 200u; // pre-split path
@@ -549,7 +569,7 @@ PreSplit run_pre_split(cuMpSGEMM_handle *h, const GemmArgs &args, bool a_kc, boo
     char *pa3 = pb + b_bytes, *pb3 = pa3 + a3_bytes;
     ok = run(PackKind::BF16X3_REAL, pa3, pb3, kPackedBf16BM, kPackedBf16BN, accept_bf16, false,
              [&](const GemmArgs &g, dim3 grid, bool walk) { launch_packed_bf16x3_s(g, grid, h->stream, walk); },
-             false);
+             kWalkDefault);
     if (!ok) return PreSplit::FAILED;
   }
   if (used_id != nullptr) *used_id = ~0u; // AUTO

@@ -10,4 +10,10 @@ namespace cumpsgemm_amd {
     CUMPSGEMM_ENTRY(Prec::BF16X2, true, AKC, BKC, 64, 32, 32, 32, 1, false, "c64x32x32_w32x32") }
 CUMPSGEMM_DEFINE_TABLE(g_tab_bf16x2_c, ROW)
 #undef ROW
+// the large complex tile over pre-split operands (planes re hi, re lo, im hi,
+// im lo; K-contiguous); `walk`: persistent form or one tile per workgroup
+void launch_packed_bf16x2_c(const GemmArgs &args, dim3 grid, hipStream_t stream, bool walk) {
+  if (walk) launch_cfg<GemmCfg<Prec::BF16X2, true, true, true, 128, 64, 32, 32, 2, true, true, false, true>>(args, grid, stream);
+  else launch_cfg<GemmCfg<Prec::BF16X2, true, true, true, 128, 64, 32, 32, 2, true, false, false, true>>(args, grid, stream);
+}
 } // namespace cumpsgemm_amd

@@ -237,7 +237,7 @@ template <Prec P_, bool CPLX_, bool A_KC_, bool B_KC_, int BM_, int BN_, int WM_
 struct GemmCfg {
   // (PACKED + SCALED: the operands were scaled when they were pre-split; the
   // kernel only folds the inverse scaling of C into alpha)
-  static_assert(!PACKED_ || (DEEP_ && (P_ == Prec::FP16TCEC || !CPLX_)),
+  static_assert(!PACKED_ || (DEEP_ && (P_ != Prec::BF16X3 || !CPLX_)),
                 "packed form");
   static constexpr bool PACKED = PACKED_;
   static_assert(!PERSIST_ || DEEP_, "persistent kernels use the three-buffer pipeline");

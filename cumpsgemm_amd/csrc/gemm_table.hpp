@@ -103,6 +103,8 @@ void launch_packed_bf16x3_s(const GemmArgs &args, dim3 grid, hipStream_t stream,
 // the uncorrected modes, 256x128 tile: one fp16 plane (FP16TC), two bf16 planes (TF32TC's stand-in)
 void launch_packed_fp16tc_s(const GemmArgs &args, dim3 grid, hipStream_t stream, bool walk);
 void launch_packed_bf16x2_s(const GemmArgs &args, dim3 grid, hipStream_t stream, bool walk);
+void launch_packed_fp16tc_c(const GemmArgs &args, dim3 grid, hipStream_t stream, bool walk);  // complex, 128x64
+void launch_packed_bf16x2_c(const GemmArgs &args, dim3 grid, hipStream_t stream, bool walk);
 // load the real pre-split kernels (GEMM and pre-pass) onto the current device
 void prepare_packed_fp16tcec_s();
 void prepare_packed_bf16x3_s();

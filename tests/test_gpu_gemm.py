@@ -363,7 +363,9 @@ def test_packed_path_matches_in_loop_split(O, handle, dev, monkeypatch, mode, op
     (N, T, 1280, 2100, 520, (0, 5, 0), 1.0, 1.0),
     (T, C, 1700, 1500, 129, (2, 0, 1), -1.0j, 0.25),
 ])
-def test_complex_packed_path_matches_in_loop_split(O, handle, dev, monkeypatch, opa, opb, m, n, k, pads, alpha, beta):
+@pytest.mark.parametrize("mode", [FP16TCEC, FP16TC, TF32TC])
+def test_complex_packed_path_matches_in_loop_split(O, handle, dev, monkeypatch, mode, opa, opb, m, n, k, pads, alpha,
+                                                   beta):
     gen = _gen(True)
     a, lda = make_operand(gen, 65, opa, m, k, pads[0])
     b, ldb = make_operand(gen, 66, opb, k, n, pads[1])
@@ -372,14 +374,17 @@ def test_complex_packed_path_matches_in_loop_split(O, handle, dev, monkeypatch, 
     outs = []
     for packed in ("1", "0"):
         monkeypatch.setenv("CUMPSGEMM_PACKED", packed)
-        c, st, mid = run_gemm(handle, dev, FP16TCEC, opa, opb, m, n, k, alpha, a, lda, b, ldb, beta, c0, ldc, True,
+        c, st, mid = run_gemm(handle, dev, mode, opa, opb, m, n, k, alpha, a, lda, b, ldb, beta, c0, ldc, True,
                               want_module_id=True)
         assert st == 0 and (mid == 200) == (packed == "1")
         outs.append(c)
     assert np.array_equal(outs[0].view(np.uint32), outs[1].view(np.uint32))
     ref = O.gemm_fp64(opa, opb, m, n, k, alpha, a, lda, b, ldb, beta, c0, ldc)
-    cf = oracle_gemm(O, FP32, opa, opb, m, n, k, alpha, a, lda, b, ldb, beta, c0, ldc)
-    assert O.residual(ref, outs[0], m, n, ldc) <= 2.0 * O.residual(ref, cf, m, n, ldc)
+    if mode == FP16TCEC:
+        cf = oracle_gemm(O, FP32, opa, opb, m, n, k, alpha, a, lda, b, ldb, beta, c0, ldc)
+        assert O.residual(ref, outs[0], m, n, ldc) <= 2.0 * O.residual(ref, cf, m, n, ldc)
+    else:
+        assert O.residual(ref, outs[0], m, n, ldc) <= (2.0 ** -10 if mode == FP16TC else 2.0 ** -14)
     if pads[2]:
         assert np.array_equal(outs[0].reshape(n, ldc)[:, m:], c0.reshape(n, ldc)[:, m:])
 
@@ -437,7 +442,7 @@ def test_batch_of_large_matrices_takes_the_pre_split_path_one_by_one(cg, torch_g
 
 
 @pytest.mark.parametrize("mode,cplx", [(FP16TCEC, False), (TF32TCEC, False), (FP16TCEC, True), (FP16TC, False),
-                                       (TF32TC, False)])
+                                       (TF32TC, False), (FP16TC, True), (TF32TC, True)])
 def test_packed_kernels_walk_and_one_tile_forms_agree(handle, dev, monkeypatch, mode, cplx):
     """The pre-split kernels exist as persistent (tile-walking) and one-tile-per-workgroup
     forms, chosen by K; both do the same arithmetic in the same order."""
