@@ -375,8 +375,9 @@ PreSplitChoice choose_pre_split(const cuMpSGEMM_handle *h, bool a_kc, bool b_kc,
   if (!CPLX && mode == CUMPSGEMM_AUTO && pays_scaled && depth == 0) {
     ch.auto_ok = make_plan(h, Prec::BF16X3, CPLX, a_kc, b_kc, m, n, k, batch, force_cls, force_split).ksplit == 1;
   }
-  // (measured: - 4 % at 3072^3, + 5 % at 4096^3, + 8 % at 6144^3, + 10 % from 8192^2 on)
-  const bool pays_bf16 = k >= 512 && mn_ratio >= 2000.0;
+  // (measured against the in-loop 256x128 class: - 3 % at 4096^3 and 4096^2 x 8192, - 6 % at 5120^3,
+  // + 8 % at 6144^3 and 6144^2 x 1024, + 4 - 7 % from 8192^2 x 512 on)
+  const bool pays_bf16 = k >= 512 && mn_ratio >= 3000.0;
   // The uncorrected modes issue a third (FP16TC) or as many (bf16x2) MFMAs per
   // element as FP16TCEC, so the same pre-pass weighs three times as much for
   // the former: it is taken for large square-ish problems only.

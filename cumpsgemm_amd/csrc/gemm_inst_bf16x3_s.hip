@@ -3,7 +3,7 @@
 #include "gemm_table.hpp"
 namespace cumpsgemm_amd {
 #define ROW(AKC, BKC) \
-  { CUMPSGEMM_ENTRY(Prec::BF16X3, false, AKC, BKC, 128, 128, 64, 32, 2, true, "128x128x32_w64x32_deep"), \
+  { CUMPSGEMM_ENTRY(Prec::BF16X3, false, AKC, BKC, 256, 128, 64, 64, 2, false, "256x128x32_w64x64"), \
     CUMPSGEMM_ENTRY(Prec::BF16X3, false, AKC, BKC, 128, 128, 64, 32, 2, true, "128x128x32_w64x32_deep"), \
     CUMPSGEMM_ENTRY(Prec::BF16X3, false, AKC, BKC, 64, 64, 32, 32, 2, false, "64x64x32_w32x32"), \
     CUMPSGEMM_ENTRY(Prec::BF16X3, false, AKC, BKC, 128, 32, 32, 32, 2, true, "128x32x32_w32x32_deep"), \
