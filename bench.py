@@ -503,7 +503,10 @@ def full_suite(torch, cg, inputs, h, dev, stream, timed, log, a, b, c, with_cpu)
         x32, y32 = (A32.t() if opa == cg.OP_T else A32), (B32.t() if opb == cg.OP_T else B32)
         vwall, _ = timed(lambda: torch.matmul(x32, y32), 6, 2)
         verr = rel_err(torch.matmul(x32, y32).double(), ref)
-        for mode_name, mode, prods in (("FP16TCEC", cg.FP16TCEC, 3), ("bf16x3", cg.TF32TCEC, 6)):
+        modes = [("FP16TCEC", cg.FP16TCEC, 3), ("bf16x3", cg.TF32TCEC, 6)]
+        if name == "NN":                     # the modes without correction terms, for scale (one layout)
+            modes += [("FP16TC", cg.FP16TC, 1), ("bf16x2", cg.TF32TC, 3)]
+        for mode_name, mode, prods in modes:
             if name == "NN" and mode_name == "FP16TCEC":
                 continue                     # the headline itself
             log(f"[bench] C2 {name} {mode_name}")
@@ -512,7 +515,9 @@ def full_suite(torch, cg, inputs, h, dev, stream, timed, log, a, b, c, with_cpu)
             res[f"C2_{name}_{mode_name}"] = {
                 "tflops": round(2.0 * n ** 3 / wall / 1e9, 2), "rel_error": rel_err(c.view(n, n).t().double(), ref),
                 "vendor_fp32_matmul_tflops": round(2.0 * n ** 3 / vwall / 1e9, 2), "rel_error_vendor_fp32": verr,
-                "dtype": "f16 hi/lo" if prods == 3 else "bf16 three-term split (stands in for TF32TCEC)",
+                "dtype": {"FP16TCEC": "f16 hi/lo", "bf16x3": "bf16 three-term split (stands in for TF32TCEC)",
+                          "FP16TC": "f16, no correction terms (FP16TC)",
+                          "bf16x2": "bf16 two-term split (stands in for TF32TC)"}[mode_name],
                 "roofline": mfma_roofline(2.0 * n ** 3, ev, prods, "pack_split_pair_kernel + gemm_tcec_kernel (packed)")}
         del ref
     del A, B, A32, B32
