@@ -364,7 +364,10 @@ PreSplitChoice choose_pre_split(const cuMpSGEMM_handle *h, bool a_kc, bool b_kc,
   // TN 703 -> 674; 8192^2 x 256 .. 768 and smaller: no gain).
   const bool pays_short = !CPLX && rounds_ok &&
                           ((k >= 256 && mn_ratio >= 8000.0 && !a_kc && b_kc) || (k >= 768 && mn_ratio >= 6000.0));
-  const bool pays = pays_nt || pays_short || (k >= 1024 && mn_ratio >= (CPLX ? 1500.0 : 3000.0) && rounds_ok);
+  // (complex, in-loop -> pre-split: 4096^3 340 -> 415 TFLOP/s, 2048^3 322 -> 375, 4096^2 x 512 304 -> 359,
+  // 8192^2 x 384 304 -> 357, 4096^2 x 256 level)
+  const bool pays = CPLX ? (k >= 384 && mn_ratio >= 1000.0 && rounds_ok)
+                         : (pays_nt || pays_short || (k >= 1024 && mn_ratio >= 3000.0 && rounds_ok));
   // With fused scaling the in-loop split costs one more instruction per pair
   // and those kernels run 8 - 25 % below the plain ones, so the pre-pass (which
   // scales as it splits) pays for every layout.
@@ -390,8 +393,7 @@ PreSplitChoice choose_pre_split(const cuMpSGEMM_handle *h, bool a_kc, bool b_kc,
   // 4096^2 x 512 303 - 326 -> 336 - 347.
   const bool pays_tc =
       rounds_ok &&
-      (CPLX ? (mode == CUMPSGEMM_FP16TC ? (k >= 256 && mn_ratio >= 1000.0)
-                                        : ((k >= 512 && mn_ratio >= 1500.0) || (k >= 256 && mn_ratio >= 4000.0)))
+      (CPLX ? (k >= 256 && mn_ratio >= 1000.0)
             : ((k >= 1024 && mn_ratio >= (mode == CUMPSGEMM_FP16TC ? 1500.0 : 2000.0)) ||
                (k >= 512 && mn_ratio >= 4000.0) || (k >= 256 && mn_ratio >= 8000.0) ||
                (mode == CUMPSGEMM_TF32TC && pays_nt_shape)));
@@ -469,7 +471,7 @@ PreSplit run_pre_split(cuMpSGEMM_handle *h, const GemmArgs &args, bool a_kc, boo
 
   const float *af = reinterpret_cast<const float *>(a), *bf = reinterpret_cast<const float *>(b);
   const int *gate = ch.auto_ok ? args.launch_flag : nullptr;
-  constexpr int kWalkDefault = 0, kWalkShort = 1, kWalkAlways = 2; // which K ranges the persistent form serves
+  constexpr int kWalkDefault = 0, kWalkShort = 1, kWalkNever = 2; // which K ranges the persistent form serves
   // one candidate: pre-pass of both operands, then the kernel over their planes
   auto run = [&](PackKind kind, char *pa, char *pb, int bm, int bn, uint32_t accept, bool scaled,
                  auto launch_kernel, int walk_rule) -> bool {
@@ -510,9 +512,10 @@ PreSplit run_pre_split(cuMpSGEMM_handle *h, const GemmArgs &args, bool a_kc, boo
     // short tiles are walked by persistent workgroups, long ones get a workgroup each
     // (measured cross-over: 16 K-steps for the fp16 kernel, which gains 6 - 8 % from
     // the one-tile form at 8192^3, the usual 32 for bf16x3, which gains nothing)
-    // (the complex 128x64 kernels with four accumulator sets: the walking form at every K -- 4096^3
-    // 350 against 308 TFLOP/s for FP16TCEC, 375 against 311 for bf16x2 in the one-tile form)
-    bool walk = walk_rule == kWalkAlways ? true
+    // (complex 4096^3: 414 - 416 against 358 TFLOP/s for FP16TCEC, 436 against 372 for bf16x2, 1000 against
+    // 826 for FP16TC in the one-tile form)
+    // (... and 4096^2 x 512 359 against 332, 4096^2 x 256 level: the complex kernels never walk)
+    bool walk = walk_rule == kWalkNever ? false
                 : (walk_rule == kWalkShort ? pargs.k / 32 < 16 : pargs.k / 32 <= persistent_max_steps());
     if (tuning().packed_walk >= 0) walk = tuning().packed_walk == 1;
     const dim3 grid = walk ? dim3((unsigned)std::min<uint64_t>(total, h->num_cus), 1, 1)
@@ -536,12 +539,12 @@ PreSplit run_pre_split(cuMpSGEMM_handle *h, const GemmArgs &args, bool a_kc, boo
                [&](const GemmArgs &g, dim3 grid, bool walk) {
                  if (fp16) launch_packed_fp16tc_c(g, grid, h->stream, walk);
                  else launch_packed_bf16x2_c(g, grid, h->stream, walk);
-               }, fp16 ? kWalkShort : kWalkAlways);
+               }, kWalkNever);
     } else {
       ok = run(PackKind::FP16_COMPLEX, pa, pb, ch.bm, ch.bn, accept, h->fused_scaling,
                [&](const GemmArgs &g, dim3 grid, bool walk) {
                  launch_packed_fp16tcec_c(g, grid, h->stream, walk, h->fused_scaling);
-               }, kWalkAlways);
+               }, kWalkNever);
     }
   } else if (ch.bf16) {
     ok = run(PackKind::BF16X3_REAL, pa, pb, ch.bm, ch.bn, accept, false,

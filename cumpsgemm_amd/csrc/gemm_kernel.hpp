@@ -507,18 +507,38 @@ struct tile_loader {
     typedef const void __attribute__((address_space(1))) *gptr_t;
     typedef void __attribute__((address_space(3))) *lptr_t;
     constexpr int PLANE = ROWS * 64;
-    if (!active(threadIdx.x)) return;
     const char *p = reinterpret_cast<const char *>(base);
+    if constexpr (!PARTIAL) {
 #pragma unroll
-    for (int u = 0; u < U; u++) {
-      const uint32_t off = (uint32_t)(threadIdx.x + u * NT) * 16u;
+      for (int u = 0; u < U; u++) {
+        const uint32_t off = (uint32_t)(threadIdx.x + u * NT) * 16u;
 #pragma unroll
-      for (int pl = 0; pl < NPL; pl++) {
+        for (int pl = 0; pl < NPL; pl++) {
+          __builtin_amdgcn_global_load_lds((gptr_t)(p + (uint32_t)pl * plane_bytes + off),
+                                           (lptr_t)(lds_op + pl * PLANE + (wave * 64 + u * NT) * 16), 16, 0, 0);
+        }
+      }
+    } else {
+      // Fewer chunks per plane than threads: the threads form NT / (ROWS * 4)
+      // groups and each group takes its share of the planes, so that every wave
+      // issues the same number of loads and waits for them with the same
+      // constant -- idle waves or masked lanes would put branches into the K loop
+      // and with them an end to the interleaving of its LDS reads and MFMAs.
+      constexpr int GROUPS = NT / (ROWS * 4);
+      static_assert(NT % (ROWS * 4) == 0 && (ROWS * 4) % 64 == 0 && NPL % GROUPS == 0, "plane groups");
+      const int group = wave / ((ROWS * 4) / 64);   // wave-uniform
+      const int wave_in = wave % ((ROWS * 4) / 64);
+      const uint32_t off = (uint32_t)(threadIdx.x % (ROWS * 4)) * 16u;
+#pragma unroll
+      for (int i = 0; i < NPL / GROUPS; i++) {
+        const int pl = group * (NPL / GROUPS) + i;
         __builtin_amdgcn_global_load_lds((gptr_t)(p + (uint32_t)pl * plane_bytes + off),
-                                         (lptr_t)(lds_op + pl * PLANE + (wave * 64 + u * NT) * 16), 16, 0, 0);
+                                         (lptr_t)(lds_op + pl * PLANE + wave_in * 64 * 16), 16, 0, 0);
       }
     }
   }
+  // global -> LDS loads that dma_packed issues per wave
+  template <int NPL> static constexpr int dma_loads() { return PARTIAL ? NPL / (NT / (ROWS * 4)) : U * NPL; }
   template <int NPL>
   __device__ static inline void store_packed(Regs &reg, char *lds_op, int tid) {
     constexpr int PLANE = ROWS * 64;
@@ -1146,16 +1166,13 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
       LA::template dma_packed<NP * NCOMP>(a_tile + (uint64_t)kc * a_kstep, (uint32_t)args.lda * 64u, sa, wave);
       LB::template dma_packed<NP * NCOMP>(b_tile + (uint64_t)kc * b_kstep, (uint32_t)args.ldb * 64u, sb, wave);
     };
-    // loads this wave issues per step (waves beyond the units of a small operand issue none for it)
-    constexpr int NDMA_A = Cfg::UA * NP * NCOMP, NDMA_B = Cfg::UB * NP * NCOMP;
+    // loads every wave issues per step
+    constexpr int NDMA_A = LA::template dma_loads<NP * NCOMP>(), NDMA_B = LB::template dma_loads<NP * NCOMP>();
     static_assert(NDMA_A + NDMA_B <= 15, "vmcnt immediate");
-    const bool loads_a = LA::active(tid), loads_b = LB::active(tid); // wave-uniform
     auto wait_previous_step = [&]() {
       // at most this step's loads still in flight <=> the previous step's have landed
       constexpr int KEEP = (7 << 4) | (15 << 8); // leave the other counters alone
-      if (loads_a && loads_b) __builtin_amdgcn_s_waitcnt((NDMA_A + NDMA_B) | KEEP);
-      else if (loads_a) __builtin_amdgcn_s_waitcnt(NDMA_A | KEEP);
-      else if (loads_b) __builtin_amdgcn_s_waitcnt(NDMA_B | KEEP);
+      __builtin_amdgcn_s_waitcnt((NDMA_A + NDMA_B) | KEEP);
     };
     Frags f0, f1;
     dma(0, 0);
