@@ -251,3 +251,16 @@ def test_python_control_module_drives_the_preloaded_library(cg):
     assert out[4] == "1"               # both removed: back to the rule
     assert out[5] == "abc,N,N,1,2,3,1,FP16TCEC" and out[6] == "''"
     assert out[7] == "True" and out[8] == "256 64" and out[9] == "9 5"
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """The benchmark is a one-GPU program: asking for more exits with a message and no JSON line."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True,
+                       timeout=120)
+    assert r.returncode != 0
+    assert "ONE GPU" in (r.stderr + r.stdout)
+    assert '"metric"' not in r.stdout
