@@ -369,17 +369,29 @@ __device__ inline void map_tile_batched(uint32_t vid, uint32_t tiles_m, uint32_t
 // in scalar registers, the offsets are computed once per kernel.
 // Out-of-range elements read as zero, which contributes nothing to the sums.
 // ---------------------------------------------------------------------------
-template <bool CPLX, bool KC, int ROWS, int U, int NT>
+template <bool CPLX, bool KC, int ROWS, int U, int NT, bool HALF_UNITS = false>
 struct tile_loader {
   static constexpr int NC = CPLX ? 2 : 1;
   static constexpr int ES = CPLX ? 2 : 1;
   static constexpr bool PARTIAL = (ROWS * 4) < NT; // fewer units than threads
+  // A complex operand with half as many units as threads: every thread takes
+  // half a unit (4 of its 8 K-values; the workgroup's first half the lower
+  // four, its second half the upper four), so that all waves have the same
+  // work and the K loop no branch around an idle half.
+  // (HALF_UNITS: the precisions this pays for, measured -- FP16TCEC and bf16x2; the
+  // costlier bf16x3 split and the single-product FP16TC kernels keep whole units)
+  static constexpr bool HALF = HALF_UNITS && CPLX && (ROWS * 4 * 2 == NT);
+  static constexpr int KV = HALF ? 4 : 8; // K-values a thread handles per unit
 
   // whether this thread stages anything of this operand (wave-uniform)
-  __device__ static inline bool active(int tid) { return !PARTIAL || tid < ROWS * 4; }
+  __device__ static inline bool active(int tid) { return !PARTIAL || HALF || tid < ROWS * 4; }
+  // ... in the register-staged copy of pre-split planes (whole 16-byte chunks)
+  __device__ static inline bool copy_active(int tid) { return !PARTIAL || tid < ROWS * 4; }
+  // which half of its unit (wave-uniform; 0 unless HALF)
+  __device__ static inline int half_of(int tid) { return HALF ? tid / (ROWS * 4) : 0; }
 
   __device__ static inline void unit_coords(int u, int tid, int &row, int &chunk) {
-    const int id = tid + u * NT;
+    const int id = (HALF ? tid % (ROWS * 4) : tid) + u * NT;
     if constexpr (KC) {
       chunk = id & 3;
       row = id >> 2;
@@ -393,7 +405,8 @@ struct tile_loader {
   __device__ static inline uint32_t unit_offset(int u, int tid, uint32_t ld) {
     int row, chunk;
     unit_coords(u, tid, row, chunk);
-    return KC ? (uint32_t)row * ld + (uint32_t)chunk * 8 : (uint32_t)chunk * 8 * ld + (uint32_t)row;
+    const uint32_t k0 = (uint32_t)chunk * 8 + (uint32_t)half_of(tid) * 4;
+    return KC ? (uint32_t)row * ld + k0 : k0 * ld + (uint32_t)row;
   }
 
   // whether every per-thread byte offset of a tile fits 32 bits
@@ -438,7 +451,7 @@ struct tile_loader {
           reg.v[u][0][4] = hi.x; reg.v[u][0][5] = hi.y; reg.v[u][0][6] = hi.z; reg.v[u][0][7] = hi.w;
         } else {
 #pragma unroll
-          for (int q = 0; q < 4; q++) {
+          for (int q = 0; q < KV / 2; q++) {
             const f4u_t t = p[q];
             reg.v[u][0][2 * q] = t.x; reg.v[u][1][2 * q] = t.y;
             reg.v[u][0][2 * q + 1] = t.z; reg.v[u][1][2 * q + 1] = t.w;
@@ -452,7 +465,7 @@ struct tile_loader {
 #pragma unroll
       for (int u = 0; u < U; u++) {
 #pragma unroll
-        for (int j = 0; j < 8; j++) {
+        for (int j = 0; j < KV; j++) {
           if constexpr (!CPLX) {
             reg.v[u][0][j] = __builtin_bit_cast(
                 float, __builtin_amdgcn_raw_buffer_load_b32(rsrc, boff[u], j * line, 0));
@@ -479,7 +492,7 @@ struct tile_loader {
   __device__ static inline void load_packed(Regs &reg, const float *__restrict__ base,
                                             uint32_t plane_bytes) {
     static_assert((NPL >= 1 && NPL <= 3) || (NPL == 4 && NC == 2), "1, 2, 3 or (complex) 2 x 2 planes");
-    if (!active(threadIdx.x)) return;
+    if (!copy_active(threadIdx.x)) return;
     const char *p = reinterpret_cast<const char *>(base);
 #pragma unroll
     for (int u = 0; u < U; u++) {
@@ -542,7 +555,7 @@ struct tile_loader {
   template <int NPL>
   __device__ static inline void store_packed(Regs &reg, char *lds_op, int tid) {
     constexpr int PLANE = ROWS * 64;
-    if (!active(tid)) return;
+    if (!copy_active(tid)) return;
 #pragma unroll
     for (int u = 0; u < U; u++) {
       const int off = (tid + u * NT) * 16;
@@ -573,12 +586,12 @@ struct tile_loader {
     for (int u = 0; u < U; u++) {
       int row, chunk;
       unit_coords(u, tid, row, chunk);
-      const int k0 = chunk * 8;
+      const int k0 = chunk * 8 + half_of(tid) * 4;
       if constexpr (KC) {
         // a unit that lies inside the matrix is 8 (complex: 16) consecutive
         // floats: wide loads, like an interior tile (a narrow operand next to a
         // long one -- C with a few columns -- sends both through this loader)
-        if (row < rows_left && k0 + 8 <= k_left) {
+        if (row < rows_left && k0 + KV <= k_left) {
           typedef float f4u_t __attribute__((ext_vector_type(4), aligned(4)));
           const f4u_t *p = reinterpret_cast<const f4u_t *>(base + ((uint64_t)row * ld + k0) * ES);
           if constexpr (!CPLX) {
@@ -587,7 +600,7 @@ struct tile_loader {
             reg.v[u][0][4] = hi.x; reg.v[u][0][5] = hi.y; reg.v[u][0][6] = hi.z; reg.v[u][0][7] = hi.w;
           } else {
 #pragma unroll
-            for (int q = 0; q < 4; q++) {
+            for (int q = 0; q < KV / 2; q++) {
               const f4u_t t = p[q];
               reg.v[u][0][2 * q] = t.x; reg.v[u][1][2 * q] = t.y;
               reg.v[u][0][2 * q + 1] = t.z; reg.v[u][1][2 * q + 1] = t.w;
@@ -597,7 +610,7 @@ struct tile_loader {
         }
       }
 #pragma unroll
-      for (int j = 0; j < 8; j++) {
+      for (int j = 0; j < KV; j++) {
         const uint64_t idx = KC ? (uint64_t)row * ld + (k0 + j) : (uint64_t)(k0 + j) * ld + row;
         float tx = 0.0f, ty = 0.0f;
         if (row < rows_left && k0 + j < k_left) {
@@ -629,6 +642,29 @@ struct tile_loader {
       unit_coords(u, tid, row, chunk);
       f8_t part[2];
       fetch(reg, u, part[0], part[1]);
+      if constexpr (HALF) {
+        // four K-values per component: the lower half of each plane chunk is
+        // computed (the upper half of the staging vector is unused) and written
+        // as 8 bytes into this thread's half of the chunk
+#pragma unroll
+        for (int c = 0; c < NC; c++) {
+#pragma unroll
+          for (int j = 4; j < 8; j++) part[c][j] = 0.0f;
+          u4_t out[NP];
+          if constexpr (SCALED) {
+            splitter<P>::run_scaled(part[c], out, s, s2048);
+          } else {
+            splitter<P>::run(part[c], out);
+          }
+#pragma unroll
+          for (int p = 0; p < NP; p++) {
+            typedef uint32_t u2v_t __attribute__((ext_vector_type(2)));
+            const u2v_t lo2 = {out[p][0], out[p][1]};
+            *reinterpret_cast<u2v_t *>(lds_op + (c * NP + p) * PLANE + lds_offset(row, chunk) + half_of(tid) * 8) = lo2;
+          }
+        }
+        continue;
+      }
 #pragma unroll
       for (int c = 0; c < NC; c++) {
         u4_t out[NP];
@@ -749,8 +785,9 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
   const uint64_t b_kstep = Cfg::PACKED ? (uint64_t)(NP * NCOMP) * args.ldb * 16
                            : Cfg::B_KC ? (uint64_t)BK * ES : (uint64_t)BK * args.ldb * ES;
 
-  using LA = tile_loader<CPLX, Cfg::A_KC, BM, Cfg::UA, NT>;
-  using LB = tile_loader<CPLX, Cfg::B_KC, BN, Cfg::UB, NT>;
+  constexpr bool HALF_UNITS = (P == Prec::FP16TCEC || P == Prec::BF16X2);
+  using LA = tile_loader<CPLX, Cfg::A_KC, BM, Cfg::UA, NT, HALF_UNITS>;
+  using LB = tile_loader<CPLX, Cfg::B_KC, BN, Cfg::UB, NT, HALF_UNITS>;
 
   const int rows_a = (int)((args.m - ml0 < (uint32_t)BM) ? args.m - ml0 : BM);
   const int rows_b = (int)((args.n - nl0 < (uint32_t)BN) ? args.n - nl0 : BN);
