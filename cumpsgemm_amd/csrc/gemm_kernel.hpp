@@ -375,9 +375,10 @@ struct tile_loader {
   static constexpr int ES = CPLX ? 2 : 1;
   static constexpr bool PARTIAL = (ROWS * 4) < NT; // fewer units than threads
   // A complex operand with half as many units as threads: every thread takes
-  // half a unit (4 of its 8 K-values; the workgroup's first half the lower
-  // four, its second half the upper four), so that all waves have the same
-  // work and the K loop no branch around an idle half.
+  // half a unit (4 of its 8 K-values; even threads the lower four, odd threads
+  // the upper four, so that a pair of lanes fills one 16-byte chunk of a plane
+  // and a wave's 8-byte LDS writes cover all banks), so that all waves have the
+  // same work and the K loop no branch around an idle half.
   // (HALF_UNITS: the precisions this pays for, measured -- FP16TCEC and bf16x2; the
   // costlier bf16x3 split and the single-product FP16TC kernels keep whole units)
   static constexpr bool HALF = HALF_UNITS && CPLX && (ROWS * 4 * 2 == NT);
@@ -387,11 +388,11 @@ struct tile_loader {
   __device__ static inline bool active(int tid) { return !PARTIAL || HALF || tid < ROWS * 4; }
   // ... in the register-staged copy of pre-split planes (whole 16-byte chunks)
   __device__ static inline bool copy_active(int tid) { return !PARTIAL || tid < ROWS * 4; }
-  // which half of its unit (wave-uniform; 0 unless HALF)
-  __device__ static inline int half_of(int tid) { return HALF ? tid / (ROWS * 4) : 0; }
+  // which half of its unit (0 unless HALF)
+  __device__ static inline int half_of(int tid) { return HALF ? (tid & 1) : 0; }
 
   __device__ static inline void unit_coords(int u, int tid, int &row, int &chunk) {
-    const int id = (HALF ? tid % (ROWS * 4) : tid) + u * NT;
+    const int id = (HALF ? tid >> 1 : tid) + u * NT;
     if constexpr (KC) {
       chunk = id & 3;
       row = id >> 2;
