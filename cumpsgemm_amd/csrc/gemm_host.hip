@@ -358,16 +358,16 @@ PreSplitChoice choose_pre_split(const cuMpSGEMM_handle *h, bool a_kc, bool b_kc,
   // (complex: four times the MFMA work per element split, so the pre-pass weighs less)
   // (5120^3, 800 tiles = 3.1 rounds: 329 TFLOP/s this way, 356 in-loop, whose planner cuts C in two)
   const bool pays_nt = pays_nt_shape && rounds_ok;
-  // Short K, operands read through the scalar-offset loader (op_A = N) or a very
-  // large C: per tile the in-loop kernels lose more to the split than the
-  // pre-pass costs (16384^2 x 256 NN 574 -> 536 us, 12288^2 x 768 NN 739 -> 681,
-  // TN 703 -> 674; 8192^2 x 256 .. 768 and smaller: no gain).
+  // Short K: per tile the in-loop kernels lose more to the split than the pre-pass
+  // costs once C is large (in-loop -> pre-split, TFLOP/s: 16384^2 x 256 271 -> 297, 16384^2 x 512 313 -> 347,
+  // 8192^2 x 512 317 -> 328, 8192^2 x 768 332 -> 352, 6144^2 x 512 279 -> 291; 8192^2 x 256 and 6144^2 x 256
+  // stay in-loop: 271 / 243 against 267 / 228, and so does 4096^2 below K = 2048).
   const bool pays_short = !CPLX && rounds_ok &&
-                          ((k >= 256 && mn_ratio >= 8000.0 && !a_kc && b_kc) || (k >= 768 && mn_ratio >= 6000.0));
+                          ((k >= 256 && mn_ratio >= 8000.0) || (k >= 512 && mn_ratio >= 3000.0));
   // (complex, in-loop -> pre-split: 4096^3 340 -> 415 TFLOP/s, 2048^3 322 -> 375, 4096^2 x 512 304 -> 359,
   // 8192^2 x 384 304 -> 357, 4096^2 x 256 level)
   const bool pays = CPLX ? (k >= 384 && mn_ratio >= 1000.0 && rounds_ok)
-                         : (pays_nt || pays_short || (k >= 1024 && mn_ratio >= 3000.0 && rounds_ok));
+                         : (pays_nt || pays_short || (k >= 2048 && mn_ratio >= 2000.0 && rounds_ok));
   // With fused scaling the in-loop split costs one more instruction per pair
   // and those kernels run 8 - 25 % below the plain ones, so the pre-pass (which
   // scales as it splits) pays for every layout.
@@ -471,7 +471,7 @@ PreSplit run_pre_split(cuMpSGEMM_handle *h, const GemmArgs &args, bool a_kc, boo
 
   const float *af = reinterpret_cast<const float *>(a), *bf = reinterpret_cast<const float *>(b);
   const int *gate = ch.auto_ok ? args.launch_flag : nullptr;
-  constexpr int kWalkDefault = 0, kWalkShort = 1, kWalkNever = 2; // which K ranges the persistent form serves
+  constexpr int kWalkAlways = 0, kWalkShort = 1, kWalkNever = 2; // which K ranges the persistent form serves
   // one candidate: pre-pass of both operands, then the kernel over their planes
   auto run = [&](PackKind kind, char *pa, char *pb, int bm, int bn, uint32_t accept, bool scaled,
                  auto launch_kernel, int walk_rule) -> bool {
@@ -515,8 +515,10 @@ PreSplit run_pre_split(cuMpSGEMM_handle *h, const GemmArgs &args, bool a_kc, boo
     // (complex 4096^3: 414 - 416 against 358 TFLOP/s for FP16TCEC, 436 against 372 for bf16x2, 1000 against
     // 826 for FP16TC in the one-tile form)
     // (... and 4096^2 x 512 359 against 332, 4096^2 x 256 level: the complex kernels never walk)
+    // (real FP16TCEC / bf16x3 / bf16x2: the tile-walking form with global -> LDS loads at every K --
+    // 8192^3 381 - 384 against 365 - 368 TFLOP/s, 16384^2 x 1024 374 against 353, 16384^2 x 256 297 against 262)
     bool walk = walk_rule == kWalkNever ? false
-                : (walk_rule == kWalkShort ? pargs.k / 32 < 16 : pargs.k / 32 <= persistent_max_steps());
+                : (walk_rule == kWalkAlways ? true : pargs.k / 32 < 16);
     if (tuning().packed_walk >= 0) walk = tuning().packed_walk == 1;
     const dim3 grid = walk ? dim3((unsigned)std::min<uint64_t>(total, h->num_cus), 1, 1)
                            : dim3((unsigned)total, 1, 1);
@@ -549,20 +551,20 @@ PreSplit run_pre_split(cuMpSGEMM_handle *h, const GemmArgs &args, bool a_kc, boo
   } else if (ch.bf16) {
     ok = run(PackKind::BF16X3_REAL, pa, pb, ch.bm, ch.bn, accept, false,
              [&](const GemmArgs &g, dim3 grid, bool walk) { launch_packed_bf16x3_s(g, grid, h->stream, walk); },
-             kWalkDefault);
+             kWalkAlways);
   } else if (ch.tc_only) {
     const bool fp16 = mode == CUMPSGEMM_FP16TC;
     ok = run(fp16 ? PackKind::FP16TC_REAL : PackKind::BF16X2_REAL, pa, pb, ch.bm, ch.bn, 0u, false,
              [&](const GemmArgs &g, dim3 grid, bool walk) {
                if (fp16) launch_packed_fp16tc_s(g, grid, h->stream, walk);
                else launch_packed_bf16x2_s(g, grid, h->stream, walk);
-             }, kWalkShort);
+             }, fp16 ? kWalkShort : kWalkAlways); // (FP16TC: two one-tile workgroups per CU from 16 K-steps on)
   } else {
     ok = run(PackKind::FP16_REAL, pa, pb, ch.bm, ch.bn, accept, h->fused_scaling,
              [&](const GemmArgs &g, dim3 grid, bool walk) {
                if (h->fused_scaling) launch_packed_scaled_fp16tcec_s(g, grid, h->stream, walk);
                else launch_packed_fp16tcec_s(g, grid, h->stream, walk);
-             }, kWalkShort);
+             }, kWalkAlways);
   }
   if (!ok) return PreSplit::FAILED;
   if (used_id != nullptr) *used_id = 200u; // pre-split path
@@ -573,7 +575,7 @@ PreSplit run_pre_split(cuMpSGEMM_handle *h, const GemmArgs &args, bool a_kc, boo
     char *pa3 = pb + b_bytes, *pb3 = pa3 + a3_bytes;
     ok = run(PackKind::BF16X3_REAL, pa3, pb3, kPackedBf16BM, kPackedBf16BN, accept_bf16, false,
              [&](const GemmArgs &g, dim3 grid, bool walk) { launch_packed_bf16x3_s(g, grid, h->stream, walk); },
-             kWalkDefault);
+             kWalkAlways);
     if (!ok) return PreSplit::FAILED;
   }
   if (used_id != nullptr) *used_id = ~0u; // AUTO

@@ -335,7 +335,7 @@ __device__ inline void map_tile(uint32_t bid, uint32_t tiles_m, uint32_t tiles_n
 // whole list, so that one XCD works on neighbouring tiles of one matrix.
 __device__ inline void map_tile_batched(uint32_t vid, uint32_t tiles_m, uint32_t tiles_n,
                                         uint32_t batch, uint32_t &tm, uint32_t &tn,
-                                        uint32_t &bat) {
+                                        uint32_t &bat, const uint32_t GROUP = 8) {
   const uint32_t per_batch = tiles_m * tiles_n;
   const uint32_t total = per_batch * batch;
   constexpr uint32_t NXCD = 8;
@@ -347,7 +347,6 @@ __device__ inline void map_tile_batched(uint32_t vid, uint32_t tiles_m, uint32_t
   }
   bat = id / per_batch;
   id -= bat * per_batch;
-  constexpr uint32_t GROUP = 8;
   const uint32_t per_group = GROUP * tiles_n;
   const uint32_t g = id / per_group;
   const uint32_t first_m = g * GROUP;
@@ -740,7 +739,9 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
   // (persistent kernels: the first tile of this workgroup's list; see below)
   uint32_t tile_m, tile_n, tile_b = blockIdx.y;
   if constexpr (Cfg::PERSIST) {
-    map_tile_batched(blockIdx.x, args.tiles_m, args.tiles_n, args.batch, tile_m, tile_n, tile_b);
+    // (the walk over pre-split real operands takes its column-group height from the host)
+    const uint32_t group = (Cfg::PACKED && !CPLX && args.raster_group) ? args.raster_group : 8u;
+    map_tile_batched(blockIdx.x, args.tiles_m, args.tiles_n, args.batch, tile_m, tile_n, tile_b, group);
   } else {
     map_tile(blockIdx.x, args.tiles_m, args.tiles_n, tile_m, tile_n, args.raster_group ? args.raster_group : 8u);
   }
@@ -1009,6 +1010,83 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
             for (int v = 0; v < 16; v++) acc[q][s][j][i][v] = 0.0f;
   };
 
+  if constexpr (Cfg::PERSIST && Cfg::PACKED && !CPLX) {
+    // ---- persistent walk over pre-split operands with global -> LDS loads -----
+    // One workgroup walks its list of tiles; the planes of step t + 2 are asked
+    // for before the MFMAs of step t, across tile boundaries.  The first step of
+    // a tile is peeled off the K loop: the stores of the previous tile's
+    // write-out stand between its loads and the next ones in the (in-order)
+    // vector-memory counter, so its wait differs -- as a constant, not a branch.
+    const uint32_t total = args.tiles_m * args.tiles_n * args.batch;
+    const uint32_t my_tiles = (total - blockIdx.x + gridDim.x - 1) / gridDim.x;
+    const int nk = klen / BK;
+    auto tile_at = [&](uint32_t i, const float *&at, const float *&bt, float *&ct, uint32_t &om0, uint32_t &on0) {
+      uint32_t tm, tn, bat;
+      map_tile_batched(blockIdx.x + (i < my_tiles ? i : my_tiles - 1) * gridDim.x, args.tiles_m,
+                       args.tiles_n, args.batch, tm, tn, bat, args.raster_group ? args.raster_group : 8u);
+      om0 = tm * BM;
+      on0 = tn * BN;
+      at = packed_origin(reinterpret_cast<const float *>(args.a), args.lda, om0);
+      bt = packed_origin(reinterpret_cast<const float *>(args.b), args.ldb, on0);
+      ct = reinterpret_cast<float *>(args.c);
+    };
+    constexpr int NDMA = LA::template dma_loads<NP * NCOMP>() + LB::template dma_loads<NP * NCOMP>();
+    constexpr int KEEP = (7 << 4) | (15 << 8);
+    const float *la = a_tile, *lb = b_tile, *la_next, *lb_next;
+    float *c_cur = c, *c_ignored;
+    uint32_t cm0 = m0, cn0 = n0, i0, i1;
+    tile_at(1, la_next, lb_next, c_ignored, i0, i1);
+    int lk = 0;
+    auto dma_next = [&](int stage) {
+      char *sa = lds + stage * Cfg::STAGE_BYTES;
+      char *sb = sa + Cfg::A_STAGE_BYTES;
+      LA::template dma_packed<NP * NCOMP>(la, (uint32_t)args.lda * 64u, sa, wave);
+      LB::template dma_packed<NP * NCOMP>(lb, (uint32_t)args.ldb * 64u, sb, wave);
+      lk++;
+      const bool wrap = (lk == nk);
+      la = wrap ? la_next : la + a_kstep;
+      lb = wrap ? lb_next : lb + b_kstep;
+      lk = wrap ? 0 : lk;
+    };
+    Frags f0, f1;
+    int b0 = 0, b1 = 1, b2 = 2;
+    // one K-step; WAIT: vector-memory operations that may still be in flight
+    // when the next step's planes are needed
+    auto step = [&](auto wait_tag) {
+      constexpr int WAIT = decltype(wait_tag)::value;
+      frag_load(f1, b0, 1);
+      dma_next(b2);
+      frag_mma(f0);
+      frag_mma(f1);
+      __builtin_amdgcn_s_waitcnt(WAIT | KEEP);
+      asm volatile("s_barrier" ::: "memory");
+      const int tmp = b0;
+      b0 = b1;
+      b1 = b2;
+      b2 = tmp;
+      frag_load(f0, b0, 0);
+    };
+    dma_next(0);
+    dma_next(1);
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    frag_load(f0, 0, 0);
+    for (uint32_t ct = 0; ct < my_tiles; ct++) {
+      // (after a write-out: its 64 stores were issued behind the loads of this
+      // tile's second step, so "at most 63 in flight" covers them)
+      step(std::integral_constant<int, (NDMA + 64 > 63 ? 63 : NDMA + 64)>{});
+      for (int kk = 1; kk < nk; kk++) step(std::integral_constant<int, NDMA>{});
+      const bool interior = cm0 + BM <= args.m && cn0 + BN <= args.n;
+      if (interior) epilogue(c_cur, cm0, cn0, cm0, cn0, std::true_type{});
+      else epilogue(c_cur, cm0, cn0, cm0, cn0, std::false_type{});
+      zero_acc();
+      const float *ua, *ub;
+      tile_at(ct + 1, ua, ub, c_cur, cm0, cn0);
+      tile_at(ct + 2, la_next, lb_next, c_ignored, i0, i1);
+    }
+    __builtin_amdgcn_s_waitcnt(0);
+    return;
+  }
   if constexpr (Cfg::PERSIST) {
     // ---- persistent walk over this workgroup's tiles ----------------------
     // Tile i of the list is virtual workgroup blockIdx.x + i * gridDim.x.  The
