@@ -471,7 +471,7 @@ PreSplit run_pre_split(cuMpSGEMM_handle *h, const GemmArgs &args, bool a_kc, boo
 
   const float *af = reinterpret_cast<const float *>(a), *bf = reinterpret_cast<const float *>(b);
   const int *gate = ch.auto_ok ? args.launch_flag : nullptr;
-  constexpr int kWalkAlways = 0, kWalkShort = 1, kWalkNever = 2; // which K ranges the persistent form serves
+  constexpr int kWalkAlways = 0, kWalkShort = 1, kWalkNever = 2, kWalkMid = 3; // K ranges of the persistent form
   // one candidate: pre-pass of both operands, then the kernel over their planes
   auto run = [&](PackKind kind, char *pa, char *pb, int bm, int bn, uint32_t accept, bool scaled,
                  auto launch_kernel, int walk_rule) -> bool {
@@ -509,16 +509,14 @@ PreSplit run_pre_split(cuMpSGEMM_handle *h, const GemmArgs &args, bool a_kc, boo
     pargs.launch_flag = gate;
     pargs.flag_accept_mask = accept;
     const uint64_t total = (uint64_t)pargs.tiles_m * pargs.tiles_n;
-    // short tiles are walked by persistent workgroups, long ones get a workgroup each
-    // (measured cross-over: 16 K-steps for the fp16 kernel, which gains 6 - 8 % from
-    // the one-tile form at 8192^3, the usual 32 for bf16x3, which gains nothing)
-    // (complex 4096^3: 414 - 416 against 358 TFLOP/s for FP16TCEC, 436 against 372 for bf16x2, 1000 against
-    // 826 for FP16TC in the one-tile form)
-    // (... and 4096^2 x 512 359 against 332, 4096^2 x 256 level: the complex kernels never walk)
+    // Persistent workgroups that walk a list of tiles, or a workgroup per tile:
     // (real FP16TCEC / bf16x3 / bf16x2: the tile-walking form with global -> LDS loads at every K --
-    // 8192^3 381 - 384 against 365 - 368 TFLOP/s, 16384^2 x 1024 374 against 353, 16384^2 x 256 297 against 262)
+    // 8192^3 381 - 384 against 365 - 368 TFLOP/s, 16384^2 x 1024 374 against 353, 16384^2 x 256 297 against 262;
+    // complex FP16TCEC / bf16x2: up to 32 K-steps -- 8192^2 x 384 390 against 367, 4096^2 x 512 381 against
+    // 370, level from there on; FP16TC, real and complex, has its two one-tile workgroups per CU)
     bool walk = walk_rule == kWalkNever ? false
-                : (walk_rule == kWalkAlways ? true : pargs.k / 32 < 16);
+                : (walk_rule == kWalkAlways ? true
+                   : (walk_rule == kWalkMid ? pargs.k / 32 <= 32 : pargs.k / 32 < 16));
     if (tuning().packed_walk >= 0) walk = tuning().packed_walk == 1;
     const dim3 grid = walk ? dim3((unsigned)std::min<uint64_t>(total, h->num_cus), 1, 1)
                            : dim3((unsigned)total, 1, 1);
@@ -541,12 +539,12 @@ PreSplit run_pre_split(cuMpSGEMM_handle *h, const GemmArgs &args, bool a_kc, boo
                [&](const GemmArgs &g, dim3 grid, bool walk) {
                  if (fp16) launch_packed_fp16tc_c(g, grid, h->stream, walk);
                  else launch_packed_bf16x2_c(g, grid, h->stream, walk);
-               }, kWalkNever);
+               }, fp16 ? kWalkNever : kWalkMid);
     } else {
       ok = run(PackKind::FP16_COMPLEX, pa, pb, ch.bm, ch.bn, accept, h->fused_scaling,
                [&](const GemmArgs &g, dim3 grid, bool walk) {
                  launch_packed_fp16tcec_c(g, grid, h->stream, walk, h->fused_scaling);
-               }, kWalkNever);
+               }, kWalkMid);
     }
   } else if (ch.bf16) {
     ok = run(PackKind::BF16X3_REAL, pa, pb, ch.bm, ch.bn, accept, false,

@@ -739,8 +739,8 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
   // (persistent kernels: the first tile of this workgroup's list; see below)
   uint32_t tile_m, tile_n, tile_b = blockIdx.y;
   if constexpr (Cfg::PERSIST) {
-    // (the walk over pre-split real operands takes its column-group height from the host)
-    const uint32_t group = (Cfg::PACKED && !CPLX && args.raster_group) ? args.raster_group : 8u;
+    // (the walk over pre-split operands takes its column-group height from the host)
+    const uint32_t group = (Cfg::PACKED && args.raster_group) ? args.raster_group : 8u;
     map_tile_batched(blockIdx.x, args.tiles_m, args.tiles_n, args.batch, tile_m, tile_n, tile_b, group);
   } else {
     map_tile(blockIdx.x, args.tiles_m, args.tiles_n, tile_m, tile_n, args.raster_group ? args.raster_group : 8u);
@@ -1010,7 +1010,7 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
             for (int v = 0; v < 16; v++) acc[q][s][j][i][v] = 0.0f;
   };
 
-  if constexpr (Cfg::PERSIST && Cfg::PACKED && !CPLX) {
+  if constexpr (Cfg::PERSIST && Cfg::PACKED) {
     // ---- persistent walk over pre-split operands with global -> LDS loads -----
     // One workgroup walks its list of tiles; the planes of step t + 2 are asked
     // for before the MFMAs of step t, across tile boundaries.  The first step of
