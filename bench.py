@@ -32,7 +32,7 @@ HBM_PEAK_GBS = 8000.0
 # plain copy of known size (profiles/gemm_fp16tcec_8192_nn.md).  This is L2-miss
 # traffic on the fabric (Infinity Cache or HBM); the algorithmic minimum is
 # 3 * 8192^2 * 4 B = 0.805e9.  The call's two pre-split passes add 1.07e9.
-GEMM_TRAFFIC_BYTES = 5.64e9
+GEMM_TRAFFIC_BYTES = 5.72e9
 
 
 def log(*a):
@@ -267,7 +267,7 @@ def main():
                               "(profiles/gemm_fp16tcec_8192_nn.md), not measured in this run",
             # one call = two pre-split passes (about 0.2 ms) + the GEMM kernel: all inside
             "kernel_ms": round(ev_ms, 4),
-            "kernels_per_step": "pack_split_pair_kernel + gemm_tcec_kernel (packed)" if module_id == 200 else
+            "kernels_per_step": "pack_split_pair_kernel + gemm_tcec_kernel (persistent, packed)" if module_id == 200 else
                                 "gemm_tcec_kernel",
             # the split-and-correct algorithm issues 3 MFMA products per logical product
             "mfma_products_per_flop": 3,
@@ -518,7 +518,9 @@ def full_suite(torch, cg, inputs, h, dev, stream, timed, log, a, b, c, with_cpu)
                 "dtype": {"FP16TCEC": "f16 hi/lo", "bf16x3": "bf16 three-term split (stands in for TF32TCEC)",
                           "FP16TC": "f16, no correction terms (FP16TC)",
                           "bf16x2": "bf16 two-term split (stands in for TF32TC)"}[mode_name],
-                "roofline": mfma_roofline(2.0 * n ** 3, ev, prods, "pack_split_pair_kernel + gemm_tcec_kernel (packed)")}
+                "roofline": mfma_roofline(2.0 * n ** 3, ev, prods, "pack_split_pair_kernel + gemm_tcec_kernel " +
+                                          ("(packed, one tile per workgroup)" if mode_name == "FP16TC"
+                                           else "(persistent, packed)"))}
         del ref
     del A, B, A32, B32
     torch.cuda.empty_cache()
@@ -600,7 +602,7 @@ def full_suite(torch, cg, inputs, h, dev, stream, timed, log, a, b, c, with_cpu)
         "rel_error_vendor_fp32": rel_err(torch.matmul(A32, B32).double(), ref), "dtype": "f16 hi/lo",
         "c_write_floor_ms": round(4.0 * mm * mm / (HBM_PEAK_GBS * 1e9) * 1e3, 4),
         "roofline": mfma_roofline(2.0 * mm * mm * kk, ev, 3,
-                                  "pack_split_pair_kernel + gemm_tcec_kernel (packed)" if mid5 == 200
+                                  "pack_split_pair_kernel + gemm_tcec_kernel (persistent, packed)" if mid5 == 200
                                   else "gemm_tcec_kernel (in-loop split, persistent)")}
     del a5, b5, c5, ref
     torch.cuda.empty_cache()
