@@ -1147,10 +1147,7 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
     block_sync_lds();
     frag_load(f0, 0, 0);
     int b0 = 0, b1 = 1, b2 = 2;
-    int ck = 0;
-    uint32_t ct = 0;
-    const uint32_t steps = my_tiles * (uint32_t)nk;
-    for (uint32_t s = 0; s < steps; s++) {
+    auto kstep = [&]() {
       frag_load(f1, b0, 1);
       frag_mma(f0);
       frag_mma(f1);
@@ -1169,17 +1166,35 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
       b0 = b1;
       b1 = b2;
       b2 = tmp;
-      if (++ck == nk) { // tile complete: write it out, move on
-        if (cm0 == clo_m && cn0 == clo_n && cm0 + BM <= args.m && cn0 + BN <= args.n) {
-          epilogue(c_cur, cm0, cn0, clo_m, clo_n, std::true_type{});
-        } else {
-          epilogue(c_cur, cm0, cn0, clo_m, clo_n, std::false_type{});
+    };
+    auto tile_done = [&](uint32_t next) { // write the finished tile out, move on to tile `next`
+      if (cm0 == clo_m && cn0 == clo_n && cm0 + BM <= args.m && cn0 + BN <= args.n) {
+        epilogue(c_cur, cm0, cn0, clo_m, clo_n, std::true_type{});
+      } else {
+        epilogue(c_cur, cm0, cn0, clo_m, clo_n, std::false_type{});
+      }
+      zero_acc();
+      origin(next, a_unused, b_unused, c_cur, cm0, cn0, clo_m, clo_n);
+      origin(next + 1, a_next, b_next, c_unused, u0, u1, u2, u3);
+    };
+    if constexpr (CPLX) {
+      // tiles outside, K-steps inside: measured + 3 - 5 % for the complex kernels
+      // (batch 64 x 512^3 CGEMM 321 -> 335 TFLOP/s) ...
+      for (uint32_t ct = 0; ct < my_tiles; ct++) {
+        for (int kk = 0; kk < nk; kk++) kstep();
+        tile_done(ct + 1);
+      }
+    } else {
+      // ... and - 5 - 25 % for the real ones, which keep one flat loop over all steps
+      int ck = 0;
+      uint32_t ct = 0;
+      const uint32_t steps = my_tiles * (uint32_t)nk;
+      for (uint32_t s = 0; s < steps; s++) {
+        kstep();
+        if (++ck == nk) {
+          ck = 0;
+          tile_done(++ct);
         }
-        zero_acc();
-        ck = 0;
-        ct++;
-        origin(ct, a_unused, b_unused, c_cur, cm0, cn0, clo_m, clo_n);
-        origin(ct + 1, a_next, b_next, c_unused, u0, u1, u2, u3);
       }
     }
     return;
