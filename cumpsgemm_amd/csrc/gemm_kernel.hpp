@@ -29,6 +29,15 @@
 #ifndef CUMPSGEMM_SCHED_VMEM
 #define CUMPSGEMM_SCHED_VMEM 1
 #endif
+// Edge of the MFMA output block: 32 (v_mfma_f32_32x32x16_*) or 16
+// (v_mfma_f32_16x16x32_*), for the kernels that read pre-split operands and
+// for those that split in the K loop.
+#ifndef CUMPSGEMM_MFMA_EDGE_PACKED
+#define CUMPSGEMM_MFMA_EDGE_PACKED 16
+#endif
+#ifndef CUMPSGEMM_MFMA_EDGE_INLOOP
+#define CUMPSGEMM_MFMA_EDGE_INLOOP 32
+#endif
 
 namespace cumpsgemm_amd {
 
@@ -38,6 +47,7 @@ typedef _Float16 h8_t __attribute__((ext_vector_type(8)));
 typedef __bf16 b8_t __attribute__((ext_vector_type(8)));
 typedef float f8_t __attribute__((ext_vector_type(8)));
 typedef float f16v_t __attribute__((ext_vector_type(16)));
+typedef float f4v_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u4_t __attribute__((ext_vector_type(4)));
 
 template <Prec P> struct prec_traits;
@@ -202,12 +212,22 @@ template <> struct splitter<Prec::BF16X2> {
 };
 
 template <bool IS_BF16>
-__device__ inline f16v_t mfma32(const u4_t a, const u4_t b, const f16v_t c) {
+__device__ inline f16v_t mfma_block(const u4_t a, const u4_t b, const f16v_t c) {
   if constexpr (IS_BF16) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(
         __builtin_bit_cast(b8_t, a), __builtin_bit_cast(b8_t, b), c, 0, 0, 0);
   } else {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(
+        __builtin_bit_cast(h8_t, a), __builtin_bit_cast(h8_t, b), c, 0, 0, 0);
+  }
+}
+template <bool IS_BF16>
+__device__ inline f4v_t mfma_block(const u4_t a, const u4_t b, const f4v_t c) {
+  if constexpr (IS_BF16) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+        __builtin_bit_cast(b8_t, a), __builtin_bit_cast(b8_t, b), c, 0, 0, 0);
+  } else {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(
         __builtin_bit_cast(h8_t, a), __builtin_bit_cast(h8_t, b), c, 0, 0, 0);
   }
 }
@@ -257,7 +277,13 @@ struct GemmCfg {
   static constexpr int BM = BM_, BN = BN_, BK = 32, WM = WM_, WN = WN_;
   static constexpr int NWAVES = (BM / WM) * (BN / WN);
   static constexpr int NT = NWAVES * 64;
-  static constexpr int TM = WM / 32, TN = WN / 32;
+  // MFMA blocks per wave tile, accumulator registers per block, and the two
+  // halves a K-step's MFMAs are issued in: the two 16-wide K-slices (edge 32) or
+  // the two halves of the wave tile's columns (edge 16, one 32-wide K-slice)
+  static constexpr int MT = PACKED_ ? CUMPSGEMM_MFMA_EDGE_PACKED : CUMPSGEMM_MFMA_EDGE_INLOOP;
+  static_assert(MT == 32 || MT == 16, "MFMA block edge");
+  static constexpr int TM = WM / MT, TN = WN / MT;
+  static constexpr int NV = MT * MT / 64;
   static constexpr int NP = prec_traits<P>::NP;
   static constexpr int NCOMP = CPLX ? 2 : 1;
   // LDS row: 32 K-values * 2 bytes = four 16-byte chunks, stored at chunk
@@ -817,7 +843,9 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
   // written out, so neither the subtraction nor a conjugation costs a single
   // vector instruction in the K loop.
   constexpr int NACCSET = CPLX ? 4 : 1;
-  f16v_t acc[NACCSET][PT::NACC][TN][TM];
+  constexpr int MT = Cfg::MT, NV = Cfg::NV;
+  typedef float accv_t __attribute__((ext_vector_type(NV)));
+  accv_t acc[NACCSET][PT::NACC][TN][TM];
 #pragma unroll
   for (int q = 0; q < NACCSET; q++)
 #pragma unroll
@@ -827,7 +855,7 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
 #pragma unroll
         for (int i = 0; i < TM; i++)
 #pragma unroll
-          for (int v = 0; v < 16; v++) acc[q][s][j][i][v] = 0.0f;
+          for (int v = 0; v < NV; v++) acc[q][s][j][i][v] = 0.0f;
 
   const int klen = (int)(kend - kbeg);
 
@@ -864,75 +892,98 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
   // (l % 32) of its operand tile and K-values 8*(l/32).. of the 16-wide slice
   // kk, i.e. 16-byte chunk 2*kk + l/32.  The swizzle only looks at the low four
   // row bits, which are the lane's own, so the two slices differ by one XOR.
-  const int frag_row = lane & 31;
-  const int frag_g = lane >> 5;
-  int a_frag_off[BK / 16], b_frag_off[BK / 16];
+  // (Edge 16: lane l of a 16x16x32 MFMA supplies row (l % 16) and K-values
+  // 8*(l/16).. of the whole 32-wide step, i.e. chunk l/16.)
+  const int frag_row = lane & (MT - 1);
+  const int frag_g = lane / MT;
+  int a_frag_off[2], b_frag_off[2];
 #pragma unroll
-  for (int kk = 0; kk < BK / 16; kk++) {
-    a_frag_off[kk] = lds_offset(wm * Cfg::WM + frag_row, 2 * kk + frag_g);
-    b_frag_off[kk] = lds_offset(wn * Cfg::WN + frag_row, 2 * kk + frag_g);
+  for (int kk = 0; kk < 2; kk++) {
+    const int chunk = MT == 32 ? 2 * kk + frag_g : frag_g;
+    a_frag_off[kk] = lds_offset(wm * Cfg::WM + frag_row, chunk);
+    b_frag_off[kk] = lds_offset(wn * Cfg::WN + frag_row, chunk);
   }
 
-  // fragments of one 16-wide K-slice: [component][plane][tile]
+  // A K-step's MFMAs are issued from two sets of fragment registers, so that
+  // one set's LDS reads run beside the MFMAs that use the other.
+  //   edge 32: set h = the 16-wide K-slice h of every block of the wave tile;
+  //   edge 16: set h = half h of the wave tile's row blocks and half h of its
+  //            column blocks over the whole 32-wide step; the four quadrants
+  //            are multiplied in the order (0,0) (0,1) (1,1) (1,0), so that
+  //            each one shares an operand half with the one before it.
+  // [component][plane][block]
+  constexpr int FA = MT == 32 ? TM : TM / 2, FB = MT == 32 ? TN : TN / 2;
+  static_assert(MT == 32 || (TM % 2 == 0 && TN % 2 == 0), "quadrants");
   struct Frags {
-    u4_t a[NCOMP][NP][TM];
-    u4_t b[NCOMP][NP][TN];
+    u4_t a[NCOMP][NP][FA];
+    u4_t b[NCOMP][NP][FB];
   };
-  auto frag_load = [&](Frags &f, int stage, int kk) {
+  auto frag_load = [&](Frags &f, int stage, int h) {
     const char *sa = lds + stage * Cfg::STAGE_BYTES;
     const char *sb = sa + Cfg::A_STAGE_BYTES;
+    const int ib = MT == 32 ? 0 : h * FA, jb = MT == 32 ? 0 : h * FB;
 #pragma unroll
     for (int q = 0; q < NCOMP; q++)
 #pragma unroll
       for (int p = 0; p < NP; p++) {
 #pragma unroll
-        for (int i = 0; i < TM; i++)
+        for (int i = 0; i < FA; i++)
           f.a[q][p][i] = *reinterpret_cast<const u4_t *>(sa + (q * NP + p) * Cfg::A_PLANE_BYTES +
-                                                         a_frag_off[kk] + i * 32 * 64);
+                                                         a_frag_off[h] + (ib + i) * MT * 64);
 #pragma unroll
-        for (int j = 0; j < TN; j++)
+        for (int j = 0; j < FB; j++)
           f.b[q][p][j] = *reinterpret_cast<const u4_t *>(sb + (q * NP + p) * Cfg::B_PLANE_BYTES +
-                                                         b_frag_off[kk] + j * 32 * 64);
+                                                         b_frag_off[h] + (jb + j) * MT * 64);
       }
   };
-  auto frag_mma = [&](Frags &f) {
-    if constexpr (!CPLX) {
+  // blocks [ib, ib + FA) x [jb, jb + FB) of the wave tile += fb.b x fa.a
+  // (one product after the other, so that the two correction products of a
+  // block are FA * FB MFMAs apart)
+  auto frag_mma_part = [&](Frags &fa, Frags &fb, const int ib, const int jb) {
 #pragma unroll
-      for (int t = 0; t < PT::NPROD; t++)
+    for (int t = 0; t < PT::NPROD; t++)
 #pragma unroll
-        for (int j = 0; j < TN; j++)
+      for (int j = 0; j < FB; j++)
 #pragma unroll
-          for (int i = 0; i < TM; i++)
-            acc[0][PT::ACC[t]][j][i] = mfma32<PT::IS_BF16>(
-                f.b[0][PT::PB[t]][j], f.a[0][PT::PA[t]][i], acc[0][PT::ACC[t]][j][i]);
-    } else {
-#pragma unroll
-      for (int t = 0; t < PT::NPROD; t++)
-#pragma unroll
-        for (int j = 0; j < TN; j++)
-#pragma unroll
-          for (int i = 0; i < TM; i++) {
-            const int s = PT::ACC[t], pa = PT::PA[t], pb = PT::PB[t];
-            acc[0][s][j][i] = mfma32<PT::IS_BF16>(f.b[0][pb][j], f.a[0][pa][i], acc[0][s][j][i]);
-            acc[1][s][j][i] = mfma32<PT::IS_BF16>(f.b[1][pb][j], f.a[1][pa][i], acc[1][s][j][i]);
-            acc[2][s][j][i] = mfma32<PT::IS_BF16>(f.b[1][pb][j], f.a[0][pa][i], acc[2][s][j][i]);
-            acc[3][s][j][i] = mfma32<PT::IS_BF16>(f.b[0][pb][j], f.a[1][pa][i], acc[3][s][j][i]);
+        for (int i = 0; i < FA; i++) {
+          const int s = PT::ACC[t], pa = PT::PA[t], pb = PT::PB[t], jj = jb + j, ii = ib + i;
+          if constexpr (!CPLX) {
+            acc[0][s][jj][ii] = mfma_block<PT::IS_BF16>(fb.b[0][pb][j], fa.a[0][pa][i], acc[0][s][jj][ii]);
+          } else {
+            acc[0][s][jj][ii] = mfma_block<PT::IS_BF16>(fb.b[0][pb][j], fa.a[0][pa][i], acc[0][s][jj][ii]);
+            acc[1][s][jj][ii] = mfma_block<PT::IS_BF16>(fb.b[1][pb][j], fa.a[1][pa][i], acc[1][s][jj][ii]);
+            acc[2][s][jj][ii] = mfma_block<PT::IS_BF16>(fb.b[1][pb][j], fa.a[0][pa][i], acc[2][s][jj][ii]);
+            acc[3][s][jj][ii] = mfma_block<PT::IS_BF16>(fb.b[0][pb][j], fa.a[1][pa][i], acc[3][s][jj][ii]);
           }
+        }
+  };
+  // all MFMAs of a step: f0 holds set 0, f1 set 1
+  auto frag_mma = [&](Frags &f0, Frags &f1) {
+    if constexpr (MT == 32) {
+      frag_mma_part(f0, f0, 0, 0);
+      frag_mma_part(f1, f1, 0, 0);
+    } else {
+      frag_mma_part(f0, f0, 0, 0);
+      frag_mma_part(f0, f1, 0, FB);
+      frag_mma_part(f1, f1, FA, FB);
+      frag_mma_part(f1, f0, FA, 0);
     }
   };
-  static_assert(BK / 16 == 2, "two K-slices per step");
+  static_assert(BK == 32, "two 16-wide K-slices, or one 32-wide, per step");
+  // MFMAs per K-step
+  constexpr int STEP_MFMAS = (MT == 32 ? 2 : 1) * PT::NPROD * TM * TN * (CPLX ? 4 : 1);
   auto mma_tile = [&](int stage) {
     Frags f0, f1;
     frag_load(f0, stage, 0);
     frag_load(f1, stage, 1);
-    frag_mma(f0);
-    frag_mma(f1);
+    frag_mma(f0, f1);
   };
 
   // ---- epilogue -----------------------------------------------------------
   // 32x32 accumulator layout: register v of lane l holds
   //   MFMA row (-> n) = 8*(v/4) + 4*(l/32) + v%4,  MFMA column (-> m) = l%32
   // so the 32 lanes of a half-wave write 128 contiguous bytes of a C column.
+  // 16x16: MFMA row (-> n) = 4*(l/16) + v, MFMA column (-> m) = l%16.
   // FULL: interior tile, no bounds checks.
   const bool beta_zero = (args.beta_re == 0.0f) && (!CPLX || args.beta_im == 0.0f);
   const float sgn_a = args.conj_a ? -1.0f : 1.0f, sgn_b = args.conj_b ? -1.0f : 1.0f;
@@ -942,56 +993,86 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
   auto epilogue = [&](float *cb, const uint32_t em0, const uint32_t en0, const uint32_t lo_m,
                       const uint32_t lo_n, auto full_tag) {
     constexpr bool FULL = decltype(full_tag)::value;
+    // one real result
+    auto put = [&](const float x, const uint32_t mm, const uint32_t nn) {
+      if (FULL || (mm < args.m && nn < args.n && mm >= lo_m && nn >= lo_n)) {
+        float *cp = cb + ((uint64_t)nn * args.ldc + mm);
+        if (args.atomic_out) {
+          atomicAdd(cp, x * alpha_re);
+        } else if (beta_zero) {
+          // the result is not read again by this kernel: streaming store
+          __builtin_nontemporal_store(x * alpha_re, cp);
+        } else {
+          *cp = x * alpha_re + args.beta_re * (*cp);
+        }
+      }
+    };
+    auto real_value = [&](const int j, const int i, const int v) {
+      float x = acc[0][0][j][i][v];
+      if constexpr (PT::NACC == 2) x += acc[0][1][j][i][v] * PT::CORR_SCALE;
+      return x;
+    };
+    if constexpr (!CPLX && MT == 16) {
+      // Two neighbouring row blocks trade their odd / even 16-lane rows, after
+      // which register v of lane l holds column 4*(2*(l/32) + w) + v, row l%32
+      // of the block pair (w = 0, 1: the first / second register of the pair):
+      // 32 lanes write 128 contiguous bytes, as with the 32x32 blocks.
+#pragma unroll
+      for (int j = 0; j < TN; j++)
+#pragma unroll
+        for (int i = 0; i < TM; i += 2) {
+          const uint32_t mm = em0 + wm * Cfg::WM + i * 16 + (lane & 31);
+#pragma unroll
+          for (int v = 0; v < 4; v++) {
+            const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(real_value(j, i, v)),
+                                                            __float_as_uint(real_value(j, i + 1, v)), false, false);
+#pragma unroll
+            for (int w = 0; w < 2; w++)
+              put(__uint_as_float(r[w]), mm, en0 + wn * Cfg::WN + j * 16 + 4 * (2 * (lane >> 5) + w) + v);
+          }
+        }
+      return;
+    }
 #pragma unroll
     for (int j = 0; j < TN; j++)
 #pragma unroll
       for (int i = 0; i < TM; i++) {
-        const uint32_t mm = em0 + wm * Cfg::WM + i * 32 + (lane & 31);
+        const uint32_t mm = em0 + wm * Cfg::WM + i * MT + (lane & (MT - 1));
 #pragma unroll
-        for (int v = 0; v < 16; v++) {
-          const uint32_t nn = en0 + wn * Cfg::WN + j * 32 + 8 * (v / 4) + 4 * (lane >> 5) + (v & 3);
-          if (FULL || (mm < args.m && nn < args.n && mm >= lo_m && nn >= lo_n)) {
+        for (int v = 0; v < NV; v++) {
+          const uint32_t nn = en0 + wn * Cfg::WN + j * MT +
+                              (MT == 32 ? 8 * (v / 4) + 4 * (lane >> 5) + (v & 3) : 4 * (lane >> 4) + v);
+          if constexpr (!CPLX) {
+            put(real_value(j, i, v), mm, nn);
+          } else if (FULL || (mm < args.m && nn < args.n && mm >= lo_m && nn >= lo_n)) {
             float *cp = cb + ((uint64_t)nn * args.ldc + mm) * ES;
-            if constexpr (!CPLX) {
-              float x = acc[0][0][j][i][v];
-              if constexpr (PT::NACC == 2) x += acc[0][1][j][i][v] * PT::CORR_SCALE;
-              if (args.atomic_out) {
-                atomicAdd(cp, x * alpha_re);
-              } else if (beta_zero) {
-                // the result is not read again by this kernel: streaming store
-                __builtin_nontemporal_store(x * alpha_re, cp);
-              } else {
-                *cp = x * alpha_re + args.beta_re * (*cp);
-              }
-            } else {
-              // re = ar*br - sa*sb*ai*bi, im = sb*ar*bi + sa*ai*br with
-              // sa (sb) = -1 when op(A) (op(B)) conjugates
-              float p[4];
+            // re = ar*br - sa*sb*ai*bi, im = sb*ar*bi + sa*ai*br with
+            // sa (sb) = -1 when op(A) (op(B)) conjugates
+            float p[4];
 #pragma unroll
-              for (int q = 0; q < 4; q++) {
-                p[q] = acc[q][0][j][i][v];
-                if constexpr (PT::NACC == 2) p[q] += acc[q][1][j][i][v] * PT::CORR_SCALE;
+            for (int q = 0; q < 4; q++) {
+              p[q] = acc[q][0][j][i][v];
+              if constexpr (PT::NACC == 2) p[q] += acc[q][1][j][i][v] * PT::CORR_SCALE;
+            }
+            const float x = p[0] - sgn_ab * p[1];
+            const float y = sgn_b * p[2] + sgn_a * p[3];
+            float rx = x * alpha_re - y * alpha_im;
+            float ry = y * alpha_re + x * alpha_im;
+            if (args.atomic_out) {
+              atomicAdd(cp, rx);
+              atomicAdd(cp + 1, ry);
+            } else {
+              if (!beta_zero) {
+                const float2 old = *reinterpret_cast<const float2 *>(cp);
+                rx = x * alpha_re - y * alpha_im +
+                     (args.beta_re * old.x - args.beta_im * old.y);
+                ry = y * alpha_re + x * alpha_im +
+                     (args.beta_im * old.x + args.beta_re * old.y);
               }
-              const float x = p[0] - sgn_ab * p[1];
-              const float y = sgn_b * p[2] + sgn_a * p[3];
-              float rx = x * alpha_re - y * alpha_im;
-              float ry = y * alpha_re + x * alpha_im;
-              if (args.atomic_out) {
-                atomicAdd(cp, rx);
-                atomicAdd(cp + 1, ry);
-              } else {
-                if (!beta_zero) {
-                  const float2 old = *reinterpret_cast<const float2 *>(cp);
-                  rx = x * alpha_re - y * alpha_im +
-                       (args.beta_re * old.x - args.beta_im * old.y);
-                  ry = y * alpha_re + x * alpha_im +
-                       (args.beta_im * old.x + args.beta_re * old.y);
-                }
-                // the result is not read again by this kernel: streaming store
-                typedef float f2v_t __attribute__((ext_vector_type(2)));
-                f2v_t out2 = {rx, ry};
-                __builtin_nontemporal_store(out2, reinterpret_cast<f2v_t *>(cp));
-              }
+              // the result is not read again by this kernel: streaming store
+              typedef float f2v_t __attribute__((ext_vector_type(2)));
+              f2v_t out2 = {rx, ry};
+              __builtin_nontemporal_store(out2, reinterpret_cast<f2v_t *>(cp));
             }
           }
         }
@@ -1007,7 +1088,7 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
 #pragma unroll
           for (int i = 0; i < TM; i++)
 #pragma unroll
-            for (int v = 0; v < 16; v++) acc[q][s][j][i][v] = 0.0f;
+            for (int v = 0; v < NV; v++) acc[q][s][j][i][v] = 0.0f;
   };
 
   if constexpr (Cfg::PERSIST && Cfg::PACKED) {
@@ -1056,8 +1137,7 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
       constexpr int WAIT = decltype(wait_tag)::value;
       frag_load(f1, b0, 1);
       dma_next(b2);
-      frag_mma(f0);
-      frag_mma(f1);
+      frag_mma(f0, f1);
       __builtin_amdgcn_s_waitcnt(WAIT | KEEP);
       asm volatile("s_barrier" ::: "memory");
       const int tmp = b0;
@@ -1149,13 +1229,12 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
     int b0 = 0, b1 = 1, b2 = 2;
     auto kstep = [&]() {
       frag_load(f1, b0, 1);
-      frag_mma(f0);
-      frag_mma(f1);
+      frag_mma(f0, f1);
       lstore(b2);
       gnext();
       frag_load(f0, b1, 0);
 #pragma unroll
-      for (int g = 0; g < 2 * PT::NPROD * TM * TN * (CPLX ? 4 : 1); g++) {
+      for (int g = 0; g < STEP_MFMAS; g++) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); // MFMA
         __builtin_amdgcn_sched_group_barrier(0x002, CUMPSGEMM_SCHED_VALU, 0); // VALU
         __builtin_amdgcn_sched_group_barrier(0x080, CUMPSGEMM_SCHED_DS, 0); // DS
@@ -1221,8 +1300,7 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
         const int cur = t & 1;
         frag_load(f0, cur, 0);
         frag_load(f1, cur, 1);
-        frag_mma(f0);
-        frag_mma(f1);
+        frag_mma(f0, f1);
         if (t + 1 < nk) lstore(cur ^ 1);
         gload(clamp(t + 2), fast_tag);
         block_sync_lds();
@@ -1250,8 +1328,7 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
       int b0 = 0, b1 = 1, b2 = 2; // buffers of tiles t, t+1, t+2
       for (int t = 0; t < nk; t++) {
         frag_load(f1, b0, 1);
-        frag_mma(f0);
-        frag_mma(f1);
+        frag_mma(f0, f1);
         lstore(b2);
         gload(clamp(t + 3), fast_tag);
         frag_load(f0, b1, 0);
@@ -1259,7 +1336,7 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
           // 24 (real) MFMAs per step: after each one up to 4 vector ALU
           // instructions, one LDS access and one global load
 #pragma unroll
-          for (int g = 0; g < 2 * PT::NPROD * TM * TN * (CPLX ? 4 : 1); g++) {
+          for (int g = 0; g < STEP_MFMAS; g++) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); // MFMA
             __builtin_amdgcn_sched_group_barrier(0x002, CUMPSGEMM_SCHED_VALU, 0); // VALU
             __builtin_amdgcn_sched_group_barrier(0x080, CUMPSGEMM_SCHED_DS, 0); // DS
@@ -1315,8 +1392,7 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
     for (int t = 0; t < nk; t++) {
       frag_load(f1, b0, 1);
       dma(t + 2, b2);
-      frag_mma(f0);
-      frag_mma(f1);
+      frag_mma(f0, f1);
       wait_previous_step();
       // (a plain barrier: a workgroup-scope fence on LDS would make the compiler
       // wait for the loads just issued as well; the "memory" clobber keeps it

@@ -36,3 +36,18 @@ def rel_diff(x, y, m, n, ld):
     xv = x.reshape(-1, ld)[:n, :m].astype(np.complex128)
     yv = y.reshape(-1, ld)[:n, :m].astype(np.complex128)
     return float(np.linalg.norm(xv - yv) / max(np.linalg.norm(yv), 1e-300))
+
+
+def assert_same_up_to_summation_order(x, y, k):
+    """x and y hold the same products added in a different order (kernels built on MFMAs of
+    different K-depth): equal within a few FP32 roundings per partial sum, as a whole
+    (Frobenius) and element by element -- a misplaced element would differ at order one."""
+    if hasattr(x, "detach"):
+        x, y = x.detach().cpu().numpy(), y.detach().cpu().numpy()
+    xv = np.ascontiguousarray(x).view(np.float32).astype(np.float64).ravel()
+    yv = np.ascontiguousarray(y).view(np.float32).astype(np.float64).ravel()
+    assert xv.shape == yv.shape and np.isfinite(xv).all() and np.isfinite(yv).all()
+    d = np.abs(xv - yv)
+    bar = 2.0 ** -24 * np.sqrt(k)
+    assert np.linalg.norm(d) <= 2.0 * bar * np.linalg.norm(yv), (np.linalg.norm(d) / np.linalg.norm(yv), bar)
+    assert d.max() <= 16.0 * bar * np.abs(yv).max(), (d.max() / np.abs(yv).max(), bar)

@@ -10,7 +10,7 @@ import numpy as np
 import pytest
 
 from cumpsgemm_amd import inputs
-from gpu_util import N, T, oracle_gemm, rel_diff
+from gpu_util import N, T, assert_same_up_to_summation_order, oracle_gemm, rel_diff
 
 pytestmark = pytest.mark.gpu
 FP16TCEC, TF32TCEC, FP32 = 1, 2, 12
@@ -50,7 +50,8 @@ def test_same_sign_operands_in_loop_kernels(O, handle, dev, monkeypatch, mode, f
 @pytest.mark.parametrize("mode", [FP16TCEC, TF32TCEC])
 def test_same_sign_operands_pre_split_kernels(cg, torch_gpu, monkeypatch, mode):
     """The pre-split kernels at K = 8192 (one tile per workgroup, 256 K-steps in one accumulator):
-    bit-identical to the in-loop kernels, and within the bars against an FP64 product."""
+    the in-loop kernels' result up to the order of summation (their MFMAs add 16 K-values, the
+    pre-split kernels' 32), and within the bars against an FP64 product."""
     torch = torch_gpu
     dev = torch.device("cuda:0")
     m, n, k = 4096, 2048, 8192
@@ -70,7 +71,7 @@ def test_same_sign_operands_pre_split_kernels(cg, torch_gpu, monkeypatch, mode):
             torch.cuda.synchronize()
             assert st == 0 and (mid == 200) == (packed == "1"), mid
             outs.append(c)
-        assert torch.equal(outs[0], outs[1])
+        assert_same_up_to_summation_order(outs[0], outs[1], k)
         ref = b.double() @ a.double().t()
         r = (torch.linalg.norm(outs[0].double() - ref) / torch.linalg.norm(ref)).item()
         r32 = (torch.linalg.norm((b @ a.t()).double() - ref) / torch.linalg.norm(ref)).item()

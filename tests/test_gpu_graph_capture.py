@@ -7,6 +7,7 @@ import numpy as np
 import pytest
 
 from cumpsgemm_amd import inputs
+from gpu_util import assert_same_up_to_summation_order
 
 pytestmark = pytest.mark.gpu
 N_OP = 111
@@ -66,7 +67,8 @@ def test_captured_calls_replay_like_eager_calls(cg, torch_gpu, mode, cplx):
 
 def test_capture_never_grows_the_workspace(cg, torch_gpu, monkeypatch):
     """A call that would take the pre-split path while its workspace is still missing must not
-    allocate or synchronise under capture: it runs the in-loop kernels instead (same bits)."""
+    allocate or synchronise under capture: it runs the in-loop kernels instead (the same result up
+    to the order of summation)."""
     torch = torch_gpu
     m, n, k = 4096, 3840, 768
     dev = torch.device("cuda:0")
@@ -102,7 +104,7 @@ def test_capture_never_grows_the_workspace(cg, torch_gpu, monkeypatch):
         st, mid = call(c_eager)                 # eager: allocates and takes the pre-split path
         torch.cuda.synchronize()
         assert st == 0 and mid == 200 and h.workspace_size() >= (m + n) * k * 4
-        assert torch.equal(c_graph, c_eager)
+        assert_same_up_to_summation_order(c_graph, c_eager, k)
     finally:
         torch.cuda.synchronize()
         h.close()

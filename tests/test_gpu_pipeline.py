@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 
 from cumpsgemm_amd import inputs
-from gpu_util import N, T, oracle_gemm
+from gpu_util import N, T, assert_same_up_to_summation_order, oracle_gemm
 
 pytestmark = pytest.mark.gpu
 FP16TCEC, TF32TCEC, AUTO, SCALING, FP32 = 1, 2, 9, 11, 12
@@ -177,10 +177,12 @@ def test_fused_scaling_matches_in_place_scaling(O, handle, dev, monkeypatch, mod
 # Large real problems in FP16TCEC_SCALING take the pre-split path: A and B are
 # scaled and split once into fp16 planes (workspace of the handle) and the GEMM
 # kernel only folds the inverse scaling of C into alpha.  Same scaling, same
-# split, same order of accumulation as the two other forms -> same bits.
+# split, same products as the two other forms (which agree bit for bit); the
+# pre-split kernels' MFMAs add 32 K-values where the in-loop kernels' add 16, so
+# they agree with those up to the order of summation.
 def test_complex_scaled_pre_split_path_matches_in_loop(cg, torch_gpu, dev, monkeypatch):
     """FP16TCEC_SCALING on a large complex problem: the pre-pass scales, splits and
-    de-interleaves; same bits as the in-loop fused form."""
+    de-interleaves; the in-loop fused form's result up to the order of summation."""
     m, n, k = 3800, 3700, 288
     C_OP = 113
     a = (inputs.complex_normal(75, m * k, 1.0) * np.float32(2.0 ** -21)).astype(np.complex64)
@@ -198,7 +200,7 @@ def test_complex_scaled_pre_split_path_matches_in_loop(cg, torch_gpu, dev, monke
             assert (h.workspace_size() >= (m + n) * k * 8) == (packed is None)
             assert np.array_equal(a_after.view(np.uint32), a.view(np.uint32))
             outs.append(c)
-        assert np.array_equal(outs[0].view(np.uint32), outs[1].view(np.uint32))
+        assert_same_up_to_summation_order(outs[0], outs[1], k)
         assert float(np.abs(outs[0]).max()) > 0
     finally:
         torch_gpu.cuda.synchronize()
@@ -238,8 +240,8 @@ def test_scaled_pre_split_path_matches_the_other_forms(O, cg, torch_gpu, dev, mo
             assert np.array_equal(a_after.view(np.uint32), a.view(np.uint32))
             assert np.array_equal(b_after.view(np.uint32), b.view(np.uint32))
             outs[form] = c
-        assert np.array_equal(outs["pre_split"].view(np.uint32), outs["in_loop"].view(np.uint32))
-        assert np.array_equal(outs["pre_split"].view(np.uint32), outs["in_place"].view(np.uint32))
+        assert np.array_equal(outs["in_loop"].view(np.uint32), outs["in_place"].view(np.uint32))
+        assert_same_up_to_summation_order(outs["pre_split"], outs["in_loop"], k)
     finally:
         torch_gpu.cuda.synchronize()
         h.close()
@@ -254,7 +256,8 @@ def test_auto_pre_split_path_steps_aside_for_bf16x3(O, cg, torch_gpu, dev, monke
     """Same shape class, but AUTO decides for TF32TCEC (no underflow tolerated):
     the gated pre-pass and the gated FP16TCEC kernel do nothing, the bf16x3
     kernel (k = 256: the in-loop one; k = 512: its own gated pre-split form)
-    produces C -- the same bits as with the pre-split path forbidden."""
+    produces C -- the same result, up to the order of summation for the pre-split
+    form, as with the pre-split path forbidden."""
     m, n = 4096, 4096
     a = (inputs.uniform(81, m * k) * np.float32(2.0 ** -22)).astype(np.float32)
     b = (inputs.uniform(82, k * n) * np.float32(2.0 ** 5)).astype(np.float32)
@@ -270,7 +273,10 @@ def test_auto_pre_split_path_steps_aside_for_bf16x3(O, cg, torch_gpu, dev, monke
             c, _, _, ids = _pipeline(h, dev, AUTO, N, N, m, n, k, a, b)
             assert h.get_dynamic_launch_flag(ids[2]) & 0x1f == TF32TCEC
             outs.append(c)
-        assert np.array_equal(outs[0].view(np.uint32), outs[1].view(np.uint32))
+        if k == 256:
+            assert np.array_equal(outs[0].view(np.uint32), outs[1].view(np.uint32))
+        else:
+            assert_same_up_to_summation_order(outs[0], outs[1], k)
     finally:
         torch_gpu.cuda.synchronize()
         h.close()
