@@ -358,16 +358,20 @@ PreSplitChoice choose_pre_split(const cuMpSGEMM_handle *h, bool a_kc, bool b_kc,
   // (complex: four times the MFMA work per element split, so the pre-pass weighs less)
   // (5120^3, 800 tiles = 3.1 rounds: 329 TFLOP/s this way, 356 in-loop, whose planner cuts C in two)
   const bool pays_nt = pays_nt_shape && rounds_ok;
-  // Short K: per tile the in-loop kernels lose more to the split than the pre-pass
-  // costs once C is large (in-loop -> pre-split, TFLOP/s: 16384^2 x 256 271 -> 297, 16384^2 x 512 313 -> 347,
-  // 8192^2 x 512 317 -> 328, 8192^2 x 768 332 -> 352, 6144^2 x 512 279 -> 291; 8192^2 x 256 and 6144^2 x 256
-  // stay in-loop: 271 / 243 against 267 / 228, and so does 4096^2 below K = 2048).
+  // Shorter K: per tile the in-loop kernels lose more to the split than the pre-pass
+  // costs once C is large (in-loop -> pre-split, TFLOP/s, NN / TN: 8192^2 x 256 261 / 270 -> 277 / 278,
+  // 8192^2 x 384 287 / 297 -> 314 / 313, 6144^2 x 384 254 / 266 -> 280 / 282, 6144^2 x 512 274 / 285 -> 306 / 307,
+  // 4096^2 x 1024 326 / 333 -> 343 / 343, 4096^2 x 2048 350 / 357 -> 384 / 384; 6144^2 x 256 and 4096^2 x 512
+  // are level and stay in-loop, 4096^2 x 256 would lose 8 - 11 %).
   const bool pays_short = !CPLX && rounds_ok &&
-                          ((k >= 256 && mn_ratio >= 8000.0) || (k >= 512 && mn_ratio >= 3000.0));
-  // (complex, in-loop -> pre-split: 4096^3 340 -> 415 TFLOP/s, 2048^3 322 -> 375, 4096^2 x 512 304 -> 359,
-  // 8192^2 x 384 304 -> 357, 4096^2 x 256 level)
-  const bool pays = CPLX ? (k >= 384 && mn_ratio >= 1000.0 && rounds_ok)
-                         : (pays_nt || pays_short || (k >= 2048 && mn_ratio >= 2000.0 && rounds_ok));
+                          ((k >= 256 && mn_ratio >= 4000.0) || (k >= 384 && mn_ratio >= 3000.0) ||
+                           (k >= 1024 && mn_ratio >= 2000.0));
+  // (complex, in-loop -> pre-split, NN / TN: 4096^3 367 / 378 -> 432 / 435 TFLOP/s, 2048^3 355 / 364 -> 401 / 400,
+  // 2048^2 x 1024 349 / 347 -> 372 / 374, 3072^2 x 384 309 / 314 -> 329 / 325, 4096^2 x 256 313 / 320 -> 342 / 349,
+  // 8192^2 x 256 323 / 321 -> 368 / 373; 2048^2 x 512 level, 2048^2 x 384 would lose 5 %, 3072^2 x 256 level)
+  const bool pays_cplx = rounds_ok && ((k >= 256 && mn_ratio >= 2000.0) || (k >= 384 && mn_ratio >= 1500.0) ||
+                                       (k >= 1024 && mn_ratio >= 1000.0));
+  const bool pays = CPLX ? pays_cplx : (pays_nt || pays_short);
   // With fused scaling the in-loop split costs one more instruction per pair
   // and those kernels run 8 - 25 % below the plain ones, so the pre-pass (which
   // scales as it splits) pays for every layout.
@@ -378,9 +382,12 @@ PreSplitChoice choose_pre_split(const cuMpSGEMM_handle *h, bool a_kc, bool b_kc,
   if (!CPLX && mode == CUMPSGEMM_AUTO && pays_scaled && depth == 0) {
     ch.auto_ok = make_plan(h, Prec::BF16X3, CPLX, a_kc, b_kc, m, n, k, batch, force_cls, force_split).ksplit == 1;
   }
-  // (measured against the in-loop 256x128 class: - 3 % at 4096^3 and 4096^2 x 8192, - 6 % at 5120^3,
-  // + 8 % at 6144^3 and 6144^2 x 1024, + 4 - 7 % from 8192^2 x 512 on)
-  const bool pays_bf16 = k >= 512 && mn_ratio >= 3000.0;
+  // (measured against the in-loop 256x128 class, NN / TN, TFLOP/s: 8192^2 x 256 167 / 172 -> 189 / 187,
+  // 6144^2 x 256 152 / 157 -> 173 / 178, 4096^2 x 512 182 / 189 -> 190 / 191, 4096^3 208 / 213 -> 231 / 228,
+  // 3072^2 x 1024 157 / 162 -> 171 / 171, 2048^2 x 2048 188 / 178 -> 200 / 198; 4096^2 x 384, 3072^2 x 512 and
+  // 2048^2 x 1024 are level, shorter K loses)
+  const bool pays_bf16 = (k >= 256 && mn_ratio >= 3000.0) || (k >= 512 && mn_ratio >= 2000.0) ||
+                         (k >= 1024 && mn_ratio >= 1500.0) || (k >= 2048 && mn_ratio >= 1000.0);
   // The uncorrected modes issue a third (FP16TC) or as many (bf16x2) MFMAs per
   // element as FP16TCEC, so the same pre-pass weighs three times as much for
   // the former: it is taken for large square-ish problems only.

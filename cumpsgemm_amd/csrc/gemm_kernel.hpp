@@ -323,6 +323,17 @@ __device__ inline int lds_swizzle(int row) {
 __device__ inline int lds_offset(int row, int chunk) {
   return row * 64 + ((chunk ^ lds_swizzle(row)) << 4);
 }
+// The same for the planes of pre-split operands, which reach LDS as linear
+// copies (no staging writes to keep apart) and are read as 16x16x32 fragments:
+// lane l takes row l % 16, chunk l / 16, and a ds_read_b128 is served in four
+// passes of lanes [8g, 8g + 8) + [32 + 8g, 40 + 8g), i.e. 8 consecutive rows at
+// chunks c and c + 2 -- rows r and r + 4 must differ in the low swizzle bit.
+__device__ inline int lds_swizzle_packed(int row) {
+  return CUMPSGEMM_MFMA_EDGE_PACKED == 16 ? ((row >> 2) & 1) : lds_swizzle(row);
+}
+__device__ inline int lds_offset_packed(int row, int chunk) {
+  return row * 64 + ((chunk ^ lds_swizzle_packed(row)) << 4);
+}
 
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also fences
 // global memory, which makes every wave wait for its outstanding global loads
@@ -900,8 +911,10 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
 #pragma unroll
   for (int kk = 0; kk < 2; kk++) {
     const int chunk = MT == 32 ? 2 * kk + frag_g : frag_g;
-    a_frag_off[kk] = lds_offset(wm * Cfg::WM + frag_row, chunk);
-    b_frag_off[kk] = lds_offset(wn * Cfg::WN + frag_row, chunk);
+    a_frag_off[kk] = Cfg::PACKED ? lds_offset_packed(wm * Cfg::WM + frag_row, chunk)
+                                 : lds_offset(wm * Cfg::WM + frag_row, chunk);
+    b_frag_off[kk] = Cfg::PACKED ? lds_offset_packed(wn * Cfg::WN + frag_row, chunk)
+                                 : lds_offset(wn * Cfg::WN + frag_row, chunk);
   }
 
   // A K-step's MFMAs are issued from two sets of fragment registers, so that
