@@ -325,11 +325,12 @@ __device__ inline int lds_offset(int row, int chunk) {
 }
 // The same for the planes of pre-split operands, which reach LDS as linear
 // copies (no staging writes to keep apart) and are read as 16x16x32 fragments:
-// lane l takes row l % 16, chunk l / 16, and a ds_read_b128 is served in four
-// passes of lanes [8g, 8g + 8) + [32 + 8g, 40 + 8g), i.e. 8 consecutive rows at
-// chunks c and c + 2 -- rows r and r + 4 must differ in the low swizzle bit.
+// lane l takes row l % 16, chunk l / 16.  Measured with SQ_LDS_BANK_CONFLICT
+// over all 256 XOR swizzles that are linear in the low four row bits: this
+// read pattern is conflict-free when the high chunk bit is flipped by row bit
+// 2 (the swizzle above costs it 4 extra cycles per ds_read_b128).
 __device__ inline int lds_swizzle_packed(int row) {
-  return CUMPSGEMM_MFMA_EDGE_PACKED == 16 ? ((row >> 2) & 1) : lds_swizzle(row);
+  return CUMPSGEMM_MFMA_EDGE_PACKED == 16 ? (((row >> 2) & 1) << 1) : lds_swizzle(row);
 }
 __device__ inline int lds_offset_packed(int row, int chunk) {
   return row * 64 + ((chunk ^ lds_swizzle_packed(row)) << 4);
