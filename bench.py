@@ -32,7 +32,7 @@ HBM_PEAK_GBS = 8000.0
 # plain copy of known size (profiles/gemm_fp16tcec_8192_nn.md).  This is L2-miss
 # traffic on the fabric (Infinity Cache or HBM); the algorithmic minimum is
 # 3 * 8192^2 * 4 B = 0.805e9.  The call's two pre-split passes add 1.07e9.
-GEMM_TRAFFIC_BYTES = 5.72e9
+GEMM_TRAFFIC_BYTES = 5.70e9
 
 
 def log(*a):
