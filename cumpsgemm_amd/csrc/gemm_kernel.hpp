@@ -30,8 +30,9 @@
 #define CUMPSGEMM_SCHED_VMEM 1
 #endif
 // Edge of the MFMA output block: 32 (v_mfma_f32_32x32x16_*) or 16
-// (v_mfma_f32_16x16x32_*), for the kernels that read pre-split operands and
-// for those that split in the K loop.
+// (v_mfma_f32_16x16x32_*), for the kernels that read pre-split operands (and
+// the in-loop complex bf16x3 ones) and for the other kernels that split in the
+// K loop.
 #ifndef CUMPSGEMM_MFMA_EDGE_PACKED
 #define CUMPSGEMM_MFMA_EDGE_PACKED 16
 #endif
@@ -280,7 +281,12 @@ struct GemmCfg {
   // MFMA blocks per wave tile, accumulator registers per block, and the two
   // halves a K-step's MFMAs are issued in: the two 16-wide K-slices (edge 32) or
   // the two halves of the wave tile's columns (edge 16, one 32-wide K-slice)
-  static constexpr int MT = PACKED_ ? CUMPSGEMM_MFMA_EDGE_PACKED : CUMPSGEMM_MFMA_EDGE_INLOOP;
+  // (in-loop kernels measured with edge 16, all sizes and batches: complex
+  // bf16x3 + 5 - 7 % throughout; the others between - 8 % and + 9 % with a mean
+  // of zero, so they keep 32)
+  static constexpr int MT = PACKED_ ? CUMPSGEMM_MFMA_EDGE_PACKED
+                            : (P_ == Prec::BF16X3 && CPLX_) ? CUMPSGEMM_MFMA_EDGE_PACKED
+                                                            : CUMPSGEMM_MFMA_EDGE_INLOOP;
   static_assert(MT == 32 || MT == 16, "MFMA block edge");
   static constexpr int TM = WM / MT, TN = WN / MT;
   static constexpr int NV = MT * MT / 64;
@@ -312,28 +318,20 @@ struct GemmCfg {
 };
 
 // Byte offset of (row, 16-byte chunk) inside one LDS plane.  Rows are 64 bytes,
-// i.e. 16 banks; the chunk is XOR-swizzled with row bits chosen such that
-//  - 8 (16) consecutive rows at one logical chunk -- a fragment read, or a
-//    staging write of a row-contiguous tile -- cover all 32 (64) banks,
-//  - 2 (4) consecutive rows x 4 chunks -- a staging write of a K-contiguous
-//    tile -- do too.
+// i.e. 16 banks; the chunk is XOR-swizzled with row bits.  The swizzle was
+// picked by measurement (SQ_LDS_BANK_CONFLICT over all 256 swizzles whose two
+// bits are parities of the low four row bits): it is one of the 16 that take
+// every access pattern of these kernels without a conflict cycle --
+//  - fragment reads, ds_read_b128: lane l at row l % 32, chunk l / 32
+//    (32x32x16 MFMAs) or at row l % 16, chunk l / 16 (16x16x32 MFMAs),
+//  - staging writes, ds_write_b128: 16 consecutive rows x 4 chunks (a
+//    K-contiguous tile) or 64 consecutive rows at one chunk (a row-contiguous
+//    one), and their 8-byte half-unit forms.
 __device__ inline int lds_swizzle(int row) {
-  return (((row >> 1) ^ (row >> 3)) & 1) | (((row >> 2) & 1) << 1);
+  return (((row >> 1) ^ (row >> 3)) & 1) | ((((row >> 2) ^ (row >> 3)) & 1) << 1);
 }
 __device__ inline int lds_offset(int row, int chunk) {
   return row * 64 + ((chunk ^ lds_swizzle(row)) << 4);
-}
-// The same for the planes of pre-split operands, which reach LDS as linear
-// copies (no staging writes to keep apart) and are read as 16x16x32 fragments:
-// lane l takes row l % 16, chunk l / 16.  Measured with SQ_LDS_BANK_CONFLICT
-// over all 256 XOR swizzles that are linear in the low four row bits: this
-// read pattern is conflict-free when the high chunk bit is flipped by row bit
-// 2 (the swizzle above costs it 4 extra cycles per ds_read_b128).
-__device__ inline int lds_swizzle_packed(int row) {
-  return CUMPSGEMM_MFMA_EDGE_PACKED == 16 ? (((row >> 2) & 1) << 1) : lds_swizzle(row);
-}
-__device__ inline int lds_offset_packed(int row, int chunk) {
-  return row * 64 + ((chunk ^ lds_swizzle_packed(row)) << 4);
 }
 
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also fences
@@ -912,10 +910,8 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
 #pragma unroll
   for (int kk = 0; kk < 2; kk++) {
     const int chunk = MT == 32 ? 2 * kk + frag_g : frag_g;
-    a_frag_off[kk] = Cfg::PACKED ? lds_offset_packed(wm * Cfg::WM + frag_row, chunk)
-                                 : lds_offset(wm * Cfg::WM + frag_row, chunk);
-    b_frag_off[kk] = Cfg::PACKED ? lds_offset_packed(wn * Cfg::WN + frag_row, chunk)
-                                 : lds_offset(wn * Cfg::WN + frag_row, chunk);
+    a_frag_off[kk] = lds_offset(wm * Cfg::WM + frag_row, chunk);
+    b_frag_off[kk] = lds_offset(wn * Cfg::WN + frag_row, chunk);
   }
 
   // A K-step's MFMAs are issued from two sets of fragment registers, so that
@@ -984,7 +980,9 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
     }
   };
   static_assert(BK == 32, "two 16-wide K-slices, or one 32-wide, per step");
-  // MFMAs per K-step
+  // MFMAs per K-step, and the vector instructions dripped in after each (half
+  // as many after a 16x16x32 MFMA, which is half as long)
+  constexpr int SCHED_VALU = MT == 32 ? CUMPSGEMM_SCHED_VALU : (CUMPSGEMM_SCHED_VALU + 1) / 2;
   constexpr int STEP_MFMAS = (MT == 32 ? 2 : 1) * PT::NPROD * TM * TN * (CPLX ? 4 : 1);
   auto mma_tile = [&](int stage) {
     Frags f0, f1;
@@ -1250,7 +1248,7 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
 #pragma unroll
       for (int g = 0; g < STEP_MFMAS; g++) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); // MFMA
-        __builtin_amdgcn_sched_group_barrier(0x002, CUMPSGEMM_SCHED_VALU, 0); // VALU
+        __builtin_amdgcn_sched_group_barrier(0x002, SCHED_VALU, 0); // VALU
         __builtin_amdgcn_sched_group_barrier(0x080, CUMPSGEMM_SCHED_DS, 0); // DS
         __builtin_amdgcn_sched_group_barrier(0x020, CUMPSGEMM_SCHED_VMEM, 0); // VMEM read
       }
@@ -1352,7 +1350,7 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
 #pragma unroll
           for (int g = 0; g < STEP_MFMAS; g++) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); // MFMA
-            __builtin_amdgcn_sched_group_barrier(0x002, CUMPSGEMM_SCHED_VALU, 0); // VALU
+            __builtin_amdgcn_sched_group_barrier(0x002, SCHED_VALU, 0); // VALU
             __builtin_amdgcn_sched_group_barrier(0x080, CUMPSGEMM_SCHED_DS, 0); // DS
             __builtin_amdgcn_sched_group_barrier(0x020, CUMPSGEMM_SCHED_VMEM, 0); // VMEM read
           }

@@ -10,7 +10,7 @@
 //   (bf16x3: the three terms in order),
 //   row < rows_pad (a multiple of 256, rows >= `rows` and K-values >= `k` are
 //   zero), and inside a row the 16-byte chunk c (8 K-values) sits at position
-//   c ^ lds_swizzle_packed(row).
+//   c ^ lds_swizzle(row).
 // HBM-bound: reads 4 bytes and writes 2 bytes per plane and element.
 #include "gemm_kernel.hpp"
 #include <algorithm>
@@ -130,7 +130,7 @@ __device__ inline void pack_split_body(const PackJob &job, const int *scale_flag
     }
   };
   // position of the thread's chunk inside the 64-row block image of one plane
-  const uint32_t pos = lrow * 64 + ((chunk ^ (uint32_t)lds_swizzle_packed((int)row)) << 4);
+  const uint32_t pos = lrow * 64 + ((chunk ^ (uint32_t)lds_swizzle((int)row)) << 4);
   auto split_to = [&](const Vals &x, uint32_t kb, int buf) {
 #pragma unroll
     for (int q = 0; q < NC; q++) {
