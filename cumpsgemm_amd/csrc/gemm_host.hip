@@ -301,8 +301,10 @@ template <> struct scalar_parts<hipComplex> {
 // ---------------------------------------------------------------------------
 // Pre-split path (FP16TCEC real and complex; bf16x3, FP16TC and bf16x2 real): split A and B once,
 // up front, into fp16 / bf16 planes held in the handle's workspace, and run the
-// kernel that only copies them into LDS.  Results are bit-identical to the
-// in-loop split (same split, same order of accumulation).  The pre-pass is one
+// kernel that only copies them into LDS.  Same split and same products as the
+// in-loop kernels; the order of summation differs (16x16x32 MFMAs add 32
+// K-values at a time, the in-loop kernels' 32x32x16 MFMAs 16), so results agree
+// to a few FP32 roundings, not bit for bit.  The pre-pass is one
 // read + write of A and B at 5 - 6 TB/s; what it buys is a K loop without split
 // arithmetic, which runs at a higher clock under the power limit.  It pays for
 // large problems (rules below, per mode and layout); the in-loop kernels serve

@@ -1370,8 +1370,8 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
     // registers, no ds_write.  In step t a wave
     //   - asks for its share of tile t + 2 (into the buffer that tile t - 1 was
     //     read from, free since the barrier that ended step t - 1),
-    //   - multiplies tile t (first K-slice from fragments fetched right after
-    //     that barrier, second fetched now),
+    //   - multiplies tile t (first set of fragments fetched right after that
+    //     barrier, second fetched now),
     //   - waits until its share of tile t + 1 -- asked for a whole step ago -- has
     //     landed, then at the barrier for everybody else's.
     // Same arithmetic in the same order as the register-staged pipeline
