@@ -322,6 +322,9 @@ struct PreSplitChoice {
   bool tc_only = false;   // FP16TC / TF32TC (no correction terms): one fp16 plane / two bf16 planes
   bool auto_ok = false;   // AUTO: the gated FP16TCEC candidate goes this way
   bool auto_bf16 = false; // AUTO: and so does the gated bf16x3 candidate
+  // not taken only because the last round of CU slots would be mostly empty:
+  // worth taking for the part of C that fills whole rounds
+  bool cut = false;
   int bm = 0, bn = 0;     // tile of the kernel that reads the planes
   unsigned planes = 0;    // planes per K-step of one operand
 };
@@ -336,7 +339,8 @@ PreSplitChoice choose_pre_split(const cuMpSGEMM_handle *h, bool a_kc, bool b_kc,
   // CUMPSGEMM_PACKED: "0" never, "1" whenever possible; the entry point that
   // allocates nothing always goes this way (its planes have a home already)
   const bool forced = h->ws_override != nullptr;
-  const bool never = tuning().packed == 0 && !forced, always = tuning().packed == 1 || forced;
+  // (depth 2: the whole rounds of a problem that was cut for this path)
+  const bool never = tuning().packed == 0 && !forced, always = tuning().packed == 1 || forced || depth == 2;
   // bf16x3 (explicit TF32TCEC mode): its in-loop three-way split costs 5.4
   // vector instructions per MFMA, so the pre-pass pays for every layout
   ch.bf16 = (mode == CUMPSGEMM_TF32TCEC);
@@ -359,21 +363,6 @@ PreSplitChoice choose_pre_split(const cuMpSGEMM_handle *h, bool a_kc, bool b_kc,
   const bool rounds_ok = last_round == 0 || 2 * last_round >= h->num_cus || ptiles >= 6ull * h->num_cus;
   // (complex: four times the MFMA work per element split, so the pre-pass weighs less)
   // (5120^3, 800 tiles = 3.1 rounds: 329 TFLOP/s this way, 356 in-loop, whose planner cuts C in two)
-  const bool pays_nt = pays_nt_shape && rounds_ok;
-  // Shorter K: per tile the in-loop kernels lose more to the split than the pre-pass
-  // costs once C is large (in-loop -> pre-split, TFLOP/s, NN / TN: 8192^2 x 256 261 / 270 -> 277 / 278,
-  // 8192^2 x 384 287 / 297 -> 314 / 313, 6144^2 x 384 254 / 266 -> 280 / 282, 6144^2 x 512 274 / 285 -> 306 / 307,
-  // 4096^2 x 1024 326 / 333 -> 343 / 343, 4096^2 x 2048 350 / 357 -> 384 / 384; 6144^2 x 256 and 4096^2 x 512
-  // are level and stay in-loop, 4096^2 x 256 would lose 8 - 11 %).
-  const bool pays_short = !CPLX && rounds_ok &&
-                          ((k >= 256 && mn_ratio >= 4000.0) || (k >= 384 && mn_ratio >= 3000.0) ||
-                           (k >= 1024 && mn_ratio >= 2000.0));
-  // (complex, in-loop -> pre-split, NN / TN: 4096^3 367 / 378 -> 432 / 435 TFLOP/s, 2048^3 355 / 364 -> 401 / 400,
-  // 2048^2 x 1024 349 / 347 -> 372 / 374, 3072^2 x 384 309 / 314 -> 329 / 325, 4096^2 x 256 313 / 320 -> 342 / 349,
-  // 8192^2 x 256 323 / 321 -> 368 / 373; 2048^2 x 512 level, 2048^2 x 384 would lose 5 %, 3072^2 x 256 level)
-  const bool pays_cplx = rounds_ok && ((k >= 256 && mn_ratio >= 2000.0) || (k >= 384 && mn_ratio >= 1500.0) ||
-                                       (k >= 1024 && mn_ratio >= 1000.0));
-  const bool pays = CPLX ? pays_cplx : (pays_nt || pays_short);
   // With fused scaling the in-loop split costs one more instruction per pair
   // and those kernels run 8 - 25 % below the plain ones, so the pre-pass (which
   // scales as it splits) pays for every layout.
@@ -390,26 +379,50 @@ PreSplitChoice choose_pre_split(const cuMpSGEMM_handle *h, bool a_kc, bool b_kc,
   // 2048^2 x 1024 are level, shorter K loses)
   const bool pays_bf16 = (k >= 256 && mn_ratio >= 3000.0) || (k >= 512 && mn_ratio >= 2000.0) ||
                          (k >= 1024 && mn_ratio >= 1500.0) || (k >= 2048 && mn_ratio >= 1000.0);
-  // The uncorrected modes issue a third (FP16TC) or as many (bf16x2) MFMAs per
-  // element as FP16TCEC, so the same pre-pass weighs three times as much for
-  // the former: it is taken for large square-ish problems only.
-  // Measured (in-loop -> pre-split, TFLOP/s): FP16TC 8192^3 580 - 624 -> 930 - 940, 4096^3 586 - 706 ->
-  // 852 - 870, 4096^2 x 1024 505 - 566 -> 634 - 654, 8192^2 x 512 482 - 520 -> 579 - 601, 16384^2 x 256
-  // 390 - 407 -> 461 - 480, 4096^2 x 512 level; bf16x2 8192^3 320 - 377 -> 394 - 396, 4096^2 x 1024
-  // 304 - 337 -> 348 - 355, 8192^2 x 512 275 - 308 -> 318 - 327, 4096^2 x 512 level except NT.
-  // Complex (the 128x64 kernels): FP16TC 4096^3 560 - 678 -> 872 - 891, 2048^3 525 - 640 -> 760 - 779,
-  // 8192^2 x 256 477 - 543 -> 624 - 643; bf16x2 4096^3 350 -> 375, 4096^2 x 1024 333 - 339 -> 365,
-  // 4096^2 x 512 303 - 326 -> 336 - 347.
-  const bool pays_tc =
-      rounds_ok &&
-      (CPLX ? (k >= 256 && mn_ratio >= 1000.0)
-            : ((k >= 1024 && mn_ratio >= (mode == CUMPSGEMM_FP16TC ? 1500.0 : 2000.0)) ||
-               (k >= 512 && mn_ratio >= 4000.0) || (k >= 256 && mn_ratio >= 8000.0) ||
-               (mode == CUMPSGEMM_TF32TC && pays_nt_shape)));
+  // The rules that depend on how well the rounds of CU slots are filled (ro:
+  // rounds_ok, or taken for granted to see whether a cut of C would pay).
+  auto worth_if = [&](const bool ro) {
+    const bool pays_nt = pays_nt_shape && ro;
+    // Shorter K: per tile the in-loop kernels lose more to the split than the pre-pass
+    // costs once C is large (in-loop -> pre-split, TFLOP/s, NN / TN: 8192^2 x 256 261 / 270 -> 277 / 278,
+    // 8192^2 x 384 287 / 297 -> 314 / 313, 6144^2 x 384 254 / 266 -> 280 / 282, 6144^2 x 512 274 / 285 -> 306 / 307,
+    // 4096^2 x 1024 326 / 333 -> 343 / 343, 4096^2 x 2048 350 / 357 -> 384 / 384; 6144^2 x 256 and 4096^2 x 512
+    // are level and stay in-loop, 4096^2 x 256 would lose 8 - 11 %).
+    const bool pays_short = !CPLX && ro &&
+                            ((k >= 256 && mn_ratio >= 4000.0) || (k >= 384 && mn_ratio >= 3000.0) ||
+                             (k >= 1024 && mn_ratio >= 2000.0));
+    // (complex, in-loop -> pre-split, NN / TN: 4096^3 367 / 378 -> 432 / 435 TFLOP/s, 2048^3 355 / 364 -> 401 / 400,
+    // 2048^2 x 1024 349 / 347 -> 372 / 374, 3072^2 x 384 309 / 314 -> 329 / 325, 4096^2 x 256 313 / 320 -> 342 / 349,
+    // 8192^2 x 256 323 / 321 -> 368 / 373; 2048^2 x 512 level, 2048^2 x 384 would lose 5 %, 3072^2 x 256 level)
+    const bool pays_cplx = ro && ((k >= 256 && mn_ratio >= 2000.0) || (k >= 384 && mn_ratio >= 1500.0) ||
+                                  (k >= 1024 && mn_ratio >= 1000.0));
+    const bool pays = CPLX ? pays_cplx : (pays_nt || pays_short);
+    // The uncorrected modes issue a third (FP16TC) or as many (bf16x2) MFMAs per
+    // element as FP16TCEC, so the same pre-pass weighs three times as much for
+    // the former: it is taken for large square-ish problems only.
+    // Measured (in-loop -> pre-split, TFLOP/s): FP16TC 8192^3 580 - 624 -> 930 - 940, 4096^3 586 - 706 ->
+    // 852 - 870, 4096^2 x 1024 505 - 566 -> 634 - 654, 8192^2 x 512 482 - 520 -> 579 - 601, 16384^2 x 256
+    // 390 - 407 -> 461 - 480, 4096^2 x 512 level; bf16x2 8192^3 320 - 377 -> 394 - 396, 4096^2 x 1024
+    // 304 - 337 -> 348 - 355, 8192^2 x 512 275 - 308 -> 318 - 327, 4096^2 x 512 level except NT.
+    // Complex (the 128x64 kernels): FP16TC 4096^3 560 - 678 -> 872 - 891, 2048^3 525 - 640 -> 760 - 779,
+    // 8192^2 x 256 477 - 543 -> 624 - 643; bf16x2 4096^3 350 -> 375, 4096^2 x 1024 333 - 339 -> 365,
+    // 4096^2 x 512 303 - 326 -> 336 - 347.
+    const bool pays_tc =
+        ro &&
+        (CPLX ? (k >= 256 && mn_ratio >= 1000.0)
+              : ((k >= 1024 && mn_ratio >= (mode == CUMPSGEMM_FP16TC ? 1500.0 : 2000.0)) ||
+                 (k >= 512 && mn_ratio >= 4000.0) || (k >= 256 && mn_ratio >= 8000.0) ||
+                 (mode == CUMPSGEMM_TF32TC && pays_nt_shape)));
+    return ch.bf16 ? (pays_bf16 || always) : (ch.tc_only ? (pays_tc || always) : (pays || pays_scaled || always));
+  };
   const bool mode_ok = mode == CUMPSGEMM_FP16TCEC || ch.bf16 || ch.auto_ok || ch.tc_only;
-  const bool worth = ch.bf16 ? (pays_bf16 || always)
-                             : (ch.tc_only ? (pays_tc || always) : (pays || pays_scaled || always));
-  ch.take = mode_ok && !never && shape_ok && worth && force_cls <= 0 && force_split <= 1;
+  const bool base_ok = mode_ok && !never && shape_ok && force_cls <= 0 && force_split <= 1;
+  ch.take = base_ok && worth_if(rounds_ok);
+  // With a mostly empty last round the path still pays for the rounds before
+  // it: the caller cuts C there (6000^2 x 2048: 332 TFLOP/s in-loop, 384 with
+  // everything pre-split and a fifth round that is 40 % full).
+  ch.cut = base_ok && !ch.take && !always && depth == 0 && mode != CUMPSGEMM_AUTO && ptiles > h->num_cus &&
+           worth_if(true);
   // AUTO: the bf16x3 candidate gets its own (gated) pre-pass and planes behind the fp16 ones
   ch.auto_bf16 = ch.take && ch.auto_ok && pays_bf16;
   return ch;
@@ -688,6 +701,43 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
     }
   }
 
+  // C's rows and columns are independent, so a problem can be cut in two along
+  // either; both parts come back here one level down (and are not cut again).
+  // depth1: the level the first part runs at (2: it takes the pre-split path).
+  auto run_cut = [&](const bool by_rows, const uint64_t m1, const uint64_t n1, const int depth1) {
+    if (by_rows) {
+      const T *a2 = a_kc ? a + m1 * lda : a + m1; // op(A) = T: columns of A^T; else rows of A
+      hipblasStatus_t st = run_gemm<T>(h, op_A, op_B, m1, n, k, alpha, a, lda, stridea, b, ldb, strideb,
+                                       beta, c, ldc, stridec, 1, mode, used_id, label, depth1);
+      if (st != HIPBLAS_STATUS_SUCCESS) return st;
+      return run_gemm<T>(h, op_A, op_B, m - m1, n, k, alpha, a2, lda, stridea, b, ldb, strideb, beta,
+                         c + m1, ldc, stridec, 1, mode, nullptr, label, 1);
+    }
+    const T *b2 = b_kc ? b + n1 * ldb : b + n1; // op(B) = N: columns of B; else rows of B^T
+    hipblasStatus_t st = run_gemm<T>(h, op_A, op_B, m, n1, k, alpha, a, lda, stridea, b, ldb, strideb,
+                                     beta, c, ldc, stridec, 1, mode, used_id, label, depth1);
+    if (st != HIPBLAS_STATUS_SUCCESS) return st;
+    return run_gemm<T>(h, op_A, op_B, m, n - n1, k, alpha, a, lda, stridea, b2, ldb, strideb, beta,
+                       c + n1 * ldc, ldc, stridec, 1, mode, nullptr, label, 1);
+  };
+
+  // The pre-split path stepped aside only because its last round of CU slots
+  // would be mostly empty: cut C where its whole rounds end.  The first part
+  // takes the path, the rest is planned on its own (in-loop -> cut, TFLOP/s:
+  // 6000^2 x 2048 306 -> 360, 4200^3 303 -> 335).
+  if (batch == 1 && depth == 0 && !fp16_served && !tuning().no_column_split) {
+    const PreSplitChoice ch =
+        choose_pre_split<CPLX>(h, a_kc, b_kc, m, n, k, batch, mode, force_cls, force_split, depth);
+    if (ch.cut) {
+      const uint64_t tm = (m + ch.bm - 1) / ch.bm, tn = (n + ch.bn - 1) / ch.bn;
+      const uint64_t whole = (tm * tn / h->num_cus) * h->num_cus; // tiles of the whole rounds
+      const uint64_t cols1 = whole / tm, rows1 = whole / tn;      // tile columns / rows that fit in them
+      const bool by_rows = rows1 * tn > cols1 * tm;               // the cut that keeps more of them
+      if (by_rows && rows1 >= 1 && rows1 < tm) return run_cut(true, rows1 * (uint64_t)ch.bm, 0, 2);
+      if (!by_rows && cols1 >= 1 && cols1 < tn) return run_cut(false, 0, cols1 * (uint64_t)ch.bn, 2);
+    }
+  }
+
   // AUTO launches two gated kernels that must agree on how C is prepared, so
   // the split-K decision is taken once, from the first candidate.
   Plan plan0 = make_plan(h, launches[0].p, CPLX, a_kc, b_kc, m, n, k, batch, force_cls, force_split);
@@ -719,22 +769,7 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
     }
     const bool by_rows = cost_rows >= 0.0 && (cost_cols < 0.0 || cost_rows < cost_cols);
     const double cost_cut = by_rows ? cost_rows : cost_cols;
-    if (cost_cut >= 0.0 && cost_cut < 0.93 * plan0.cost) {
-      if (by_rows) {
-        const T *a2 = a_kc ? a + m1 * lda : a + m1; // op(A) = T: columns of A^T; else rows of A
-        hipblasStatus_t st = run_gemm<T>(h, op_A, op_B, m1, n, k, alpha, a, lda, stridea, b, ldb, strideb,
-                                         beta, c, ldc, stridec, 1, mode, used_id, label, 1);
-        if (st != HIPBLAS_STATUS_SUCCESS) return st;
-        return run_gemm<T>(h, op_A, op_B, m - m1, n, k, alpha, a2, lda, stridea, b, ldb, strideb, beta,
-                           c + m1, ldc, stridec, 1, mode, nullptr, label, 1);
-      }
-      const T *b2 = b_kc ? b + n1 * ldb : b + n1; // op(B) = N: columns of B; else rows of B^T
-      hipblasStatus_t st = run_gemm<T>(h, op_A, op_B, m, n1, k, alpha, a, lda, stridea, b, ldb, strideb,
-                                       beta, c, ldc, stridec, 1, mode, used_id, label, 1);
-      if (st != HIPBLAS_STATUS_SUCCESS) return st;
-      return run_gemm<T>(h, op_A, op_B, m, n - n1, k, alpha, a, lda, stridea, b2, ldb, strideb, beta,
-                         c + n1 * ldc, ldc, stridec, 1, mode, nullptr, label, 1);
-    }
+    if (cost_cut >= 0.0 && cost_cut < 0.93 * plan0.cost) return run_cut(by_rows, m1, n1, 1);
   }
 
   if (split) {

@@ -497,6 +497,40 @@ def test_column_split_matches_single_launch(O, handle, dev, monkeypatch, cplx, o
         assert np.array_equal(c.reshape(n, ldc)[:, m:], c0.reshape(n, ldc)[:, m:])
 
 
+# A problem that is worth the pre-split path but whose tiles leave the last round of CU slots
+# mostly empty is cut where the whole rounds end: the first part takes the path (module id 200,
+# workspace allocated), the rest is planned on its own.
+@pytest.mark.parametrize("cplx,mode,opa,opb,m,n,k,alpha,beta", [
+    (False, FP16TCEC, N, N, 4352, 4352, 1024, 1.0, 0.0),       # 17 x 34 tiles of 256 x 128 = 2.26 rounds
+    (False, FP16TCEC, T, N, 4400, 4300, 1030, 1.5, -0.5),      # ragged; cut along the rows or the columns
+    (False, FP16TC, N, T, 4352, 4352, 1024, 1.0, 1.0),         # the uncorrected mode, same tiles
+    (True, FP16TCEC, C, N, 3072, 1536, 1024, 1.0 - 0.5j, 0.25), # 24 x 24 tiles of 128 x 64 = 2.25 rounds ...
+    (True, FP16TCEC, N, N, 2200, 2200, 1024, 1.0, 0.0),        # ... and 18 x 35 = 2.46
+])
+def test_pre_split_path_on_the_whole_rounds_of_a_cut_problem(handle, dev, monkeypatch, cplx, mode, opa, opb,
+                                                              m, n, k, alpha, beta):
+    gen = _gen(cplx)
+    a, lda = make_operand(gen, 75, opa, m, k, 1)
+    b, ldb = make_operand(gen, 76, opb, k, n, 2)
+    ldc = m + 3
+    c0 = gen(77, ldc * n)
+    outs = {}
+    for form in ("cut", "in_loop"):
+        monkeypatch.delenv("CUMPSGEMM_PACKED", raising=False)
+        if form == "in_loop":
+            monkeypatch.setenv("CUMPSGEMM_PACKED", "0")
+        c, st, mid = run_gemm(handle, dev, mode, opa, opb, m, n, k, alpha, a, lda, b, ldb, beta, c0, ldc, cplx,
+                              want_module_id=True)
+        assert st == 0 and (mid == 200) == (form == "cut"), (form, mid)
+        outs[form] = c
+    # every element of C, both sides of the cut: the in-loop result up to the order of summation
+    # (the second part of either form may split K)
+    assert rel_diff(outs["cut"], outs["in_loop"], m, n, ldc) < 2.0 ** -22 * np.sqrt(k)
+    x, y = outs["cut"].view(np.float32).astype(np.float64), outs["in_loop"].view(np.float32).astype(np.float64)
+    assert np.abs(x - y).max() <= 2.0 ** -18 * np.sqrt(k) * np.abs(y).max()
+    assert np.array_equal(outs["cut"].reshape(n, ldc)[:, m:], c0.reshape(n, ldc)[:, m:])
+
+
 # ---- degenerate and skinny shapes ----------------------------------------------------
 @pytest.mark.parametrize("cplx", [False, True])
 def test_k_zero_scales_c(O, handle, dev, cplx):
