@@ -30,6 +30,7 @@ Tuning read_tuning_env() {
   t.force_split = as_int("CUMPSGEMM_FORCE_KSPLIT", 0);
   t.no_persistent = std::getenv("CUMPSGEMM_NO_PERSISTENT") != nullptr;
   t.no_column_split = std::getenv("CUMPSGEMM_NO_COLUMN_SPLIT") != nullptr;
+  t.no_kslices = std::getenv("CUMPSGEMM_NO_KSLICE_GROUPS") != nullptr;
   t.no_fused_scaling = std::getenv("CUMPSGEMM_NO_FUSED_SCALING") != nullptr;
   if (const char *v = std::getenv("CUMPSGEMM_PERSISTENT_MAX_STEPS")) t.persistent_max_steps = (unsigned)std::atoi(v);
   if (const char *v = std::getenv("CUMPSGEMM_MAX_WORKSPACE_BYTES")) t.max_workspace_bytes = std::strtoull(v, nullptr, 10);
@@ -813,7 +814,21 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
       launch_walk(args, grid, h->stream);
     } else {
       const dim3 grid(plan.tiles_m * plan.tiles_n, (unsigned)batch, plan.ksplit);
-      launch_plain(args, grid, h->stream);
+      // At most one small workgroup per CU: its four waves, one per SIMD, are
+      // bound by the latency of their own chain of LDS reads, MFMAs and staging,
+      // so the form with two wave groups (a K-slice of every step each) is
+      // launched -- where it was measured faster: op(B) K-contiguous and a mode
+      // with correction terms or bf16 planes (1024^3, plain -> two groups, us:
+      // FP16TCEC NN 19.3 -> 16.4, TN 16.2 -> 14.8, bf16x3 NN 28.1 -> 21.5, bf16x2
+      // NN 19.7 -> 16.5; FP16TC level; with op(B) = T 4 - 15 % slower).
+      const uint64_t groups = (uint64_t)grid.x * grid.y * grid.z;
+      auto launch_groups = launch_plain == e->launch_scaled ? e->launch_scaled_kslices : e->launch_kslices;
+      if (launch_groups != nullptr && groups <= (uint64_t)h->num_cus && b_kc &&
+          launches[i].p != Prec::FP16TC && !tuning().no_kslices) {
+        launch_groups(args, grid, h->stream);
+      } else {
+        launch_plain(args, grid, h->stream);
+      }
     }
     if (used_id != nullptr) {
       *used_id = (mode == CUMPSGEMM_AUTO) ? ~0u : (unsigned)plan.cls + (split ? 100u : 0u);

@@ -252,10 +252,17 @@ __device__ inline f4v_t mfma_block(const u4_t a, const u4_t b, const f4v_t c) {
 //         and B were split beforehand into fp16 / bf16 planes laid out as the
 //         LDS image of every (tile, K-step), see pack_split_kernel; staging is
 //         a plain 16-byte copy, no arithmetic.
+//   KS2 (real two-buffer kernels): twice the waves; the two wave groups take
+//         one 16-wide K-slice of every step each and add their accumulators
+//         through LDS at the end, and one group stages A, the other B.  For a
+//         problem of no more tiles than CUs: two waves per SIMD instead of one
+//         shorten the chain LDS read -> MFMA -> split -> LDS write of a step.
 template <Prec P_, bool CPLX_, bool A_KC_, bool B_KC_, int BM_, int BN_, int WM_,
           int WN_, int OCC_ = 1, bool DEEP_ = false, bool PERSIST_ = false, bool SCALED_ = false,
-          bool PACKED_ = false>
+          bool PACKED_ = false, bool KS2_ = false>
 struct GemmCfg {
+  static_assert(!KS2_ || (!CPLX_ && !DEEP_ && !PACKED_), "K-slice split: real two-buffer kernels");
+  static constexpr bool KS2 = KS2_;
   // (PACKED + SCALED: the operands were scaled when they were pre-split; the
   // kernel only folds the inverse scaling of C into alpha)
   static_assert(!PACKED_ || (DEEP_ && (P_ != Prec::BF16X3 || !CPLX_)),
@@ -276,11 +283,10 @@ struct GemmCfg {
   static constexpr bool A_KC = A_KC_;
   static constexpr bool B_KC = B_KC_;
   static constexpr int BM = BM_, BN = BN_, BK = 32, WM = WM_, WN = WN_;
-  static constexpr int NWAVES = (BM / WM) * (BN / WN);
+  static constexpr int TILE_WAVES = (BM / WM) * (BN / WN); // waves that cover the tile once
+  static constexpr int NWAVES = TILE_WAVES * (KS2_ ? 2 : 1);
   static constexpr int NT = NWAVES * 64;
-  // MFMA blocks per wave tile, accumulator registers per block, and the two
-  // halves a K-step's MFMAs are issued in: the two 16-wide K-slices (edge 32) or
-  // the two halves of the wave tile's columns (edge 16, one 32-wide K-slice)
+  // MFMA block edge, blocks per wave tile, accumulator registers per block
   // (in-loop kernels measured with edge 16, all sizes and batches: complex
   // bf16x3 + 5 - 7 % throughout; the others between - 8 % and + 9 % with a mean
   // of zero, so they keep 32)
@@ -304,7 +310,10 @@ struct GemmCfg {
   static constexpr int A_STAGE_BYTES = A_PLANE_BYTES * NP * NCOMP;
   static constexpr int B_STAGE_BYTES = B_PLANE_BYTES * NP * NCOMP;
   static constexpr int STAGE_BYTES = A_STAGE_BYTES + B_STAGE_BYTES;
-  static constexpr int LDS_BYTES = NSTAGE * STAGE_BYTES;
+  // (KS2: the second wave group's accumulators pass through LDS once)
+  static constexpr int REDUCE_BYTES = KS2_ ? TILE_WAVES * 64 * prec_traits<P>::NACC * TM * TN * NV * 4 : 0;
+  static constexpr int LDS_BYTES = NSTAGE * STAGE_BYTES > REDUCE_BYTES ? NSTAGE * STAGE_BYTES : REDUCE_BYTES;
+  static_assert(!KS2_ || (MT == 32 && BM * 4 + BN * 4 == NT), "one staging unit per thread: A then B");
   // staging units: one unit = (row, chunk of 8 K-values)
   // (when a tile has fewer units than the workgroup has threads, the surplus
   // waves simply stage nothing for that operand)
@@ -404,7 +413,9 @@ __device__ inline void map_tile_batched(uint32_t vid, uint32_t tiles_m, uint32_t
 // in scalar registers, the offsets are computed once per kernel.
 // Out-of-range elements read as zero, which contributes nothing to the sums.
 // ---------------------------------------------------------------------------
-template <bool CPLX, bool KC, int ROWS, int U, int NT, bool HALF_UNITS = false>
+//   TID0: with fewer units than threads, the first thread that stages this
+//         operand (the ROWS * 4 threads from there on do).
+template <bool CPLX, bool KC, int ROWS, int U, int NT, bool HALF_UNITS = false, int TID0 = 0>
 struct tile_loader {
   static constexpr int NC = CPLX ? 2 : 1;
   static constexpr int ES = CPLX ? 2 : 1;
@@ -417,17 +428,20 @@ struct tile_loader {
   // (HALF_UNITS: the precisions this pays for, measured -- FP16TCEC and bf16x2; the
   // costlier bf16x3 split and the single-product FP16TC kernels keep whole units)
   static constexpr bool HALF = HALF_UNITS && CPLX && (ROWS * 4 * 2 == NT);
+  static_assert(TID0 == 0 || (PARTIAL && !HALF), "TID0: partial tiles of whole units");
   static constexpr int KV = HALF ? 4 : 8; // K-values a thread handles per unit
 
   // whether this thread stages anything of this operand (wave-uniform)
-  __device__ static inline bool active(int tid) { return !PARTIAL || HALF || tid < ROWS * 4; }
+  __device__ static inline bool active(int tid) {
+    return !PARTIAL || HALF || (tid >= TID0 && tid < TID0 + ROWS * 4);
+  }
   // ... in the register-staged copy of pre-split planes (whole 16-byte chunks)
   __device__ static inline bool copy_active(int tid) { return !PARTIAL || tid < ROWS * 4; }
   // which half of its unit (0 unless HALF)
   __device__ static inline int half_of(int tid) { return HALF ? (tid & 1) : 0; }
 
   __device__ static inline void unit_coords(int u, int tid, int &row, int &chunk) {
-    const int id = (HALF ? tid >> 1 : tid) + u * NT;
+    const int id = (HALF ? tid >> 1 : tid - TID0) + u * NT;
     if constexpr (KC) {
       chunk = id & 3;
       row = id >> 2;
@@ -769,8 +783,11 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm = wave % (BM / Cfg::WM);
-  const int wn = wave / (BM / Cfg::WM);
+  // (KS2: two groups of waves cover the tile, each with one K-slice of every step)
+  const int wave_t = Cfg::KS2 ? wave % Cfg::TILE_WAVES : wave;
+  const int kgrp = Cfg::KS2 ? wave / Cfg::TILE_WAVES : 0;
+  const int wm = wave_t % (BM / Cfg::WM);
+  const int wn = wave_t / (BM / Cfg::WM);
 
   // (persistent kernels: the first tile of this workgroup's list; see below)
   uint32_t tile_m, tile_n, tile_b = blockIdx.y;
@@ -825,7 +842,7 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
 
   constexpr bool HALF_UNITS = (P == Prec::FP16TCEC || P == Prec::BF16X2);
   using LA = tile_loader<CPLX, Cfg::A_KC, BM, Cfg::UA, NT, HALF_UNITS>;
-  using LB = tile_loader<CPLX, Cfg::B_KC, BN, Cfg::UB, NT, HALF_UNITS>;
+  using LB = tile_loader<CPLX, Cfg::B_KC, BN, Cfg::UB, NT, HALF_UNITS, Cfg::KS2 ? BM * 4 : 0>;
 
   const int rows_a = (int)((args.m - ml0 < (uint32_t)BM) ? args.m - ml0 : BM);
   const int rows_b = (int)((args.n - nl0 < (uint32_t)BN) ? args.n - nl0 : BN);
@@ -909,7 +926,7 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
   int a_frag_off[2], b_frag_off[2];
 #pragma unroll
   for (int kk = 0; kk < 2; kk++) {
-    const int chunk = MT == 32 ? 2 * kk + frag_g : frag_g;
+    const int chunk = MT == 32 ? 2 * (Cfg::KS2 ? kgrp : kk) + frag_g : frag_g;
     a_frag_off[kk] = lds_offset(wm * Cfg::WM + frag_row, chunk);
     b_frag_off[kk] = lds_offset(wn * Cfg::WN + frag_row, chunk);
   }
@@ -984,11 +1001,16 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
   // as many after a 16x16x32 MFMA, which is half as long)
   constexpr int SCHED_VALU = MT == 32 ? CUMPSGEMM_SCHED_VALU : (CUMPSGEMM_SCHED_VALU + 1) / 2;
   constexpr int STEP_MFMAS = (MT == 32 ? 2 : 1) * PT::NPROD * TM * TN * (CPLX ? 4 : 1);
+  // a whole K-step from one LDS buffer (KS2: this wave group's K-slice of it)
   auto mma_tile = [&](int stage) {
     Frags f0, f1;
     frag_load(f0, stage, 0);
-    frag_load(f1, stage, 1);
-    frag_mma(f0, f1);
+    if constexpr (Cfg::KS2) {
+      frag_mma_part(f0, f0, 0, 0);
+    } else {
+      frag_load(f1, stage, 1);
+      frag_mma(f0, f1);
+    }
   };
 
   // ---- epilogue -----------------------------------------------------------
@@ -1310,9 +1332,7 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
       block_sync_lds();
       for (int t = 0; t < nk; t++) {
         const int cur = t & 1;
-        frag_load(f0, cur, 0);
-        frag_load(f1, cur, 1);
-        frag_mma(f0, f1);
+        mma_tile(cur);
         if (t + 1 < nk) lstore(cur ^ 1);
         gload(clamp(t + 2), fast_tag);
         block_sync_lds();
@@ -1435,6 +1455,34 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
     }
   } else {
     pipeline((klen + BK - 1) / BK, std::false_type{});
+  }
+
+  if constexpr (Cfg::KS2) {
+    // the second wave group hands its sums over (register r of lane l of wave w
+    // at float (w * NREG + r) * 64 + l: consecutive lanes, consecutive banks)
+    constexpr int NREG = PT::NACC * TN * TM * NV;
+    float *red = reinterpret_cast<float *>(lds) + wave_t * NREG * 64 + lane;
+    __syncthreads(); // (every wave is done with the last tile's fragments)
+    if (kgrp == 1) {
+#pragma unroll
+      for (int s = 0; s < PT::NACC; s++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+          for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int v = 0; v < NV; v++) red[(((s * TN + j) * TM + i) * NV + v) * 64] = acc[0][s][j][i][v];
+    }
+    __syncthreads();
+    if (kgrp == 1) return;
+#pragma unroll
+    for (int s = 0; s < PT::NACC; s++)
+#pragma unroll
+      for (int j = 0; j < TN; j++)
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+          for (int v = 0; v < NV; v++) acc[0][s][j][i][v] += red[(((s * TN + j) * TM + i) * NV + v) * 64];
   }
 
   if (ml0 == m0 && nl0 == n0 && rows_a == BM && rows_b == BN) {

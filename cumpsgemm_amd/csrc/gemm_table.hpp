@@ -19,6 +19,10 @@ struct KernelEntry {
   // tables only, else nullptr)
   void (*launch_scaled)(const GemmArgs &, dim3 grid, hipStream_t stream);
   void (*launch_scaled_persistent)(const GemmArgs &, dim3 grid, hipStream_t stream);
+  // variant with twice the waves, each group taking one K-slice of every step
+  // (small real tiles only, else nullptr): for problems of no more tiles than CUs
+  void (*launch_kslices)(const GemmArgs &, dim3 grid, hipStream_t stream);
+  void (*launch_scaled_kslices)(const GemmArgs &, dim3 grid, hipStream_t stream); // (FP16TCEC tables only)
   int bm, bn;      // workgroup tile
   int wm, wn;      // wave tile
   int threads;     // workgroup size
@@ -71,6 +75,14 @@ template <class Cfg> constexpr KernelEntry make_entry(const char *name) {
     e.launch_scaled = &launch_cfg<typename Cfg::scaled_type>;
     if constexpr (Cfg::DEEP)
       e.launch_scaled_persistent = &launch_cfg<typename Cfg::scaled_type::persistent_type>;
+  }
+  if constexpr (!Cfg::CPLX && !Cfg::DEEP && Cfg::MT == 32 && Cfg::BM * 4 + Cfg::BN * 4 == 2 * Cfg::NT) {
+    e.launch_kslices = &launch_cfg<GemmCfg<Cfg::P, false, Cfg::A_KC, Cfg::B_KC, Cfg::BM, Cfg::BN, Cfg::WM, Cfg::WN,
+                                           Cfg::OCC, false, false, false, false, true>>;
+    if constexpr (Cfg::P == Prec::FP16TCEC) {
+      e.launch_scaled_kslices = &launch_cfg<GemmCfg<Cfg::P, false, Cfg::A_KC, Cfg::B_KC, Cfg::BM, Cfg::BN, Cfg::WM,
+                                                    Cfg::WN, Cfg::OCC, false, false, true, false, true>>;
+    }
   }
   e.bm = Cfg::BM;
   e.bn = Cfg::BN;

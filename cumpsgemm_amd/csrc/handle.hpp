@@ -70,6 +70,7 @@ struct Tuning {
   int force_split = 0;  // CUMPSGEMM_FORCE_KSPLIT
   bool no_persistent = false;    // CUMPSGEMM_NO_PERSISTENT
   bool no_column_split = false;  // CUMPSGEMM_NO_COLUMN_SPLIT
+  bool no_kslices = false;       // CUMPSGEMM_NO_KSLICE_GROUPS
   bool no_fused_scaling = false; // CUMPSGEMM_NO_FUSED_SCALING
   unsigned persistent_max_steps = 32; // CUMPSGEMM_PERSISTENT_MAX_STEPS
   // CUMPSGEMM_MAX_WORKSPACE_BYTES: the pre-split path is not taken when its

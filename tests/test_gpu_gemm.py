@@ -531,6 +531,52 @@ def test_pre_split_path_on_the_whole_rounds_of_a_cut_problem(handle, dev, monkey
     assert np.array_equal(outs["cut"].reshape(n, ldc)[:, m:], c0.reshape(n, ldc)[:, m:])
 
 
+# ---- small problems: two wave groups per workgroup --------------------------------------
+# A real problem of no more small tiles than CUs runs the 64 x 64 kernel with twice the waves:
+# each group takes one K-slice of every step and the sums meet in LDS at the end.  Same products
+# as the four-wave kernel, another order of summation.
+@pytest.mark.parametrize("mode", [FP16TCEC, TF32TCEC, TF32TC])
+@pytest.mark.parametrize("opa,opb,m,n,k,batch,alpha,beta", [
+    (N, N, 1024, 1024, 1024, 1, 1.0, 0.0),        # 256 interior tiles
+    (T, N, 1000, 900, 777, 1, 1.5, -0.5),         # edge tiles, ragged K, beta != 0
+    (N, N, 300, 200, 4100, 1, 1.0, 1.0),          # K split between workgroups as well (atomic write-out)
+    (T, N, 256, 192, 520, 16, -1.0, 0.25),        # a batch: 12 tiles x 16 matrices
+    (N, N, 70, 33, 50, 1, 1.0, 0.0),              # one partial tile, two K-steps
+])
+def test_two_wave_groups_match_the_four_wave_kernel(O, handle, dev, monkeypatch, mode, opa, opb, m, n, k, batch,
+                                                    alpha, beta):
+    gen = _gen(False)
+    ar, ac = (m, k) if opa == N else (k, m)
+    lda, ldb, ldc = ar + 1, k + 2, m + 3
+    sa, sb, sc = lda * ac + 5, ldb * n + 3, ldc * n + 7
+    a, b, c0 = gen(85, sa * batch), gen(86, sb * batch), gen(87, sc * batch)
+    da, db = dev.up(a), dev.up(b)
+    outs = []
+    for plain in (False, True):
+        if plain:
+            monkeypatch.setenv("CUMPSGEMM_NO_KSLICE_GROUPS", "1")
+        else:
+            monkeypatch.delenv("CUMPSGEMM_NO_KSLICE_GROUPS", raising=False)
+        dc = dev.up(c0)
+        st = handle.gemm_strided_batch(opa, opb, m, n, k, alpha, da, lda, sa, db, ldb, sb, beta, dc, ldc, sc,
+                                       batch, mode)
+        assert st == 0
+        outs.append(dev.down(dc, np.float32))
+    for i in (0, batch - 1):
+        x, y = outs[0][i * sc:i * sc + ldc * n], outs[1][i * sc:i * sc + ldc * n]
+        assert rel_diff(x, y, m, n, ldc) < 2.0 ** -22 * np.sqrt(k)
+        assert np.array_equal(x.reshape(n, ldc)[:, m:], c0[i * sc:i * sc + ldc * n].reshape(n, ldc)[:, m:])
+        ai, bi, ci0 = a[i * sa:(i + 1) * sa], b[i * sb:(i + 1) * sb], c0[i * sc:i * sc + ldc * n]
+        ref = O.gemm_fp64(opa, opb, m, n, k, alpha, ai, lda, bi, ldb, beta, ci0, ldc)
+        if mode == TF32TC:
+            assert O.residual(ref, x, m, n, ldc) <= 2.0 ** -14
+        else:
+            cf = oracle_gemm(O, FP32, opa, opb, m, n, k, alpha, ai, lda, bi, ldb, beta, ci0, ldc)
+            assert O.residual(ref, x, m, n, ldc) <= 2.0 * O.residual(ref, cf, m, n, ldc) + 2.0 ** -24
+    # (the gaps between the matrices of the batch stay as they were)
+    assert np.array_equal(outs[0][ldc * n:sc], c0[ldc * n:sc])
+
+
 # ---- degenerate and skinny shapes ----------------------------------------------------
 @pytest.mark.parametrize("cplx", [False, True])
 def test_k_zero_scales_c(O, handle, dev, cplx):
