@@ -1,7 +1,6 @@
 """The micro-benchmarks under tests/native/microbench (the measurements behind the MFMA shape, the
 LDS swizzle of the pre-split planes and the placement of the write-out's stores) build and run:
-short runs, checked for a clean exit and plausible figures -- the figures themselves are in
-profiles/."""
+short runs, checked for a clean exit and plausible figures."""
 import os
 import re
 import subprocess
