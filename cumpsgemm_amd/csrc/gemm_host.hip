@@ -820,7 +820,8 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
       // launched -- where it was measured faster: op(B) K-contiguous and a mode
       // with correction terms or bf16 planes (1024^3, plain -> two groups, us:
       // FP16TCEC NN 19.3 -> 16.4, TN 16.2 -> 14.8, bf16x3 NN 28.1 -> 21.5, bf16x2
-      // NN 19.7 -> 16.5; FP16TC level; with op(B) = T 4 - 15 % slower).
+      // NN 19.7 -> 16.5; complex FP16TCEC NN 38.6 -> 34.5, bf16x2 38.0 -> 33.5;
+      // FP16TC level; with op(B) = T 4 - 15 % slower).
       const uint64_t groups = (uint64_t)grid.x * grid.y * grid.z;
       auto launch_groups = launch_plain == e->launch_scaled ? e->launch_scaled_kslices : e->launch_kslices;
       if (launch_groups != nullptr && groups <= (uint64_t)h->num_cus && b_kc &&

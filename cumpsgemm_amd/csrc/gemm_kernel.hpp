@@ -252,16 +252,17 @@ __device__ inline f4v_t mfma_block(const u4_t a, const u4_t b, const f4v_t c) {
 //         and B were split beforehand into fp16 / bf16 planes laid out as the
 //         LDS image of every (tile, K-step), see pack_split_kernel; staging is
 //         a plain 16-byte copy, no arithmetic.
-//   KS2 (real two-buffer kernels): twice the waves; the two wave groups take
+//   KS2 (two-buffer kernels): twice the waves; the two wave groups take
 //         one 16-wide K-slice of every step each and add their accumulators
-//         through LDS at the end, and one group stages A, the other B.  For a
+//         through LDS at the end, and one group stages A, the other B (complex
+//         half-unit loaders: every thread half a unit of each).  For a
 //         problem of no more tiles than CUs: two waves per SIMD instead of one
 //         shorten the chain LDS read -> MFMA -> split -> LDS write of a step.
 template <Prec P_, bool CPLX_, bool A_KC_, bool B_KC_, int BM_, int BN_, int WM_,
           int WN_, int OCC_ = 1, bool DEEP_ = false, bool PERSIST_ = false, bool SCALED_ = false,
           bool PACKED_ = false, bool KS2_ = false>
 struct GemmCfg {
-  static_assert(!KS2_ || (!CPLX_ && !DEEP_ && !PACKED_), "K-slice split: real two-buffer kernels");
+  static_assert(!KS2_ || (!DEEP_ && !PACKED_), "K-slice split: two-buffer kernels");
   static constexpr bool KS2 = KS2_;
   // (PACKED + SCALED: the operands were scaled when they were pre-split; the
   // kernel only folds the inverse scaling of C into alpha)
@@ -311,7 +312,8 @@ struct GemmCfg {
   static constexpr int B_STAGE_BYTES = B_PLANE_BYTES * NP * NCOMP;
   static constexpr int STAGE_BYTES = A_STAGE_BYTES + B_STAGE_BYTES;
   // (KS2: the second wave group's accumulators pass through LDS once)
-  static constexpr int REDUCE_BYTES = KS2_ ? TILE_WAVES * 64 * prec_traits<P>::NACC * TM * TN * NV * 4 : 0;
+  static constexpr int REDUCE_BYTES =
+      KS2_ ? TILE_WAVES * 64 * (CPLX_ ? 4 : 1) * prec_traits<P>::NACC * TM * TN * NV * 4 : 0;
   static constexpr int LDS_BYTES = NSTAGE * STAGE_BYTES > REDUCE_BYTES ? NSTAGE * STAGE_BYTES : REDUCE_BYTES;
   static_assert(!KS2_ || (MT == 32 && BM * 4 + BN * 4 == NT), "one staging unit per thread: A then B");
   // staging units: one unit = (row, chunk of 8 K-values)
@@ -842,7 +844,9 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
 
   constexpr bool HALF_UNITS = (P == Prec::FP16TCEC || P == Prec::BF16X2);
   using LA = tile_loader<CPLX, Cfg::A_KC, BM, Cfg::UA, NT, HALF_UNITS>;
-  using LB = tile_loader<CPLX, Cfg::B_KC, BN, Cfg::UB, NT, HALF_UNITS, Cfg::KS2 ? BM * 4 : 0>;
+  // (KS2: the second wave group stages B, unless every thread takes half a unit of each operand)
+  constexpr bool HALF_B = HALF_UNITS && CPLX && (BN * 4 * 2 == NT);
+  using LB = tile_loader<CPLX, Cfg::B_KC, BN, Cfg::UB, NT, HALF_UNITS, (Cfg::KS2 && !HALF_B) ? BM * 4 : 0>;
 
   const int rows_a = (int)((args.m - ml0 < (uint32_t)BM) ? args.m - ml0 : BM);
   const int rows_b = (int)((args.n - nl0 < (uint32_t)BN) ? args.n - nl0 : BN);
@@ -1460,10 +1464,26 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
   if constexpr (Cfg::KS2) {
     // the second wave group hands its sums over (register r of lane l of wave w
     // at float (w * NREG + r) * 64 + l: consecutive lanes, consecutive banks)
-    constexpr int NREG = PT::NACC * TN * TM * NV;
+    constexpr int NREG = NACCSET * PT::NACC * TN * TM * NV;
     float *red = reinterpret_cast<float *>(lds) + wave_t * NREG * 64 + lane;
     __syncthreads(); // (every wave is done with the last tile's fragments)
     if (kgrp == 1) {
+#pragma unroll
+      for (int q = 0; q < NACCSET; q++)
+#pragma unroll
+        for (int s = 0; s < PT::NACC; s++)
+#pragma unroll
+          for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+              for (int v = 0; v < NV; v++)
+                red[((((q * PT::NACC + s) * TN + j) * TM + i) * NV + v) * 64] = acc[q][s][j][i][v];
+    }
+    __syncthreads();
+    if (kgrp == 1) return;
+#pragma unroll
+    for (int q = 0; q < NACCSET; q++)
 #pragma unroll
       for (int s = 0; s < PT::NACC; s++)
 #pragma unroll
@@ -1471,18 +1491,8 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
 #pragma unroll
           for (int i = 0; i < TM; i++)
 #pragma unroll
-            for (int v = 0; v < NV; v++) red[(((s * TN + j) * TM + i) * NV + v) * 64] = acc[0][s][j][i][v];
-    }
-    __syncthreads();
-    if (kgrp == 1) return;
-#pragma unroll
-    for (int s = 0; s < PT::NACC; s++)
-#pragma unroll
-      for (int j = 0; j < TN; j++)
-#pragma unroll
-        for (int i = 0; i < TM; i++)
-#pragma unroll
-          for (int v = 0; v < NV; v++) acc[0][s][j][i][v] += red[(((s * TN + j) * TM + i) * NV + v) * 64];
+            for (int v = 0; v < NV; v++)
+              acc[q][s][j][i][v] += red[((((q * PT::NACC + s) * TN + j) * TM + i) * NV + v) * 64];
   }
 
   if (ml0 == m0 && nl0 == n0 && rows_a == BM && rows_b == BN) {

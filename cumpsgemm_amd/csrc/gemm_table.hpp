@@ -76,12 +76,12 @@ template <class Cfg> constexpr KernelEntry make_entry(const char *name) {
     if constexpr (Cfg::DEEP)
       e.launch_scaled_persistent = &launch_cfg<typename Cfg::scaled_type::persistent_type>;
   }
-  if constexpr (!Cfg::CPLX && !Cfg::DEEP && Cfg::MT == 32 && Cfg::BM * 4 + Cfg::BN * 4 == 2 * Cfg::NT) {
-    e.launch_kslices = &launch_cfg<GemmCfg<Cfg::P, false, Cfg::A_KC, Cfg::B_KC, Cfg::BM, Cfg::BN, Cfg::WM, Cfg::WN,
-                                           Cfg::OCC, false, false, false, false, true>>;
+  if constexpr (!Cfg::DEEP && Cfg::MT == 32 && Cfg::BM * 4 + Cfg::BN * 4 == 2 * Cfg::NT) {
+    e.launch_kslices = &launch_cfg<GemmCfg<Cfg::P, Cfg::CPLX, Cfg::A_KC, Cfg::B_KC, Cfg::BM, Cfg::BN, Cfg::WM,
+                                           Cfg::WN, Cfg::OCC, false, false, false, false, true>>;
     if constexpr (Cfg::P == Prec::FP16TCEC) {
-      e.launch_scaled_kslices = &launch_cfg<GemmCfg<Cfg::P, false, Cfg::A_KC, Cfg::B_KC, Cfg::BM, Cfg::BN, Cfg::WM,
-                                                    Cfg::WN, Cfg::OCC, false, false, true, false, true>>;
+      e.launch_scaled_kslices = &launch_cfg<GemmCfg<Cfg::P, Cfg::CPLX, Cfg::A_KC, Cfg::B_KC, Cfg::BM, Cfg::BN,
+                                                    Cfg::WM, Cfg::WN, Cfg::OCC, false, false, true, false, true>>;
     }
   }
   e.bm = Cfg::BM;

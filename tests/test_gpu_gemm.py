@@ -532,20 +532,22 @@ def test_pre_split_path_on_the_whole_rounds_of_a_cut_problem(handle, dev, monkey
 
 
 # ---- small problems: two wave groups per workgroup --------------------------------------
-# A real problem of no more small tiles than CUs runs the 64 x 64 kernel with twice the waves:
+# A problem of no more small tiles than CUs (op(B) K-contiguous) runs the 64 x 64 kernel with twice the waves:
 # each group takes one K-slice of every step and the sums meet in LDS at the end.  Same products
 # as the four-wave kernel, another order of summation.
 @pytest.mark.parametrize("mode", [FP16TCEC, TF32TCEC, TF32TC])
-@pytest.mark.parametrize("opa,opb,m,n,k,batch,alpha,beta", [
-    (N, N, 1024, 1024, 1024, 1, 1.0, 0.0),        # 256 interior tiles
-    (T, N, 1000, 900, 777, 1, 1.5, -0.5),         # edge tiles, ragged K, beta != 0
-    (N, N, 300, 200, 4100, 1, 1.0, 1.0),          # K split between workgroups as well (atomic write-out)
-    (T, N, 256, 192, 520, 16, -1.0, 0.25),        # a batch: 12 tiles x 16 matrices
-    (N, N, 70, 33, 50, 1, 1.0, 0.0),              # one partial tile, two K-steps
+@pytest.mark.parametrize("cplx,opa,opb,m,n,k,batch,alpha,beta", [
+    (False, N, N, 1024, 1024, 1024, 1, 1.0, 0.0),        # 256 interior tiles
+    (False, T, N, 1000, 900, 777, 1, 1.5, -0.5),         # edge tiles, ragged K, beta != 0
+    (False, N, N, 300, 200, 4100, 1, 1.0, 1.0),          # K split between workgroups as well (atomic write-out)
+    (False, T, N, 256, 192, 520, 16, -1.0, 0.25),        # a batch: 12 tiles x 16 matrices
+    (False, N, N, 70, 33, 50, 1, 1.0, 0.0),              # one partial tile, two K-steps
+    (True, N, N, 512, 512, 512, 1, 1.0, 0.0),            # complex: every thread stages half a unit of A and of B
+    (True, C, N, 500, 450, 333, 2, 1.0 - 0.5j, 0.5j),    # conjugated A, edge tiles, ragged K, complex scalars
 ])
-def test_two_wave_groups_match_the_four_wave_kernel(O, handle, dev, monkeypatch, mode, opa, opb, m, n, k, batch,
-                                                    alpha, beta):
-    gen = _gen(False)
+def test_two_wave_groups_match_the_four_wave_kernel(O, handle, dev, monkeypatch, mode, cplx, opa, opb, m, n, k,
+                                                    batch, alpha, beta):
+    gen = _gen(cplx)   # (complex bf16x3 has no two-group form: both runs launch the same kernel)
     ar, ac = (m, k) if opa == N else (k, m)
     lda, ldb, ldc = ar + 1, k + 2, m + 3
     sa, sb, sc = lda * ac + 5, ldb * n + 3, ldc * n + 7
@@ -559,9 +561,9 @@ def test_two_wave_groups_match_the_four_wave_kernel(O, handle, dev, monkeypatch,
             monkeypatch.delenv("CUMPSGEMM_NO_KSLICE_GROUPS", raising=False)
         dc = dev.up(c0)
         st = handle.gemm_strided_batch(opa, opb, m, n, k, alpha, da, lda, sa, db, ldb, sb, beta, dc, ldc, sc,
-                                       batch, mode)
+                                       batch, mode, cplx=cplx)
         assert st == 0
-        outs.append(dev.down(dc, np.float32))
+        outs.append(dev.down(dc, np.complex64 if cplx else np.float32))
     for i in (0, batch - 1):
         x, y = outs[0][i * sc:i * sc + ldc * n], outs[1][i * sc:i * sc + ldc * n]
         assert rel_diff(x, y, m, n, ldc) < 2.0 ** -22 * np.sqrt(k)
