@@ -817,14 +817,14 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
       // At most one small workgroup per CU: its four waves, one per SIMD, are
       // bound by the latency of their own chain of LDS reads, MFMAs and staging,
       // so the form with two wave groups (a K-slice of every step each) is
-      // launched -- where it was measured faster: op(B) K-contiguous and a mode
-      // with correction terms or bf16 planes (1024^3, plain -> two groups, us:
-      // FP16TCEC NN 19.3 -> 16.4, TN 16.2 -> 14.8, bf16x3 NN 28.1 -> 21.5, bf16x2
-      // NN 19.7 -> 16.5; complex FP16TCEC NN 38.6 -> 34.5, bf16x2 38.0 -> 33.5;
-      // FP16TC level; with op(B) = T 4 - 15 % slower).
+      // launched -- where it was measured faster: an operand K-contiguous and a
+      // mode with correction terms or bf16 planes (1024^3, plain -> two groups,
+      // us: FP16TCEC NN 19.3 -> 16.4, TN 16.2 -> 14.8, TT 18.6 -> 17.9, bf16x3 NN
+      // 28.1 -> 21.5, bf16x2 NN 19.7 -> 16.5; complex FP16TCEC NN 38.6 -> 34.5,
+      // bf16x2 38.0 -> 33.5; FP16TC level or slower; op(A) = N with op(B) = T level).
       const uint64_t groups = (uint64_t)grid.x * grid.y * grid.z;
       auto launch_groups = launch_plain == e->launch_scaled ? e->launch_scaled_kslices : e->launch_kslices;
-      if (launch_groups != nullptr && groups <= (uint64_t)h->num_cus && b_kc &&
+      if (launch_groups != nullptr && groups <= (uint64_t)h->num_cus && (a_kc || b_kc) &&
           launches[i].p != Prec::FP16TC && !tuning().no_kslices) {
         launch_groups(args, grid, h->stream);
       } else {

@@ -532,7 +532,7 @@ def test_pre_split_path_on_the_whole_rounds_of_a_cut_problem(handle, dev, monkey
 
 
 # ---- small problems: two wave groups per workgroup --------------------------------------
-# A problem of no more small tiles than CUs (op(B) K-contiguous) runs the 64 x 64 kernel with twice the waves:
+# A problem of no more small tiles than CUs (an operand K-contiguous) runs the 64 x 64 kernel with twice the waves:
 # each group takes one K-slice of every step and the sums meet in LDS at the end.  Same products
 # as the four-wave kernel, another order of summation.
 @pytest.mark.parametrize("mode", [FP16TCEC, TF32TCEC, TF32TC])
@@ -542,6 +542,7 @@ def test_pre_split_path_on_the_whole_rounds_of_a_cut_problem(handle, dev, monkey
     (False, N, N, 300, 200, 4100, 1, 1.0, 1.0),          # K split between workgroups as well (atomic write-out)
     (False, T, N, 256, 192, 520, 16, -1.0, 0.25),        # a batch: 12 tiles x 16 matrices
     (False, N, N, 70, 33, 50, 1, 1.0, 0.0),              # one partial tile, two K-steps
+    (False, T, T, 640, 500, 300, 1, 1.0, 0.0),           # op(B) = T: the groups trade operands
     (True, N, N, 512, 512, 512, 1, 1.0, 0.0),            # complex: every thread stages half a unit of A and of B
     (True, C, N, 500, 450, 333, 2, 1.0 - 0.5j, 0.5j),    # conjugated A, edge tiles, ragged K, complex scalars
 ])
@@ -549,8 +550,9 @@ def test_two_wave_groups_match_the_four_wave_kernel(O, handle, dev, monkeypatch,
                                                     batch, alpha, beta):
     gen = _gen(cplx)   # (complex bf16x3 has no two-group form: both runs launch the same kernel)
     ar, ac = (m, k) if opa == N else (k, m)
-    lda, ldb, ldc = ar + 1, k + 2, m + 3
-    sa, sb, sc = lda * ac + 5, ldb * n + 3, ldc * n + 7
+    br, bc = (k, n) if opb == N else (n, k)
+    lda, ldb, ldc = ar + 1, br + 2, m + 3
+    sa, sb, sc = lda * ac + 5, ldb * bc + 3, ldc * n + 7
     a, b, c0 = gen(85, sa * batch), gen(86, sb * batch), gen(87, sc * batch)
     da, db = dev.up(a), dev.up(b)
     outs = []
