@@ -819,7 +819,7 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
       // so the form with two wave groups (a K-slice of every step each) is
       // launched -- where it was measured faster: an operand K-contiguous and a
       // mode with correction terms or bf16 planes (1024^3, plain -> two groups,
-      // us: FP16TCEC NN 19.3 -> 16.4, TN 16.2 -> 14.8, TT 18.6 -> 17.9, bf16x3 NN
+      // us: FP16TCEC NN 19.3 -> 16.4, TN 16.2 -> 13.8, TT 18.6 -> 16.1, bf16x3 NN
       // 28.1 -> 21.5, bf16x2 NN 19.7 -> 16.5; complex FP16TCEC NN 38.6 -> 34.5,
       // bf16x2 38.0 -> 33.5; FP16TC level or slower; op(A) = N with op(B) = T level).
       const uint64_t groups = (uint64_t)grid.x * grid.y * grid.z;

@@ -422,14 +422,14 @@ struct tile_loader {
   static constexpr int NC = CPLX ? 2 : 1;
   static constexpr int ES = CPLX ? 2 : 1;
   static constexpr bool PARTIAL = (ROWS * 4) < NT; // fewer units than threads
-  // A complex operand with half as many units as threads: every thread takes
+  // An operand with half as many units as threads: every thread takes
   // half a unit (4 of its 8 K-values; even threads the lower four, odd threads
   // the upper four, so that a pair of lanes fills one 16-byte chunk of a plane
   // and a wave's 8-byte LDS writes cover all banks), so that all waves have the
   // same work and the K loop no branch around an idle half.
   // (HALF_UNITS: the precisions this pays for, measured -- FP16TCEC and bf16x2; the
   // costlier bf16x3 split and the single-product FP16TC kernels keep whole units)
-  static constexpr bool HALF = HALF_UNITS && CPLX && (ROWS * 4 * 2 == NT);
+  static constexpr bool HALF = HALF_UNITS && (ROWS * 4 * 2 == NT);
   static_assert(TID0 == 0 || (PARTIAL && !HALF), "TID0: partial tiles of whole units");
   static constexpr int KV = HALF ? 4 : 8; // K-values a thread handles per unit
 
@@ -498,9 +498,12 @@ struct tile_loader {
         typedef float f4u_t __attribute__((ext_vector_type(4), aligned(4)));
         const f4u_t *p = reinterpret_cast<const f4u_t *>(reinterpret_cast<const char *>(base) + boff[u]);
         if constexpr (!CPLX) {
-          const f4u_t lo = p[0], hi = p[1];
+          const f4u_t lo = p[0];
           reg.v[u][0][0] = lo.x; reg.v[u][0][1] = lo.y; reg.v[u][0][2] = lo.z; reg.v[u][0][3] = lo.w;
-          reg.v[u][0][4] = hi.x; reg.v[u][0][5] = hi.y; reg.v[u][0][6] = hi.z; reg.v[u][0][7] = hi.w;
+          if constexpr (!HALF) {
+            const f4u_t hi = p[1];
+            reg.v[u][0][4] = hi.x; reg.v[u][0][5] = hi.y; reg.v[u][0][6] = hi.z; reg.v[u][0][7] = hi.w;
+          }
         } else {
 #pragma unroll
           for (int q = 0; q < KV / 2; q++) {
@@ -647,9 +650,12 @@ struct tile_loader {
           typedef float f4u_t __attribute__((ext_vector_type(4), aligned(4)));
           const f4u_t *p = reinterpret_cast<const f4u_t *>(base + ((uint64_t)row * ld + k0) * ES);
           if constexpr (!CPLX) {
-            const f4u_t lo = p[0], hi = p[1];
+            const f4u_t lo = p[0];
             reg.v[u][0][0] = lo.x; reg.v[u][0][1] = lo.y; reg.v[u][0][2] = lo.z; reg.v[u][0][3] = lo.w;
-            reg.v[u][0][4] = hi.x; reg.v[u][0][5] = hi.y; reg.v[u][0][6] = hi.z; reg.v[u][0][7] = hi.w;
+            if constexpr (!HALF) {
+              const f4u_t hi = p[1];
+              reg.v[u][0][4] = hi.x; reg.v[u][0][5] = hi.y; reg.v[u][0][6] = hi.z; reg.v[u][0][7] = hi.w;
+            }
           } else {
 #pragma unroll
             for (int q = 0; q < KV / 2; q++) {
@@ -842,12 +848,17 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
   const uint64_t b_kstep = Cfg::PACKED ? (uint64_t)(NP * NCOMP) * args.ldb * 16
                            : Cfg::B_KC ? (uint64_t)BK * ES : (uint64_t)BK * args.ldb * ES;
 
-  constexpr bool HALF_UNITS = (P == Prec::FP16TCEC || P == Prec::BF16X2);
-  // KS2: the first wave group stages one operand and the second the other,
-  // unless every thread takes half a unit of each.  A row-contiguous operand
-  // (eight 4-byte loads per thread) goes to the first group: measured at
-  // 1024^3, op(A) = T with op(B) = T, 17.9 us that way and 19.7 us the other.
-  constexpr bool HALF_B = HALF_UNITS && CPLX && (BN * 4 * 2 == NT);
+  // (real data: only the two-wave-group kernels have tiles of half as many units
+  // as threads; there it pays when op(A) is K-contiguous -- 1024^3, us, one
+  // operand per group -> half units: op(A) = T 14.8 -> 14.0, with op(B) = T as
+  // well 17.8 -> 16.1, but op(A) = N 16.3 -> 18.0)
+  constexpr bool HALF_UNITS = (P == Prec::FP16TCEC || P == Prec::BF16X2) && (CPLX || Cfg::A_KC);
+  // KS2: every thread takes half a unit of each operand (above), or the first
+  // wave group stages one operand and the second the other.  A row-contiguous
+  // operand (eight 4-byte loads per thread) then goes to the first group:
+  // measured at 1024^3, op(A) = T with op(B) = T, 17.9 us that way and 19.7 us
+  // the other.
+  constexpr bool HALF_B = HALF_UNITS && (BN * 4 * 2 == NT);
   constexpr bool SPLIT_AB = Cfg::KS2 && !HALF_B;
   constexpr bool B_FIRST = Cfg::A_KC && !Cfg::B_KC;
   using LA = tile_loader<CPLX, Cfg::A_KC, BM, Cfg::UA, NT, HALF_UNITS, (SPLIT_AB && B_FIRST) ? BN * 4 : 0>;
