@@ -354,6 +354,60 @@ __device__ inline void block_sync_lds() {
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
+// Immediate of s_waitcnt that waits until at most `n` vector-memory operations
+// of the wave are in flight and leaves the other counters alone.  gfx9 family
+// encoding: vmcnt[3:0] in bits 3:0 and vmcnt[5:4] in bits 15:14; expcnt (bits
+// 6:4) and lgkmcnt (bits 11:8) at their maxima mean "do not wait".
+constexpr int waitcnt_vm(int n) { return (n & 15) | ((n >> 4) << 14) | (7 << 4) | (15 << 8); }
+static_assert(waitcnt_vm(6) == 0x0f76 && waitcnt_vm(63) == 0xcf7f, "s_waitcnt vmcnt immediate");
+
+// The tile-walking pre-split kernel keeps global -> LDS loads in flight across
+// a tile's write-out, and a wave learns that a load has landed only from its
+// vector-memory counter, which counts loads and stores alike and retires them
+// in issue order: "at most n in flight" means everything but the n youngest
+// operations is complete.  Seen from one wave, around a write-out:
+//     L1   the `ndma` loads of the next tile's second K-step   (its last step)
+//     S    the write-out's stores                               (epilogue)
+//     L2   the `ndma` loads of the next tile's third K-step    (its first step)
+//     wait(first), barrier, read the second K-step's planes -> L1 must be complete
+// so the first step's wait is safe iff first <= ndma + S.  This function plays
+// the sequence for two tiles of `nk` steps with S stores between them and
+// reports whether every buffer is complete when its barrier is passed.
+constexpr bool walk_waits_cover(int ndma, int stores, int first, int nk) {
+  // ages[i]: issue number of the loads of step i (two tiles, steps 0 .. 2 nk - 1)
+  int issued = 0;       // operations issued so far
+  int complete = 0;     // operations known complete (a prefix, by the in-order rule)
+  int load_end[64] = {}; // issue count right after the loads of step i
+  if (2 * nk + 2 > 64 || nk < 2) return false;
+  auto issue_loads = [&](int step) {
+    issued += ndma;
+    load_end[step] = issued;
+  };
+  auto wait = [&](int n) {
+    if (issued - n > complete) complete = issued - n;
+  };
+  issue_loads(0);
+  issue_loads(1);
+  wait(0);
+  for (int t = 0; t < 2; t++) {
+    for (int s = 0; s < nk; s++) {
+      const int step = t * nk + s;
+      issue_loads(step + 2);
+      wait(s == 0 && t > 0 ? first : ndma);
+      // barrier; the next step reads the planes of step + 1
+      if (load_end[step + 1] > complete) return false;
+    }
+    issued += stores; // write-out
+  }
+  return true;
+}
+constexpr bool walk_waits_cover_range(int ndma, int stores_lo, int stores_hi, int first) {
+  for (int s = stores_lo; s <= stores_hi; s++)
+    for (int nk = 2; nk <= 6; nk++)
+      if (!walk_waits_cover(ndma, s, first, nk)) return false;
+  return true;
+}
+
 // Map a linear workgroup id to a tile so that (a) workgroups that the
 // dispatcher places on the same XCD (id mod 8) work on neighbouring tiles and
 // share that XCD's L2, (b) tiles are walked in column groups of GROUP tile
@@ -1039,6 +1093,10 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
   // so the 32 lanes of a half-wave write 128 contiguous bytes of a C column.
   // 16x16: MFMA row (-> n) = 4*(l/16) + v, MFMA column (-> m) = l%16.
   // FULL: interior tile, no bounds checks.
+  // Vector-memory operations every wave issues in an unguarded (FULL) write-out,
+  // at least: one store (or atomic, or load + store) per result register; a
+  // complex result is one 8-byte store.  The loops below are tied to it.
+  constexpr int EPI_VMEM = TN * TM * Cfg::NV;
   const bool beta_zero = (args.beta_re == 0.0f) && (!CPLX || args.beta_im == 0.0f);
   const float sgn_a = args.conj_a ? -1.0f : 1.0f, sgn_b = args.conj_b ? -1.0f : 1.0f;
   const float sgn_ab = sgn_a * sgn_b;
@@ -1067,6 +1125,7 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
       return x;
     };
     if constexpr (!CPLX && MT == 16) {
+      static_assert(TN * (TM / 2) * 4 * 2 == EPI_VMEM, "stores of the write-out");
       // Two neighbouring row blocks trade their odd / even 16-lane rows, after
       // which register v of lane l holds column 4*(2*(l/32) + w) + v, row l%32
       // of the block pair (w = 0, 1: the first / second register of the pair):
@@ -1149,9 +1208,13 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
     // ---- persistent walk over pre-split operands with global -> LDS loads -----
     // One workgroup walks its list of tiles; the planes of step t + 2 are asked
     // for before the MFMAs of step t, across tile boundaries.  The first step of
-    // a tile is peeled off the K loop: the stores of the previous tile's
-    // write-out stand between its loads and the next ones in the (in-order)
-    // vector-memory counter, so its wait differs -- as a constant, not a branch.
+    // a tile is peeled off the K loop: the previous tile's write-out stands
+    // between its loads and the next ones in the (in-order) vector-memory
+    // counter, so its wait differs -- as a constant, not a branch inside the loop
+    // (see walk_waits_cover).  After an interior tile, whose write-out issues at
+    // least EPI_VMEM operations in every wave, that many more may stay in flight;
+    // after an edge tile -- guarded stores, none at all from a wave that lies
+    // outside C -- nothing is assumed and the plain count is used.
     const uint32_t total = args.tiles_m * args.tiles_n * args.batch;
     const uint32_t my_tiles = (total - blockIdx.x + gridDim.x - 1) / gridDim.x;
     const int nk = klen / BK;
@@ -1166,7 +1229,11 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
       ct = reinterpret_cast<float *>(args.c);
     };
     constexpr int NDMA = LA::template dma_loads<NP * NCOMP>() + LB::template dma_loads<NP * NCOMP>();
-    constexpr int KEEP = (7 << 4) | (15 << 8);
+    static_assert(NDMA <= 15, "a K-step's loads must leave room in the 6-bit counter");
+    constexpr int WAIT_AFTER_FULL = NDMA + EPI_VMEM > 63 ? 63 : NDMA + EPI_VMEM;
+    static_assert(walk_waits_cover_range(NDMA, EPI_VMEM, 2 * EPI_VMEM, WAIT_AFTER_FULL),
+                  "first-step wait after an interior write-out");
+    static_assert(walk_waits_cover_range(NDMA, 0, 2 * EPI_VMEM, NDMA), "first-step wait after an edge write-out");
     const float *la = a_tile, *lb = b_tile, *la_next, *lb_next;
     float *c_cur = c, *c_ignored;
     uint32_t cm0 = m0, cn0 = n0, i0, i1;
@@ -1192,7 +1259,7 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
       frag_load(f1, b0, 1);
       dma_next(b2);
       frag_mma(f0, f1);
-      __builtin_amdgcn_s_waitcnt(WAIT | KEEP);
+      __builtin_amdgcn_s_waitcnt(waitcnt_vm(WAIT));
       asm volatile("s_barrier" ::: "memory");
       const int tmp = b0;
       b0 = b1;
@@ -1205,14 +1272,15 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
     frag_load(f0, 0, 0);
+    bool after_full = false; // the previous tile was written out by the unguarded epilogue
     for (uint32_t ct = 0; ct < my_tiles; ct++) {
-      // (after a write-out: its 64 stores were issued behind the loads of this
-      // tile's second step, so "at most 63 in flight" covers them)
-      step(std::integral_constant<int, (NDMA + 64 > 63 ? 63 : NDMA + 64)>{});
+      if (after_full) step(std::integral_constant<int, WAIT_AFTER_FULL>{});
+      else step(std::integral_constant<int, NDMA>{});
       for (int kk = 1; kk < nk; kk++) step(std::integral_constant<int, NDMA>{});
       const bool interior = cm0 + BM <= args.m && cn0 + BN <= args.n;
       if (interior) epilogue(c_cur, cm0, cn0, cm0, cn0, std::true_type{});
       else epilogue(c_cur, cm0, cn0, cm0, cn0, std::false_type{});
+      after_full = interior;
       zero_acc();
       const float *ua, *ub;
       tile_at(ct + 1, ua, ub, c_cur, cm0, cn0);
@@ -1428,11 +1496,10 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
     };
     // loads every wave issues per step
     constexpr int NDMA_A = LA::template dma_loads<NP * NCOMP>(), NDMA_B = LB::template dma_loads<NP * NCOMP>();
-    static_assert(NDMA_A + NDMA_B <= 15, "vmcnt immediate");
+    static_assert(NDMA_A + NDMA_B <= 15, "a K-step's loads must leave room in the 6-bit counter");
     auto wait_previous_step = [&]() {
       // at most this step's loads still in flight <=> the previous step's have landed
-      constexpr int KEEP = (7 << 4) | (15 << 8); // leave the other counters alone
-      __builtin_amdgcn_s_waitcnt((NDMA_A + NDMA_B) | KEEP);
+      __builtin_amdgcn_s_waitcnt(waitcnt_vm(NDMA_A + NDMA_B));
     };
     Frags f0, f1;
     dma(0, 0);
