@@ -39,11 +39,6 @@
 #ifndef CUMPSGEMM_MFMA_EDGE_INLOOP
 #define CUMPSGEMM_MFMA_EDGE_INLOOP 32
 #endif
-// Tile-walking pre-split kernel: ask for the next tile's third K-step before
-// the write-out (1) or in that tile's first step, behind the stores (0).
-#ifndef CUMPSGEMM_WALK_EARLY_LOADS
-#define CUMPSGEMM_WALK_EARLY_LOADS 1
-#endif
 
 namespace cumpsgemm_amd {
 
@@ -372,24 +367,19 @@ static_assert(waitcnt_vm(6) == 0x0f76 && waitcnt_vm(63) == 0xcf7f, "s_waitcnt vm
 // in issue order: "at most n in flight" means everything but the n youngest
 // operations is complete.  Seen from one wave, around a write-out (L(i): the
 // `ndma` loads of the next tile's K-step i):
-//     last step of a tile:  L(1), MFMAs, wait, barrier
-//     after the K loop:     L(2)              -- ahead of the stores, so that its
-//                                                data is not queued behind them
+//     last step of a tile:  L(1), MFMAs, wait(ndma), barrier
 //     write-out:            S stores
-//     first step:           MFMAs, wait(w), barrier; step 1 is read next -> L(1) complete?
-//     second step:          L(3), MFMAs, wait(w), barrier; step 2 is read next -> L(2) complete?
-//     third step on:        L(i + 2), MFMAs, wait(ndma), barrier
-// Younger than L(1) at the first wait: L(2) and the stores; younger than L(2)
-// at the second: the stores and L(3).  Both waits are safe iff w <= ndma + S.
-// (`early` false: L(2) is issued in the first step instead, and only that
-// step's wait differs from ndma.)  This function plays the sequence for three
+//     first step:           L(2), MFMAs, wait(w), barrier; step 1 is read next -> L(1) complete?
+//     second step on:       L(i + 2), MFMAs, wait(ndma), barrier
+// Younger than L(1) at the first step's wait: the stores and L(2), so that
+// wait is safe iff w <= ndma + S.  This function plays the sequence for three
 // tiles of `nk` steps with S stores after each and reports whether every
 // buffer is complete when the barrier before its first read is passed.
-constexpr bool walk_waits_cover(int ndma, int stores, int w, int nk, bool early) {
+constexpr bool walk_waits_cover(int ndma, int stores, int w, int nk) {
   int issued = 0;        // operations issued so far
   int complete = 0;      // operations known complete (a prefix, by the in-order rule)
   int load_end[64] = {}; // issue count right after the loads of step i
-  if (3 * nk + 3 > 64 || nk < 3) return false;
+  if (3 * nk + 2 > 64 || nk < 2) return false;
   auto issue_loads = [&](int step) {
     issued += ndma;
     load_end[step] = issued;
@@ -399,32 +389,28 @@ constexpr bool walk_waits_cover(int ndma, int stores, int w, int nk, bool early)
   };
   issue_loads(0);
   issue_loads(1);
-  if (early) issue_loads(2);
   wait(0);
   for (int t = 0; t < 3; t++) {
     for (int s = 0; s < nk; s++) {
       const int step = t * nk + s;
-      if (!(early && s == 0)) issue_loads(step + 2);
-      const bool after_writeout = t > 0 && (s == 0 || (early && s == 1));
-      wait(after_writeout ? w : ndma);
+      issue_loads(step + 2);
+      wait(t > 0 && s == 0 ? w : ndma);
       // barrier; the next step reads the planes of step + 1
       if (load_end[step + 1] > complete) return false;
     }
-    if (early) issue_loads((t + 1) * nk + 2);
     issued += stores; // write-out
   }
   return true;
 }
-constexpr bool walk_waits_cover_range(int ndma, int stores_lo, int stores_hi, int w, bool early) {
+constexpr bool walk_waits_cover_range(int ndma, int stores_lo, int stores_hi, int w) {
   for (int s = stores_lo; s <= stores_hi; s++)
-    for (int nk = 3; nk <= 6; nk++)
-      if (!walk_waits_cover(ndma, s, w, nk, early)) return false;
+    for (int nk = 2; nk <= 6; nk++)
+      if (!walk_waits_cover(ndma, s, w, nk)) return false;
   return true;
 }
 // (the model itself: one store fewer than the wait allows for must fail it)
-static_assert(walk_waits_cover_range(6, 57, 128, 63, true) && !walk_waits_cover(6, 56, 63, 4, true) &&
-                  walk_waits_cover_range(6, 57, 128, 63, false) && !walk_waits_cover(6, 56, 63, 4, false) &&
-                  walk_waits_cover_range(6, 0, 64, 6, true) && !walk_waits_cover(6, 0, 7, 4, true),
+static_assert(walk_waits_cover_range(6, 57, 128, 63) && !walk_waits_cover(6, 56, 63, 4) &&
+                  walk_waits_cover_range(6, 0, 64, 6) && !walk_waits_cover(6, 0, 7, 4),
               "model of the in-order vector-memory counter");
 
 // Map a linear workgroup id to a tile so that (a) workgroups that the
@@ -1249,11 +1235,10 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
     };
     constexpr int NDMA = LA::template dma_loads<NP * NCOMP>() + LB::template dma_loads<NP * NCOMP>();
     static_assert(NDMA <= 15, "a K-step's loads must leave room in the 6-bit counter");
-    constexpr bool EARLY = CUMPSGEMM_WALK_EARLY_LOADS != 0;
     constexpr int WAIT_AFTER_FULL = NDMA + EPI_VMEM > 63 ? 63 : NDMA + EPI_VMEM;
-    static_assert(walk_waits_cover_range(NDMA, EPI_VMEM, 2 * EPI_VMEM, WAIT_AFTER_FULL, EARLY),
-                  "waits after an interior write-out");
-    static_assert(walk_waits_cover_range(NDMA, 0, 2 * EPI_VMEM, NDMA, EARLY), "waits after an edge write-out");
+    static_assert(walk_waits_cover_range(NDMA, EPI_VMEM, 2 * EPI_VMEM, WAIT_AFTER_FULL),
+                  "first-step wait after an interior write-out");
+    static_assert(walk_waits_cover_range(NDMA, 0, 2 * EPI_VMEM, NDMA), "first-step wait after an edge write-out");
     const float *la = a_tile, *lb = b_tile, *la_next, *lb_next;
     float *c_cur = c, *c_ignored;
     uint32_t cm0 = m0, cn0 = n0, i0, i1;
@@ -1273,14 +1258,13 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
     Frags f0, f1;
     int b0 = 0, b1 = 1, b2 = 2;
     bool after_full = false; // the previous tile was written out by the unguarded epilogue
-    // one K-step.  LOAD: whether it asks for the planes of the step after next.
-    // AFTER_WRITEOUT: whether stores of the previous tile's write-out may stand
-    // between the loads it waits for and younger ones -- then the number of
+    // one K-step.  AFTER_WRITEOUT: the stores of the previous tile's write-out
+    // stand between the loads it waits for and this step's own, so the number of
     // operations that may stay in flight depends on which epilogue ran (one
     // scalar branch around the wait, outside the K loop proper).
-    auto step = [&](auto after_writeout_tag, auto load_tag) {
+    auto step = [&](auto after_writeout_tag) {
       frag_load(f1, b0, 1);
-      if constexpr (decltype(load_tag)::value) dma_next(b2);
+      dma_next(b2);
       frag_mma(f0, f1);
       if constexpr (decltype(after_writeout_tag)::value) {
         if (after_full) __builtin_amdgcn_s_waitcnt(waitcnt_vm(WAIT_AFTER_FULL));
@@ -1297,23 +1281,12 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
     };
     dma_next(0);
     dma_next(1);
-    if constexpr (EARLY) dma_next(2);
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
     frag_load(f0, 0, 0);
     for (uint32_t ct = 0; ct < my_tiles; ct++) {
-      if constexpr (EARLY) {
-        step(std::true_type{}, std::false_type{});
-        step(std::true_type{}, std::true_type{});
-        for (int kk = 2; kk < nk; kk++) step(std::false_type{}, std::true_type{});
-        // the loader moves on to the tile after the next one while it is asked
-        // for that tile's third step: its origin must be known by now
-        tile_at(ct + 2, la_next, lb_next, c_ignored, i0, i1);
-        dma_next(b2); // (the buffer read in the last step, free since its barrier)
-      } else {
-        step(std::true_type{}, std::true_type{});
-        for (int kk = 1; kk < nk; kk++) step(std::false_type{}, std::true_type{});
-      }
+      step(std::true_type{});
+      for (int kk = 1; kk < nk; kk++) step(std::false_type{});
       const bool interior = cm0 + BM <= args.m && cn0 + BN <= args.n;
       if (interior) epilogue(c_cur, cm0, cn0, cm0, cn0, std::true_type{});
       else epilogue(c_cur, cm0, cn0, cm0, cn0, std::false_type{});
@@ -1321,7 +1294,7 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
       zero_acc();
       const float *ua, *ub;
       tile_at(ct + 1, ua, ub, c_cur, cm0, cn0);
-      if constexpr (!EARLY) tile_at(ct + 2, la_next, lb_next, c_ignored, i0, i1);
+      tile_at(ct + 2, la_next, lb_next, c_ignored, i0, i1);
     }
     __builtin_amdgcn_s_waitcnt(0);
     return;
