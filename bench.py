@@ -39,6 +39,16 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
+def host_cores():
+    """Threads of the host-core legs: the share of the host this job was given (OMP_NUM_THREADS when the
+    environment sets it -- a GPU box hands a one-GPU job part of its cores --, else every core)."""
+    env = int(os.environ.get("OMP_NUM_THREADS", "0") or 0)
+    if env > 0:
+        return env, f"{env} threads = OMP_NUM_THREADS as set by the environment, of {os.cpu_count()} cores visible"
+    n = os.cpu_count() or 1
+    return n, f"all {n} cores"
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -53,9 +63,6 @@ def main():
     ap.add_argument("--kernel", default="gemm", choices=["gemm", "copy", "exp_stats", "exp_max", "scale", "mx2x2"],
                     help="with --kernel-only: which kernel to run (copy = a plain device copy of the "
                          "same bytes, the reference point for the HBM traffic counters)")
-    ap.add_argument("--tile-sweep", action="store_true",
-                    help="time every tile class of the table for each layout over a list of shapes (split in the "
-                         "K loop, no workspace) next to the planner's own choice; prints a table")
     ap.add_argument("--shape", default=None,
                     help="with --kernel-only: M,N,K[,BATCH] instead of a square --size (BATCH > 1: strided batch)")
     ap.add_argument("--cplx", action="store_true", help="with --kernel-only --shape: complex64 operands (CGEMM)")
@@ -82,10 +89,6 @@ def main():
 
     n = args.size
     m = k = n
-    if args.tile_sweep:
-        tile_sweep(args, torch, cg, h, dev, stream)
-        h.close()
-        return
     if args.kernel_only and args.kernel != "gemm":
         hbm_kernel_only(args, torch, cg, inputs, h, dev, stream)
         h.close()
@@ -209,7 +212,7 @@ def main():
         log("[bench] CPU baseline (oracle)")
         from oracle import oracle as O
         O.lib()
-        cores = int(os.environ.get("OMP_NUM_THREADS", "0")) or min(os.cpu_count() or 1, 16)
+        cores, cores_why = host_cores()
         os.environ["OMP_NUM_THREADS"] = str(cores)
 
         def cpu_run(cn):
@@ -229,7 +232,7 @@ def main():
         frac = "the whole" if cn == n else f"1/{(n // cn) ** 3} of the"
         cpu = {"value": round(2.0 * cn ** 3 / dt / 1e12, 5), "unit": "TFLOP/s", "cores": cores, "kind": "port",
                "sample": f"one FP16TCEC SGEMM NN {cn}^3 (same generator, seeds 1,2) = {frac} "
-                         f"{n}^3 step, split included, {dt:.1f} s"}
+                         f"{n}^3 step, split included, {dt:.1f} s; {cores_why}"}
 
     out = {
         "metric": "effective FP32 TFLOP/s (2MNK/t) at 8192^3 FP16TCEC + rel. error vs FP64",
@@ -254,101 +257,16 @@ def main():
         "error_ratio_vs_sgemm": (err_tcec / err_sgemm) if err_sgemm else None,
         "hipblas_sgemm_tflops": round(hb_tflops, 2) if hb_tflops else None,
         "speedup_vs_hipblas_sgemm": round(value / hb_tflops, 3) if hb_tflops else None,
-        "roofline": {
-            "bound": "mfma",
-            # algorithmic flops 2MNK of one launch over the kernel's average
-            # duration between HIP events on the launch stream
-            "achieved": round(kernel_tflops, 2),
-            "peak": FP16_MFMA_PEAK_TFLOPS,
-            "unit": "TFLOP/s",
-            "frac": round(kernel_tflops / FP16_MFMA_PEAK_TFLOPS, 4),
-            "traffic": GEMM_TRAFFIC_BYTES if n == 8192 else None,
-            "traffic_source": "constant from the committed rocprofv3 counter runs "
-                              "(profiles/gemm_fp16tcec_8192_nn.md), not measured in this run",
-            # one call = two pre-split passes (about 0.2 ms) + the GEMM kernel: all inside
-            "kernel_ms": round(ev_ms, 4),
-            "kernels_per_step": "pack_split_pair_kernel + gemm_tcec_kernel (persistent, packed)" if module_id == 200 else
-                                "gemm_tcec_kernel",
-            # the split-and-correct algorithm issues 3 MFMA products per logical product
-            "mfma_products_per_flop": 3,
-            "mfma_issued_tflops": round(3.0 * kernel_tflops, 1),
-            "frac_of_emulation_peak": round(3.0 * kernel_tflops / FP16_MFMA_PEAK_TFLOPS, 4),
-        },
+        # frac = the fraction of the emulation roofline (fp16 MFMA peak / products): `achieved` is the fp16 MFMA
+        # work the kernel issues -- 3 products per real multiply-add of the algorithm, i.e. 3 x the algorithmic
+        # 2MNK flops of one launch -- over the launch's average duration between HIP events on its stream
+        "roofline": headline_roofline(flops, ev_ms, module_id, n),
         "cpu_baseline": cpu,
     }
     if extra:
         out["extra"] = extra
     print(json.dumps(out), flush=True)
     h.close()
-
-
-def tile_sweep(args, torch, cg, h, dev, stream):
-    """Effective TFLOP/s of each tile class (CUMPSGEMM_FORCE_TILE_CLASS, 0 - 4) for the four layouts, with the
-    split in the K loop (CUMPSGEMM_PACKED=0), then what the planner picks on its own (same restriction)
-    and the default path (pre-split operands where the rules allow: module id 200)."""
-    L = cg.lib()
-    mode = getattr(cg, args.mode)
-
-    def setenv(**kw):
-        for key in ("CUMPSGEMM_PACKED", "CUMPSGEMM_FORCE_TILE_CLASS"):
-            os.environ.pop(key, None)
-        for key, v in kw.items():
-            os.environ["CUMPSGEMM_" + key] = v
-        L.cuMpSGEMM_reload_tuning_env()
-
-    def bench(fn, steps=6, warm=2):
-        best = None
-        for _ in range(2):
-            for _ in range(warm):
-                fn()
-            torch.cuda.synchronize()
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record(stream)
-            for _ in range(steps):
-                fn()
-            e1.record(stream)
-            torch.cuda.synchronize()
-            t = e0.elapsed_time(e1) / steps
-            best = t if best is None else min(best, t)
-        return best
-
-    squares = [512, 768, 1024, 1280, 1536, 1792, 2048, 2560, 3072, 3584, 4096, 5120, 6144, 8192]
-    shapes = [(s, s, s) for s in squares] + [(4096, 4096, 1024), (8192, 8192, 1024), (2048, 8192, 2048),
-                                             (8192, 2048, 2048), (16384, 16384, 256), (1024, 1024, 8192),
-                                             (4096, 1024, 4096),
-                                             # C with a few columns / rows: classes 3 and 4 (memory-bound: the
-                                             # vendor FP32 routine is the yardstick)
-                                             (8192, 8, 8192), (8192, 32, 8192), (8, 8192, 8192), (32, 8192, 8192),
-                                             (65536, 16, 1024), (16384, 4, 16384), (8192, 1, 8192)]
-    ncls = 5
-    print("| shape | layout | " + " | ".join(f"class {c}" for c in range(ncls)) +
-          " | best | planner, in-loop | default path (module id) | vendor FP32 |")
-    print("|---|---|" + "---|" * (ncls + 4))
-    for (m, n, k) in shapes:
-        a = torch.rand(m * k, device=dev) * 2 - 1
-        b = torch.rand(k * n, device=dev) * 2 - 1
-        c = torch.zeros(m * n, device=dev)
-        for lay, opa, opb, lda, ldb in (("NN", 111, 111, m, k), ("TN", 112, 111, k, k), ("NT", 111, 112, m, n),
-                                        ("TT", 112, 112, k, n)):
-            fn = lambda: h.gemm(opa, opb, m, n, k, 1.0, a, lda, b, ldb, 0.0, c, m, mode)
-            gf = 2.0 * m * n * k / 1e9
-            tf = []
-            for cl in range(ncls):
-                setenv(PACKED="0", FORCE_TILE_CLASS=str(cl))
-                tf.append(gf / bench(fn))
-            setenv(PACKED="0")
-            auto = gf / bench(fn)
-            setenv()
-            dflt = gf / bench(fn)
-            _, mid = h.gemm(opa, opb, m, n, k, 1.0, a, lda, b, ldb, 0.0, c, m, mode, want_module_id=True)
-            am = a.view(k, m).t() if opa == 111 else a.view(m, k)      # logical m x k over the same memory
-            bm = b.view(n, k).t() if opb == 111 else b.view(k, n)
-            vend = gf / bench(lambda: torch.matmul(am, bm))
-            print(f"| {m}x{n}x{k} | {lay} | " + " | ".join(f"{x:.1f}" if x < 10 else f"{x:.0f}" for x in tf) +
-                  f" | {max(range(ncls), key=lambda i: tf[i])} | {auto:.1f} | {dflt:.1f} ({mid}) | {vend:.1f} |",
-                  flush=True)
-        del a, b, c
-    setenv()
 
 
 def shape_kernel_only(args, torch, cg, h, dev, stream):
@@ -442,14 +360,27 @@ def hbm_kernel_only(args, torch, cg, inputs, h, dev, stream):
 
 
 def mfma_roofline(flops, ev_ms, products, kernels):
-    """Roofline entry of an MFMA-bound configuration: algorithmic flops of one call over its
-    duration between HIP events on the launch stream, against the dense fp16 / bf16 MFMA peak;
-    `products` MFMA products are issued per real multiply-add of the algorithm."""
-    t = flops / (ev_ms * 1e-3) / 1e12
-    return {"bound": "mfma", "achieved": round(t, 2), "peak": FP16_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
-            "frac": round(t / FP16_MFMA_PEAK_TFLOPS, 4), "kernel_ms": round(ev_ms, 4),
-            "mfma_products_per_real_mac": products,
-            "frac_of_emulation_peak": round(products * t / FP16_MFMA_PEAK_TFLOPS, 4), "kernels": kernels}
+    """Roofline entry of an MFMA-bound configuration.  `flops`: algorithmic flops of one call (2MNK, 8MNK
+    complex); `ev_ms`: its duration between HIP events on the launch stream; `products`: MFMA products issued
+    per real multiply-add of the algorithm.  achieved = products x flops / t, the fp16 / bf16 MFMA work
+    issued, against the dense MFMA peak -- so frac is the fraction of the emulation roofline (peak / products)."""
+    eff = flops / (ev_ms * 1e-3) / 1e12
+    return {"bound": "mfma", "achieved": round(products * eff, 2), "peak": FP16_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+            "frac": round(products * eff / FP16_MFMA_PEAK_TFLOPS, 4), "kernel_ms": round(ev_ms, 4),
+            "mfma_products_per_real_mac": products, "effective_tflops": round(eff, 2),
+            "emulation_roofline_tflops": round(FP16_MFMA_PEAK_TFLOPS / products, 1),
+            "effective_over_raw_peak": round(eff / FP16_MFMA_PEAK_TFLOPS, 4), "kernels": kernels}
+
+
+def headline_roofline(flops, ev_ms, module_id, n):
+    r = mfma_roofline(flops, ev_ms, 3,
+                      "pack_split_pair_kernel + gemm_tcec_kernel (persistent, packed)" if module_id == 200
+                      else "gemm_tcec_kernel")
+    # one call = one pre-split launch for both operands (about 0.2 ms) + the GEMM kernel: all inside kernel_ms
+    r["traffic"] = GEMM_TRAFFIC_BYTES if n == 8192 else None
+    r["traffic_source"] = ("constant from the committed rocprofv3 counter runs (profiles/gemm_fp16tcec_8192_nn.md), "
+                           "not measured in this run")
+    return r
 
 
 def hbm_roofline(nbytes, ev_ms, kernels):
@@ -471,7 +402,7 @@ def full_suite(torch, cg, inputs, h, dev, stream, timed, log, a, b, c, with_cpu)
     if with_cpu:
         from oracle import oracle as O
         O.lib()
-        cores = int(os.environ.get("OMP_NUM_THREADS", "0")) or min(os.cpu_count() or 1, 16)
+        cores, _ = host_cores()
         s1 = 1024
         ca, cb = inputs.uniform(1, s1 * s1), inputs.uniform(2, s1 * s1)
         cc, c32 = np.zeros(s1 * s1, np.float32), np.zeros(s1 * s1, np.float32)
@@ -567,6 +498,9 @@ def full_suite(torch, cg, inputs, h, dev, stream, timed, log, a, b, c, with_cpu)
     err_fp32 = rel_err((a4.view(n, n).t() @ b4.view(n, n).t()).double(), ref)
     st_ms = timed(lambda: h.exp_stats_ext(n, n, a4, n), 20, 3)[1]
     mx_ms = timed(lambda: h.exp_max_ext(n, n, a4, n), 20, 3)[1]
+    # what the pipelines launch: A and B scanned by one launch per pass
+    stp_ms = timed(lambda: h.exp_stats_pair(n, n, a4, n, n, n, b4, n), 20, 3)[1]
+    mxp_ms = timed(lambda: h.exp_max_pair(n, n, a4, n, n, n, b4, n), 20, 3)[1]
     sid = h.exp_max_ext(n, n, a4, n)
     sc_ms = timed(lambda: (h.scale_A(sid, 1, n, n, a4, n), h.reset_scale_A(sid, 1, n, n, a4, n)), 20, 3)[1] / 2
     nbytes = 4.0 * n * n
@@ -580,6 +514,9 @@ def full_suite(torch, cg, inputs, h, dev, stream, timed, log, a, b, c, with_cpu)
         # two passes (stage 1 + stage 2) over one 64 MiB matrix / one pass / read + write
         "roofline_exp_stats": hbm_roofline(2 * nbytes, st_ms, "exp_stats_kernel<0> + exp_stats_kernel<1>"),
         "roofline_exp_max": hbm_roofline(nbytes, mx_ms, "exp_stats_kernel<2>"),
+        # A and B (2 x 64 MiB) in one launch per pass, as the FP16TCEC_SCALING / AUTO pipelines scan them
+        "roofline_exp_stats_pair": hbm_roofline(4 * nbytes, stp_ms, "exp_stats_kernel<0> + exp_stats_kernel<1>, A and B per launch"),
+        "roofline_exp_max_pair": hbm_roofline(2 * nbytes, mxp_ms, "exp_stats_kernel<2>, A and B in one launch"),
         "roofline_scaling": hbm_roofline(2 * nbytes, sc_ms, "scaling_kernel")}
     del a4, b4, c4, ref
     torch.cuda.empty_cache()

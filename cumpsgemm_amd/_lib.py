@@ -107,6 +107,11 @@ def _declare(L):
                  "cuMpSGEMM_exp_max_ext_s", "cuMpSGEMM_exp_max_ext_c"):
         getattr(L, name).argtypes = stats_args
         getattr(L, name).restype = _u32
+    L.cuMpSGEMM_exp_stats_pair_s.argtypes = [_ptr, _u32, _u32, _ptr, _u32, _u32, _u32, _ptr, _u32, _int,
+                                             ctypes.POINTER(_u32)]
+    L.cuMpSGEMM_exp_stats_pair_s.restype = None
+    L.cuMpSGEMM_exp_max_pair_s.argtypes = [_ptr, _u32, _u32, _ptr, _u32, _u32, _u32, _ptr, _u32, ctypes.POINTER(_u32)]
+    L.cuMpSGEMM_exp_max_pair_s.restype = None
     L.cuMpSGEMM_get_exp_stats.argtypes = [_ptr, _u32, ctypes.POINTER(_u64), ctypes.POINTER(_u64)]
     L.cuMpSGEMM_get_exp_stats.restype = None
     L.cuMpSGEMM_get_max_exp.argtypes = [_ptr, _u32]
@@ -269,6 +274,18 @@ class Handle:
     def exp_max_ext(self, m, n, ptr, ld, batch=1, stride=0, cplx=False):
         fn = self._L.cuMpSGEMM_exp_max_ext_c if cplx else self._L.cuMpSGEMM_exp_max_ext_s
         return fn(self._h, m, n, _dptr(ptr), ld, batch, stride)
+
+    def exp_stats_pair(self, m_a, n_a, a, lda, m_b, n_b, b, ldb, flag_id=-1):
+        """Full statistics of A and B with one launch per pass; returns their two slots."""
+        ids = (_u32 * 2)()
+        self._L.cuMpSGEMM_exp_stats_pair_s(self._h, m_a, n_a, _dptr(a), lda, m_b, n_b, _dptr(b), ldb, flag_id, ids)
+        return ids[0], ids[1]
+
+    def exp_max_pair(self, m_a, n_a, a, lda, m_b, n_b, b, ldb):
+        """Maximum exponents of A and B with one launch; returns their two slots."""
+        ids = (_u32 * 2)()
+        self._L.cuMpSGEMM_exp_max_pair_s(self._h, m_a, n_a, _dptr(a), lda, m_b, n_b, _dptr(b), ldb, ids)
+        return ids[0], ids[1]
 
     def get_exp_stats(self, buffer_id):
         """(underflow, total) like cumpsgemm::get_exp_stats."""

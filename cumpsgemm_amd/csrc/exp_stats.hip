@@ -585,6 +585,28 @@ unsigned cuMpSGEMM_exp_max_ext_c(cuMpSGEMM_handle_t h, unsigned m, unsigned n,
                                  unsigned stride) {
   return cumpsgemm::exp_max_ext<hipComplex>(h, m, n, ptr, ld, batch, stride);
 }
+void cuMpSGEMM_exp_stats_pair_s(cuMpSGEMM_handle_t h, unsigned m_a, unsigned n_a, const float *a,
+                                unsigned lda, unsigned m_b, unsigned n_b, const float *b,
+                                unsigned ldb, int flag_id, unsigned *ids_out) {
+  unsigned ia = 0, ib = 0;
+  exp_stats_pair<float>(h, MatrixView<float>{a, m_a, n_a, lda, 1u, 0u}, MatrixView<float>{b, m_b, n_b, ldb, 1u, 0u},
+                        ia, ib, flag_id);
+  if (ids_out != nullptr) {
+    ids_out[0] = ia;
+    ids_out[1] = ib;
+  }
+}
+void cuMpSGEMM_exp_max_pair_s(cuMpSGEMM_handle_t h, unsigned m_a, unsigned n_a, const float *a,
+                              unsigned lda, unsigned m_b, unsigned n_b, const float *b,
+                              unsigned ldb, unsigned *ids_out) {
+  unsigned ia = 0, ib = 0;
+  exp_max_pair<float>(h, MatrixView<float>{a, m_a, n_a, lda, 1u, 0u}, MatrixView<float>{b, m_b, n_b, ldb, 1u, 0u},
+                      ia, ib);
+  if (ids_out != nullptr) {
+    ids_out[0] = ia;
+    ids_out[1] = ib;
+  }
+}
 // The read-backs synchronise the stream and the C++ forms throw when HIP
 // reports an error; no exception may cross the C boundary, so the C forms log
 // (check_hip already has) and return zeros / UNDEFINED instead.

@@ -36,8 +36,12 @@ Tuning read_tuning_env() {
   if (const char *v = std::getenv("CUMPSGEMM_MAX_WORKSPACE_BYTES")) t.max_workspace_bytes = std::strtoull(v, nullptr, 10);
   return t;
 }
-Tuning g_tuning;
-std::once_flag g_tuning_once;
+// The current snapshot of the tuning variables.  A reload publishes a new,
+// immutable object and leaves the old one in place (never freed: a few dozen
+// bytes per reload, and reloads are a test facility), so a thread that took a
+// reference before the reload keeps reading a consistent set of values.
+std::atomic<const Tuning *> g_tuning{nullptr};
+std::mutex g_tuning_mutex;
 } // namespace
 
 // ---- home of the pre-split planes for the entry point that allocates nothing
@@ -78,8 +82,16 @@ void *scratch_address(int dev) {
 } // namespace
 
 const Tuning &tuning() {
-  std::call_once(g_tuning_once, [] { g_tuning = read_tuning_env(); });
-  return g_tuning;
+  const Tuning *t = g_tuning.load(std::memory_order_acquire);
+  if (t == nullptr) {
+    std::lock_guard<std::mutex> lock(g_tuning_mutex);
+    t = g_tuning.load(std::memory_order_acquire);
+    if (t == nullptr) {
+      t = new Tuning(read_tuning_env());
+      g_tuning.store(t, std::memory_order_release);
+    }
+  }
+  return *t;
 }
 
 void check_hip(hipError_t err, const char *what) {
@@ -417,7 +429,9 @@ PreSplitChoice choose_pre_split(const cuMpSGEMM_handle *h, bool a_kc, bool b_kc,
     return ch.bf16 ? (pays_bf16 || always) : (ch.tc_only ? (pays_tc || always) : (pays || pays_scaled || always));
   };
   const bool mode_ok = mode == CUMPSGEMM_FP16TCEC || ch.bf16 || ch.auto_ok || ch.tc_only;
-  const bool base_ok = mode_ok && !never && shape_ok && force_cls <= 0 && force_split <= 1;
+  // (CUMPSGEMM_FORCE_TILE_CLASS / _FORCE_KSPLIT pick among the in-loop kernels and keep a call off this
+  // path -- except a call of the entry point that allocates nothing, which is defined to take it)
+  const bool base_ok = mode_ok && !never && shape_ok && (forced || (force_cls <= 0 && force_split <= 1));
   ch.take = base_ok && worth_if(rounds_ok);
   // With a mostly empty last round the path still pays for the rounds before
   // it: the caller cuts C there (6000^2 x 2048: 332 TFLOP/s in-loop, 384 with
@@ -1119,8 +1133,8 @@ const void *cuMpSGEMM_get_workspace_pointer(cuMpSGEMM_handle_t handle) {
   return handle != nullptr ? handle->pack_ws : nullptr;
 }
 void cuMpSGEMM_reload_tuning_env(void) {
-  (void)tuning();
-  g_tuning = read_tuning_env();
+  std::lock_guard<std::mutex> lock(g_tuning_mutex);
+  g_tuning.store(new Tuning(read_tuning_env()), std::memory_order_release);
 }
 
 int cuMpSGEMM_describe_tile_config(int compute_mode, int is_complex, int op_A, int op_B,

@@ -27,6 +27,13 @@ hipblasStatus_t gemm_pipeline(cuMpSGEMM_handle_t h, hipblasOperation_t op_A,
     log_error("FP16TCEC_SCALING / AUTO: a size, leading dimension or stride does not fit 32 bits");
     return HIPBLAS_STATUS_INVALID_VALUE;
   }
+  // A null matrix would make the statistics pass skip its launch (nothing to
+  // scan) and leave the slots and the launch flag that everything after it
+  // reads with whatever the ring held before: refuse the call before any launch.
+  if (needs_stats && m != 0 && n != 0 && batch != 0 && (c == nullptr || (k != 0 && (a == nullptr || b == nullptr)))) {
+    log_error("FP16TCEC_SCALING / AUTO: null matrix pointer");
+    return HIPBLAS_STATUS_INVALID_VALUE;
+  }
   // stored shapes of A and B (rows x cols as laid out in memory)
   const unsigned a_rows = (unsigned)(op_A == HIPBLAS_OP_N ? m : k);
   const unsigned a_cols = (unsigned)(op_A == HIPBLAS_OP_N ? k : m);
@@ -54,7 +61,17 @@ hipblasStatus_t gemm_pipeline(cuMpSGEMM_handle_t h, hipblasOperation_t op_A,
   // GEMM-with-beta, then scale_C over all of C also rescales beta*C_old,
   // src/cumpsgemm_cublas.cu:549-559; the stand-alone form here divides C_old
   // by that power of two first, which the final scale_C undoes exactly.)
-  const bool fused = scaled && restore_AB && !tuning().no_fused_scaling;
+  bool beta_nonzero;
+  if constexpr (std::is_same<T, hipComplex>::value) beta_nonzero = beta != nullptr && (beta->x != 0.0f || beta->y != 0.0f);
+  else beta_nonzero = beta != nullptr && *beta != 0.0f;
+  // restore_AB == false with beta != 0: the stand-alone sequence would have to
+  // divide C_old by the product of the two scaling factors before the GEMM
+  // (so that the final pass over C, which multiplies everything by it, leaves
+  // beta * C_old alone), and that quotient can leave the FP32 range (factors
+  // down to 2^-88 for operands near 2^-30).  The fused GEMM has no such
+  // intermediate; A and B are scaled in place afterwards, as the caller asked.
+  const bool scale_ab_after = scaled && !restore_AB && beta_nonzero && !tuning().no_fused_scaling;
+  const bool fused = scaled && (restore_AB || scale_ab_after) && !tuning().no_fused_scaling;
   if (mode == CUMPSGEMM_AUTO) {
     // (the second statistics pass also writes the launch flag: the reference's
     // set_dynamic_launch_buffer_by_exp_stats, src/cumpsgemm_cublas.cu:463-466,
@@ -75,9 +92,7 @@ hipblasStatus_t gemm_pipeline(cuMpSGEMM_handle_t h, hipblasOperation_t op_A,
     }
   }
   if (scaled && !fused) {
-    bool beta_nonzero;
-    if constexpr (std::is_same<T, hipComplex>::value) beta_nonzero = beta != nullptr && (beta->x != 0.0f || beta->y != 0.0f);
-    else beta_nonzero = beta != nullptr && *beta != 0.0f;
+    // (only with CUMPSGEMM_NO_FUSED_SCALING: C_old / factor must stay inside the FP32 range)
     if (beta_nonzero)
       unscale_C<T>(h, a_id, b_id, flag_id, (unsigned)m, (unsigned)n, c, (unsigned)ldc, sb, sc_stride);
   }
@@ -98,6 +113,10 @@ hipblasStatus_t gemm_pipeline(cuMpSGEMM_handle_t h, hipblasOperation_t op_A,
                             gemm_mode);
   }
   h->fused_scaling = false;
+  if (scale_ab_after) {
+    cumpsgemm::scale_A<T>(h, a_id, flag_id, a_rows, a_cols, a, (unsigned)lda, sb, sa_stride);
+    cumpsgemm::scale_B<T>(h, b_id, flag_id, b_rows, b_cols, b, (unsigned)ldb, sb, sb_stride);
+  }
   if (scaled && !fused) {
     cumpsgemm::scale_C<T>(h, a_id, b_id, flag_id, (unsigned)m, (unsigned)n, c, (unsigned)ldc, sb,
                           sc_stride);

@@ -36,6 +36,9 @@ hipblasStatus_t cuMpSGEMM_cgemm_ex(cuMpSGEMM_handle_t handle, hipblasOperation_t
  * takes the pre-split path and keeps the fp16 / bf16 planes of A and B in a
  * static device array inside the library instead of the handle's grow-on-demand
  * workspace: it calls no hipMalloc / hipFree and does not synchronise.
+ * (The variables that steer cuMpSGEMM_sgemm away from that path --
+ * CUMPSGEMM_PACKED=0, CUMPSGEMM_FORCE_TILE_CLASS, CUMPSGEMM_FORCE_KSPLIT -- do
+ * not apply to this call.)
  * Limits: k >= 128 and
  *   (roundup(m, 256) + roundup(n, 256)) * roundup(k, 32) * 4 bytes (6 for
  *   TF32TCEC) <= cuMpSGEMM_get_static_scratch_size() (64 MiB);
@@ -70,10 +73,13 @@ const void *cuMpSGEMM_get_workspace_pointer(cuMpSGEMM_handle_t handle);
 
 /* The tuning variables of the GEMM path (CUMPSGEMM_PACKED, _PACKED_WALK,
  * _RASTER_GROUP, _FORCE_TILE_CLASS, _FORCE_KSPLIT, _NO_PERSISTENT,
- * _NO_COLUMN_SPLIT, _NO_FUSED_SCALING, _PERSISTENT_MAX_STEPS,
- * _MAX_WORKSPACE_BYTES) are read from the environment once per process; this
- * reads them again.  For tests and experiments: not to be called while another
- * thread is inside a GEMM call.  The reference has no such variables. */
+ * _NO_COLUMN_SPLIT, _NO_KSLICE_GROUPS, _NO_FUSED_SCALING,
+ * _PERSISTENT_MAX_STEPS, _MAX_WORKSPACE_BYTES) are read from the environment
+ * once per process; this reads them again and publishes the new set as one
+ * immutable snapshot.  Safe to call while other threads run GEMMs: a call in
+ * flight goes on with the values it has already looked up and may take later
+ * ones from the new set.  For tests and experiments.  The reference has no
+ * such variables. */
 void cuMpSGEMM_reload_tuning_env(void);
 
 /* The whole mode pipeline of an intercepted call, callable directly:
@@ -142,6 +148,22 @@ unsigned cuMpSGEMM_exp_max_ext_s(cuMpSGEMM_handle_t h, unsigned m, unsigned n, c
 unsigned cuMpSGEMM_exp_max_ext_c(cuMpSGEMM_handle_t h, unsigned m, unsigned n,
                                  const hipComplex *ptr, unsigned ld, unsigned batch,
                                  unsigned stride);
+/* The statistics of the two operands of one GEMM with ONE launch per pass
+ * (the workgroups are shared out between A and B in proportion to their
+ * sizes) -- what the FP16TCEC_SCALING and AUTO pipelines use, a kernel
+ * boundary being worth several microseconds.  Same results and slot numbering
+ * as the _ext call for A followed by the one for B; ids_out[0 / 1] receive the
+ * slots of A / B.  exp_stats: flag_id >= 0 also writes that launch flag from
+ * the two decisions (cumpsgemm::set_dynamic_launch_buffer_by_exp_stats,
+ * reference src/dynamic_scaling.cu:364-397), -1 leaves the flags alone.  No
+ * counterpart in the reference, which scans A and B with separate launches
+ * (src/cumpsgemm_cublas.cu:455-462, :527-536). */
+void cuMpSGEMM_exp_stats_pair_s(cuMpSGEMM_handle_t h, unsigned m_a, unsigned n_a, const float *a,
+                                unsigned lda, unsigned m_b, unsigned n_b, const float *b,
+                                unsigned ldb, int flag_id, unsigned *ids_out /* [2] */);
+void cuMpSGEMM_exp_max_pair_s(cuMpSGEMM_handle_t h, unsigned m_a, unsigned n_a, const float *a,
+                              unsigned lda, unsigned m_b, unsigned n_b, const float *b,
+                              unsigned ldb, unsigned *ids_out /* [2] */);
 /* cumpsgemm::get_exp_stats (cumpsgemm.hpp:48-49): synchronises the stream */
 void cuMpSGEMM_get_exp_stats(cuMpSGEMM_handle_t h, unsigned id, uint64_t *underflow,
                              uint64_t *total);

@@ -305,10 +305,11 @@ def test_pipeline_rejects_what_the_statistics_cannot_address(handle, dev, mode):
 
 @pytest.mark.parametrize("mode", [SCALING, AUTO])
 @pytest.mark.parametrize("cplx", [False, True])
-@pytest.mark.parametrize("restore,fused", [(True, True), (True, False), (False, False)])
+@pytest.mark.parametrize("restore,fused", [(True, True), (True, False), (False, False), (False, True)])
 def test_scaled_pipelines_with_beta(O, handle, dev, monkeypatch, mode, cplx, restore, fused):
     """alpha * op(A) * op(B) + beta * C in the scaled modes, beta != 0, against FP64: the fused form
-    (A, B untouched), the stand-alone passes with restoration and the form that leaves A and B scaled
+    (A, B untouched), the stand-alone passes with restoration and the two forms that leave A and B
+    scaled (stand-alone passes; fused GEMM with A and B scaled afterwards)
     all keep beta * C_old out of the rescaling of C.  (Rescaling the finished C, as the reference's
     sequence does, src/cumpsgemm_cublas.cu:549-559, would multiply beta * C_old by 2^-17 here.)"""
     m, n, k = 200, 136, 160
@@ -337,9 +338,62 @@ def test_scaled_pipelines_with_beta(O, handle, dev, monkeypatch, mode, cplx, res
     if mode == AUTO:
         assert handle.get_dynamic_launch_flag(ids[2]) == (FP16TCEC | 0x40)
     assert np.array_equal(a_after, a) == restore
+    if not restore:   # A is left multiplied by 2^14 / 2^floor(log2 max|A|), whichever form ran
+        ma = handle.get_max_exp(ids[0])
+        want = O.scale_matrix(a.view(np.float32).copy(), (2 if cplx else 1) * k, m, (2 if cplx else 1) * k,
+                              O.lib().oracle_scale_ab_coef(ma))
+        assert np.array_equal(a_after.view(np.float32), want)
     ref = O.gemm_fp64(T, N, m, n, k, alpha, a, k, b, k, beta, c0, ldc)
     cf = oracle_gemm(O, FP32, T, N, m, n, k, alpha, a, k, b, k, beta, c0, ldc)
     r, r32 = O.residual(ref, c, m, n, ldc), O.residual(ref, cf, m, n, ldc)
     assert r <= 2.0 * r32 + 2.0 ** -24, (r, r32)
     # rows m .. ldc of every column are not part of C
     assert np.array_equal(c.reshape(n, ldc)[:, m:], c0.reshape(n, ldc)[:, m:])
+
+
+@pytest.mark.parametrize("mode", [SCALING, AUTO])
+@pytest.mark.parametrize("restore", [True, False])
+def test_scaled_pipeline_keeps_a_large_c_with_tiny_operands(handle, dev, mode, restore):
+    """A and B near 2^-30 are scaled up by 2^44 each, so the product of the two inverse factors is
+    2^-88; with beta != 0 and C_old near 2^45 nothing on the way may divide C_old by that product
+    (2^133 is outside FP32).  alpha * A * B (about 2^-55) vanishes next to beta * C_old here, so the
+    result is beta * C_old exactly."""
+    m = n = k = 128
+    a = (inputs.uniform(71, m * k) * np.float32(2.0 ** -30)).astype(np.float32)
+    b = (inputs.uniform(72, k * n) * np.float32(2.0 ** -30)).astype(np.float32)
+    c0 = (inputs.uniform(73, m * n) * np.float32(2.0 ** 45)).astype(np.float32)
+    if mode == AUTO:
+        handle.set_exp_stats_params(0.0, 2.0 ** -15, 0.1)
+    try:
+        da, db, dc = dev.up(a), dev.up(b), dev.up(c0)
+        st, ids = handle.gemm_pipeline(N, N, m, n, k, 1.0, da, m, db, k, 0.5, dc, m, mode, restore_ab=restore)
+        assert st == 0
+        c = dev.down(dc)
+        a_after = dev.down(da)
+    finally:
+        handle.set_exp_stats_params(0.0, 2.0 ** -15, 0.0)
+    assert np.isfinite(c).all()
+    assert np.array_equal(c, np.float32(0.5) * c0)
+    assert np.array_equal(a_after, a) == restore
+    if not restore:
+        assert 2.0 ** 14 <= np.abs(a_after).max() < 2.0 ** 15
+
+
+@pytest.mark.parametrize("mode", [SCALING, AUTO])
+@pytest.mark.parametrize("missing", ["a", "b", "c"])
+def test_scaled_pipeline_refuses_a_null_matrix_before_any_launch(handle, dev, mode, missing):
+    """A null operand leaves the statistics nothing to scan; the call is refused before the scaling
+    passes and the GEMM could run on whatever the slot and flag rings held: C and the operands stay
+    as they were and no slot or flag is taken from the rings."""
+    m = n = k = 96
+    a, b = inputs.uniform(74, m * k), inputs.uniform(75, k * n)
+    c0 = inputs.uniform(76, m * n)
+    da, db, dc = dev.up(a), dev.up(b), dev.up(c0)
+    slot_before = handle.get_current_exp_stats_buffer_id()
+    args = {"a": da, "b": db, "c": dc}
+    args[missing] = None
+    st, _ = handle.gemm_pipeline(N, N, m, n, k, 1.0, args["a"], m, args["b"], k, 0.0, args["c"], m, mode,
+                                 restore_ab=False)
+    assert st == 3                       # HIPBLAS_STATUS_INVALID_VALUE
+    assert handle.get_current_exp_stats_buffer_id() == slot_before
+    assert np.array_equal(dev.down(dc), c0) and np.array_equal(dev.down(da), a) and np.array_equal(dev.down(db), b)

@@ -194,3 +194,27 @@ def test_launch_flag_combination(O, handle, dev):
             assert handle.get_dynamic_launch_flag(fid) == O.lib().oracle_combine_flag(ma, mb)
     assert handle.get_dynamic_launch_flag(0) == TF32TCEC
     assert handle.get_dynamic_launch_flag(1) == (3 << 5) | FP16TCEC
+
+
+@pytest.mark.parametrize("shapes", [((700, 300), (300, 900)), ((4096, 4096), (64, 64)), ((1, 1), (2048, 1024))])
+def test_pair_launch_matches_two_single_launches(O, handle, dev, shapes):
+    """A and B of a GEMM scanned by one launch per pass: the same slots, counts, maxima and
+    decisions as one call per matrix (and as the oracle), and the launch flag of the pair."""
+    (ma, na), (mb, nb) = shapes
+    a = inputs.normal(81, ma * na, 2.0 ** -14)       # some elements below the underflow threshold
+    b = inputs.normal(82, mb * nb, 1.0)
+    da, db = dev.up(a), dev.up(b)
+    handle.set_exp_stats_params(0.0, 2.0 ** -15, 0.0)
+    flag = handle.get_next_dynamic_launch_buffer_id()
+    ia, ib = handle.exp_stats_pair(ma, na, da, ma, mb, nb, db, mb, flag_id=flag)
+    assert ib == ia + 1 or ib == 2
+    for sid, x, mm, nn in ((ia, a, ma, na), (ib, b, mb, nb)):
+        o = O.exp_stats(x, mm, nn, mm)
+        assert handle.get_exp_stats(sid) == (o.underflow, o.total)
+        assert int(np.float32(handle.get_max_exp(sid)).view(np.uint32)) == o.max_exp_bits
+        assert handle.get_exp_stats_compute_mode_level(sid) == o.mode
+    oa, ob = O.exp_stats(a, ma, na, ma), O.exp_stats(b, mb, nb, mb)
+    assert handle.get_dynamic_launch_flag(flag) == O.lib().oracle_combine_flag(oa.mode, ob.mode)
+    ja, jb = handle.exp_max_pair(ma, na, da, ma, mb, nb, db, mb)
+    assert int(np.float32(handle.get_max_exp(ja)).view(np.uint32)) == oa.max_exp_bits
+    assert int(np.float32(handle.get_max_exp(jb)).view(np.uint32)) == ob.max_exp_bits

@@ -15,7 +15,7 @@ N_OP, T_OP = 111, 112
 FP16TCEC, TF32TCEC, FP16TC = 1, 2, 3
 
 
-def _pair(cg, torch, h, mode, opa, opb, m, n, k, alpha, beta, seed):
+def _pair(cg, torch, h, mode, opa, opb, m, n, k, alpha, beta, seed, fp64_bar=False):
     dev = torch.device("cuda:0")
     pad = 3
     lda = (m if opa == N_OP else k) + pad
@@ -41,6 +41,14 @@ def _pair(cg, torch, h, mode, opa, opb, m, n, k, alpha, beta, seed):
         assert float((x - y).norm() / y.norm()) <= 4 * 2.0 ** -24 * np.sqrt(k), (m, n, k, mid)
     # the padding of C (rows m .. ldc) is untouched
     assert torch.equal(c_new.view(n, ldc)[:, m:], c0.view(n, ldc)[:, m:])
+    if fp64_bar:   # small problems: against FP64 as well, within the reference's bar 2^-23 sqrt(K)
+        A = a.view(-1, lda)[:, :(m if opa == N_OP else k)].double()
+        A = A.t() if opa == N_OP else A                 # logical m x k
+        B = b.view(-1, ldb)[:, :(k if opb == N_OP else n)].double()
+        B = B.t() if opb == N_OP else B                 # logical k x n
+        ref = alpha * (A @ B) + beta * c0.view(n, ldc)[:, :m].t().double()
+        got = c_new.view(n, ldc)[:, :m].t().double()
+        assert float((got - ref).norm() / ref.norm()) <= 2.0 ** -23 * np.sqrt(k), (m, n, k)
 
 
 @pytest.mark.parametrize("mode", [FP16TCEC, TF32TCEC])
@@ -53,6 +61,26 @@ def test_no_alloc_matches_sgemm_on_two_calls_in_a_row(cg, torch_gpu, mode):
         # ... then smaller, ragged problems over the same array: other layouts, beta != 0
         _pair(cg, torch_gpu, h, mode, T_OP, N_OP, 1000, 777, 520, 0.5, 0.25, 110)
         _pair(cg, torch_gpu, h, mode, N_OP, T_OP, 300, 2500, 131, -1.0, 1.0, 120)
+    finally:
+        torch_gpu.cuda.synchronize()
+        h.close()
+
+
+@pytest.mark.parametrize("mode", [FP16TCEC, TF32TCEC])
+def test_no_alloc_on_problems_smaller_than_one_tile(cg, torch_gpu, mode, monkeypatch):
+    """The call takes the pre-split path whatever the shape: results narrower or lower than the
+    256 x 128 (128 x 128) tile of its kernels, down to a single row or column -- and whatever
+    the variables say that steer cuMpSGEMM_sgemm away from that path."""
+    h = cg.Handle()
+    h.set_stream(torch_gpu.cuda.current_stream())
+    try:
+        _pair(cg, torch_gpu, h, mode, N_OP, N_OP, 70, 33, 130, 1.0, 0.0, 130, fp64_bar=True)
+        _pair(cg, torch_gpu, h, mode, T_OP, N_OP, 1, 4096, 256, 1.5, -0.5, 140, fp64_bar=True)
+        _pair(cg, torch_gpu, h, mode, N_OP, T_OP, 4100, 1, 160, 1.0, 1.0, 150, fp64_bar=True)
+        monkeypatch.setenv("CUMPSGEMM_PACKED", "0")
+        monkeypatch.setenv("CUMPSGEMM_FORCE_TILE_CLASS", "2")
+        monkeypatch.setenv("CUMPSGEMM_FORCE_KSPLIT", "4")
+        _pair(cg, torch_gpu, h, mode, N_OP, N_OP, 300, 200, 256, 1.0, 0.0, 160, fp64_bar=True)
     finally:
         torch_gpu.cuda.synchronize()
         h.close()
