@@ -66,6 +66,10 @@ def main():
     ap.add_argument("--shape", default=None,
                     help="with --kernel-only: M,N,K[,BATCH] instead of a square --size (BATCH > 1: strided batch)")
     ap.add_argument("--cplx", action="store_true", help="with --kernel-only --shape: complex64 operands (CGEMM)")
+    ap.add_argument("--stamps", action="store_true",
+                    help="with --kernel-only --shape and a library built with -DCUMPSGEMM_WALK_STAMPS=1 "
+                         "(CUMPSGEMM_LIBRARY=...): print the in-kernel clock stamps of one call of the "
+                         "tile-walking pre-split kernel, tile by tile")
     ap.add_argument("--op", default="NN", choices=["NN", "TN", "NT", "TT"])
     ap.add_argument("--data", default="uniform", choices=["uniform", "zeros", "ones", "ints", "fp16"],
                     help="with --kernel-only: operand values (the part is power-limited and the MFMAs' "
@@ -313,6 +317,42 @@ def shape_kernel_only(args, torch, cg, h, dev, stream):
     flops = (8.0 if args.cplx else 2.0) * m * n * k * batch
     print(json.dumps({"kernel_only": True, "shape": [m, n, k, batch], "cplx": args.cplx, "op": args.op, "mode": args.mode,
                       "data": args.data, "kernel_ms": round(ms, 4), "tflops": round(flops / ms / 1e9, 2)}), flush=True)
+    if args.stamps:
+        walk_stamps(torch, cg, dev, fn, k)
+
+
+def walk_stamps(torch, cg, dev, fn, k):
+    """One more call with the stamp buffer installed; per tile of the two traced workgroups: clocks from the
+    previous event to `this wave is done with the step` and from there to `past the barrier`, for every
+    K-step, and the clocks the write-out took to issue."""
+    L = cg.lib()
+    buf = torch.zeros(1024, dtype=torch.int64, device=dev)
+    if L.cuMpSGEMM_set_walk_stamp_buffer(buf.data_ptr()) != 0:
+        sys.exit("bench.py --stamps: this library was not built with -DCUMPSGEMM_WALK_STAMPS=1")
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    fn()
+    e1.record()
+    torch.cuda.synchronize()
+    L.cuMpSGEMM_set_walk_stamp_buffer(None)
+    us = e0.elapsed_time(e1) * 1e3
+    t = buf.cpu().numpy()
+    nk = (k + 31) // 32
+    per = 2 * nk + 1
+    for wg, base in ((0, 0), (101, 512)):
+        cnt = int(t[base])
+        ev = [int(x) % (1 << 64) for x in t[base + 1: base + 1 + cnt]]
+        clk = [e & ((1 << 60) - 1) for e in ev]
+        if cnt < 2 * per:
+            print(f"workgroup {wg}: {cnt} stamps (the call did not run the tile-walking pre-split kernel?)")
+            continue
+        print(f"workgroup {wg}: call {us:.0f} us, {cnt} stamps over {clk[-1] - clk[0]} clocks "
+              f"({(clk[-1] - clk[0]) / us:.0f} clocks per us)")
+        for ti in range(1, min(cnt // per, 6)):
+            seg = clk[ti * per - 1: (ti + 1) * per]
+            d = [seg[i + 1] - seg[i] for i in range(len(seg) - 1)]
+            print(f"  tile {ti}: own work + wait {[d[2 * i] for i in range(nk)]} at the barrier "
+                  f"{[d[2 * i + 1] for i in range(nk)]} write-out {d[-1]}")
 
 
 def hbm_kernel_only(args, torch, cg, inputs, h, dev, stream):

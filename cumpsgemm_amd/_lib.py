@@ -3,7 +3,8 @@ import os
 import subprocess
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-_LIB = os.path.join(_HERE, "libcumpsgemm.so")
+# CUMPSGEMM_LIBRARY: another build of the library (a diagnostic one, say) instead of the in-tree file
+_LIB = os.environ.get("CUMPSGEMM_LIBRARY") or os.path.join(_HERE, "libcumpsgemm.so")
 _RULE_LIB = os.path.join(_HERE, "libcumpsgemm_rule.so")
 
 # hipblasOperation_t
@@ -78,6 +79,7 @@ def _declare(L):
     L.cuMpSGEMM_cgemm.argtypes = [_ptr, _int, _int] + gemm_tail + [c2p, _ptr, _u64, _ptr, _u64, c2p, _ptr, _u64, _int]
     L.cuMpSGEMM_sgemm_ex.argtypes = L.cuMpSGEMM_sgemm.argtypes + [ctypes.POINTER(_u32)]
     L.cuMpSGEMM_sgemm_no_alloc.argtypes = L.cuMpSGEMM_sgemm.argtypes
+    L.cuMpSGEMM_set_walk_stamp_buffer.argtypes = [_ptr]
     L.cuMpSGEMM_get_static_scratch_size.argtypes = []
     L.cuMpSGEMM_get_static_scratch_size.restype = ctypes.c_size_t
     L.cuMpSGEMM_cgemm_ex.argtypes = L.cuMpSGEMM_cgemm.argtypes + [ctypes.POINTER(_u32)]

@@ -25,6 +25,7 @@ Tuning read_tuning_env() {
   if (const char *v = std::getenv("CUMPSGEMM_PACKED_WALK")) t.packed_walk = v[0] == '1' ? 1 : 0;
   const int rg = as_int("CUMPSGEMM_RASTER_GROUP", 0);
   t.raster_group = (rg >= 1 && rg <= 64) ? rg : 0;
+  t.fetch_from_one_patch = std::getenv("CUMPSGEMM_EXP_FETCH_FROM_ONE_PATCH") != nullptr;
   t.force_cls = as_int("CUMPSGEMM_FORCE_TILE_CLASS", -1);
   if (t.force_cls < 0 || t.force_cls >= kNumTileClasses) t.force_cls = -1;
   t.force_split = as_int("CUMPSGEMM_FORCE_KSPLIT", 0);
@@ -40,6 +41,7 @@ Tuning read_tuning_env() {
 // immutable object and leaves the old one in place (never freed: a few dozen
 // bytes per reload, and reloads are a test facility), so a thread that took a
 // reference before the reload keeps reading a consistent set of values.
+std::atomic<unsigned long long *> g_walk_stamps{nullptr}; // (diagnostic builds only)
 std::atomic<const Tuning *> g_tuning{nullptr};
 std::mutex g_tuning_mutex;
 } // namespace
@@ -348,7 +350,7 @@ PreSplitChoice choose_pre_split(const cuMpSGEMM_handle *h, bool a_kc, bool b_kc,
                                 int force_cls, int force_split, int depth) {
   PreSplitChoice ch;
   ch.tc_only = mode == CUMPSGEMM_FP16TC || mode == CUMPSGEMM_TF32TC;
-  if (CPLX && mode != CUMPSGEMM_FP16TCEC && !ch.tc_only) return ch; // (complex bf16x3 has no pre-split form)
+  if (CPLX && mode != CUMPSGEMM_FP16TCEC && mode != CUMPSGEMM_TF32TCEC && !ch.tc_only) return ch; // (AUTO: real only)
   // CUMPSGEMM_PACKED: "0" never, "1" whenever possible; the entry point that
   // allocates nothing always goes this way (its planes have a home already)
   const bool forced = h->ws_override != nullptr;
@@ -360,6 +362,7 @@ PreSplitChoice choose_pre_split(const cuMpSGEMM_handle *h, bool a_kc, bool b_kc,
   ch.bm = CPLX ? kPackedCplxBM : (ch.bf16 ? kPackedBf16BM : kPackedBM);
   ch.bn = CPLX ? kPackedCplxBN : (ch.bf16 ? kPackedBf16BN : kPackedBN);
   ch.planes = (CPLX ? 2u : 1u) * (ch.bf16 ? 3u : (mode == CUMPSGEMM_FP16TC ? 1u : 2u));
+  // (complex bf16x3: the 128x64 complex tile, like the other complex modes)
   // (the pre-pass launches workgroups of 64 rows x 32 .. 256 K-values on a 2-D grid)
   const bool shape_ok = batch == 1 && k >= 128 &&
                         (forced || (uint64_t)m * n >= (uint64_t)h->num_cus * ch.bm * ch.bn) && k / 32 < 65535;
@@ -426,7 +429,12 @@ PreSplitChoice choose_pre_split(const cuMpSGEMM_handle *h, bool a_kc, bool b_kc,
               : ((k >= 1024 && mn_ratio >= (mode == CUMPSGEMM_FP16TC ? 1500.0 : 2000.0)) ||
                  (k >= 512 && mn_ratio >= 4000.0) || (k >= 256 && mn_ratio >= 8000.0) ||
                  (mode == CUMPSGEMM_TF32TC && pays_nt_shape)));
-    return ch.bf16 ? (pays_bf16 || always) : (ch.tc_only ? (pays_tc || always) : (pays || pays_scaled || always));
+    // (complex bf16x3, two-buffer pre-split kernel against the in-loop one, NN / TN, TFLOP/s: 4096^3 228 / 238 ->
+    // 237 / 237, 3072^2 x 1024 205 / 215 -> 223 / 223, 4096^2 x 512 211 / 216 -> 230 / 226, 8192^2 x 256 197 / 205 ->
+    // 219 / 218, 3072^2 x 384 189 / 199 -> 203 / 202, 2048^2 x 1024 222 / 230 -> 231 / 231, 4096^2 x 256 198 / 205 ->
+    // 206 / 210; 2048^2 x 512 level: the complex rule above)
+    const bool pays_b3 = CPLX ? pays_cplx : pays_bf16;
+    return ch.bf16 ? (pays_b3 || always) : (ch.tc_only ? (pays_tc || always) : (pays || pays_scaled || always));
   };
   const bool mode_ok = mode == CUMPSGEMM_FP16TCEC || ch.bf16 || ch.auto_ok || ch.tc_only;
   // (CUMPSGEMM_FORCE_TILE_CLASS / _FORCE_KSPLIT pick among the in-loop kernels and keep a call off this
@@ -555,6 +563,8 @@ PreSplit run_pre_split(cuMpSGEMM_handle *h, const GemmArgs &args, bool a_kc, boo
                 : (walk_rule == kWalkAlways ? true
                    : (walk_rule == kWalkMid ? pargs.k / 32 <= 32 : pargs.k / 32 < 16));
     if (tuning().packed_walk >= 0) walk = tuning().packed_walk == 1;
+    if (kind == PackKind::BF16X3_COMPLEX) walk = false; // (its kernel has the one-tile form only)
+    if (walk && tuning().fetch_from_one_patch) pargs.raster_group |= kFetchFromOnePatch; // (profiler experiment)
     const dim3 grid = walk ? dim3((unsigned)std::min<uint64_t>(total, h->num_cus), 1, 1)
                            : dim3((unsigned)total, 1, 1);
     launch_kernel(pargs, grid, walk);
@@ -570,7 +580,10 @@ PreSplit run_pre_split(cuMpSGEMM_handle *h, const GemmArgs &args, bool a_kc, boo
   const uint32_t accept = ch.auto_ok ? accept_fp16 : 0u;
   bool ok;
   if constexpr (CPLX) {
-    if (ch.tc_only) {
+    if (ch.bf16) {
+      ok = run(PackKind::BF16X3_COMPLEX, pa, pb, ch.bm, ch.bn, 0u, false,
+               [&](const GemmArgs &g, dim3 grid, bool) { launch_packed_bf16x3_c(g, grid, h->stream); }, kWalkNever);
+    } else if (ch.tc_only) {
       const bool fp16 = mode == CUMPSGEMM_FP16TC;
       ok = run(fp16 ? PackKind::FP16TC_COMPLEX : PackKind::BF16X2_COMPLEX, pa, pb, ch.bm, ch.bn, 0u, false,
                [&](const GemmArgs &g, dim3 grid, bool walk) {
@@ -655,6 +668,9 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
   scalar_parts<T>::get(beta, args.beta_re, args.beta_im);
   args.conj_a = (CPLX && op_A == HIPBLAS_OP_C) ? 1u : 0u;
   args.conj_b = (CPLX && op_B == HIPBLAS_OP_C) ? 1u : 0u;
+#if CUMPSGEMM_WALK_STAMPS
+  args.stamps = g_walk_stamps.load();
+#endif
   args.raster_group = (uint32_t)tuning().raster_group; // experiments: tile order of the one-tile kernels
 
   // which kernels to launch: one for a fixed mode; for AUTO both candidates,
@@ -1122,6 +1138,16 @@ hipblasStatus_t cuMpSGEMM_sgemm_no_alloc(cuMpSGEMM_handle_t handle, hipblasOpera
   handle->ws_override = nullptr;
   handle->ws_override_bytes = 0;
   return st;
+}
+
+hipblasStatus_t cuMpSGEMM_set_walk_stamp_buffer(void *device_buffer) {
+#if CUMPSGEMM_WALK_STAMPS
+  g_walk_stamps.store(static_cast<unsigned long long *>(device_buffer));
+  return HIPBLAS_STATUS_SUCCESS;
+#else
+  (void)device_buffer;
+  return HIPBLAS_STATUS_NOT_SUPPORTED;
+#endif
 }
 
 size_t cuMpSGEMM_get_static_scratch_size(void) { return (size_t)kStaticScratchBytes; }

@@ -9,5 +9,10 @@ namespace cumpsgemm_amd {
     CUMPSGEMM_ENTRY(Prec::BF16X3, true, AKC, BKC, 64, 32, 32, 32, 1, false, "c64x32x32_w32x32"), \
     CUMPSGEMM_ENTRY(Prec::BF16X3, true, AKC, BKC, 64, 32, 32, 32, 1, false, "c64x32x32_w32x32") }
 CUMPSGEMM_DEFINE_TABLE(g_tab_bf16x3_c, ROW)
+// the large complex tile over pre-split operands (planes re b0, b1, b2, im b0,
+// b1, b2; K-contiguous): two LDS buffers, one tile per workgroup
+void launch_packed_bf16x3_c(const GemmArgs &args, dim3 grid, hipStream_t stream) {
+  launch_cfg<GemmCfg<Prec::BF16X3, true, true, true, 128, 64, 32, 32, 2, false, false, false, true>>(args, grid, stream);
+}
 #undef ROW
 } // namespace cumpsgemm_amd

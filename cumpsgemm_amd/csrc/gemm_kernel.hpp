@@ -39,6 +39,13 @@
 #ifndef CUMPSGEMM_MFMA_EDGE_INLOOP
 #define CUMPSGEMM_MFMA_EDGE_INLOOP 32
 #endif
+// Diagnostic build (-DCUMPSGEMM_WALK_STAMPS=1): the tile-walking pre-split
+// kernel records the shader clock in front of and behind every K-step's barrier
+// and after every write-out (first wave of two workgroups), see
+// cuMpSGEMM_set_walk_stamp_buffer.  Off in the library that is shipped.
+#ifndef CUMPSGEMM_WALK_STAMPS
+#define CUMPSGEMM_WALK_STAMPS 0
+#endif
 
 namespace cumpsgemm_amd {
 
@@ -110,7 +117,7 @@ struct GemmArgs {
   uint32_t tiles_m, tiles_n;
   uint32_t batch;      // persistent kernels walk (tile, batch) pairs themselves
   uint32_t atomic_out; // split-K: C += alpha*acc with float atomics
-  uint32_t raster_group; // tile rows per column group of the tile order (0: 8)
+  uint32_t raster_group; // tile rows per column group of the tile order (0: 8); | kFetchFromOnePatch
   // AUTO mode: device flag consulted before doing any work.  The kernel runs
   // only if ((1u << (flag & 31)) & flag_accept_mask) != 0.
   const int *launch_flag;
@@ -121,7 +128,14 @@ struct GemmArgs {
   // flag -- so that no host synchronisation is needed.
   const uint32_t *scale_max_a, *scale_max_b; // bits of 2^floor(log2 max|x|)
   const int *scale_flag;                     // bit 6: scale A, bit 5: scale B
+#if CUMPSGEMM_WALK_STAMPS
+  unsigned long long *stamps; // 2 x 512 words: [count, stamps...] of workgroups 0 and 101
+#endif
 };
+
+// Bit of GemmArgs::raster_group understood by the tile-walking pre-split kernel
+// only: a profiler experiment (see there), never set by a normal call.
+constexpr uint32_t kFetchFromOnePatch = 0x80000000u;
 
 // ---- split one group of 8 FP32 values into NP packed 16-byte plane chunks ----
 template <Prec P> struct splitter;
@@ -248,7 +262,7 @@ __device__ inline f4v_t mfma_block(const u4_t a, const u4_t b, const f4v_t c) {
 //   SCALED (FP16TCEC only): op(A), op(B) are multiplied by powers of two read
 //         from device memory while they are split, and the result by the
 //         inverse product when it is written out (see GemmArgs).
-//   PACKED (three-buffer kernels; FP16TCEC real and complex, real bf16x3): A
+//   PACKED (three-buffer kernels; complex bf16x3: two buffers): A
 //         and B were split beforehand into fp16 / bf16 planes laid out as the
 //         LDS image of every (tile, K-step), see pack_split_kernel; staging is
 //         a plain 16-byte copy, no arithmetic.
@@ -266,8 +280,11 @@ struct GemmCfg {
   static constexpr bool KS2 = KS2_;
   // (PACKED + SCALED: the operands were scaled when they were pre-split; the
   // kernel only folds the inverse scaling of C into alpha)
-  static_assert(!PACKED_ || (DEEP_ && (P_ != Prec::BF16X3 || !CPLX_)),
-                "packed form");
+  // (three buffers of pre-split planes, except for complex bf16x3, whose six
+  // planes per operand leave room for two: its pre-split kernel is the
+  // two-buffer, one-tile form)
+  static_assert(!PACKED_ || (DEEP_ != (P_ == Prec::BF16X3 && CPLX_)), "packed form");
+  static_assert(!(PACKED_ && !DEEP_) || !PERSIST_, "two-buffer packed form: one tile per workgroup");
   static constexpr bool PACKED = PACKED_;
   static_assert(!PERSIST_ || DEEP_, "persistent kernels use the three-buffer pipeline");
   static_assert(!SCALED_ || P_ == Prec::FP16TCEC, "scaling guards the fp16 range only");
@@ -860,7 +877,8 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
   uint32_t tile_m, tile_n, tile_b = blockIdx.y;
   if constexpr (Cfg::PERSIST) {
     // (the walk over pre-split operands takes its column-group height from the host)
-    const uint32_t group = (Cfg::PACKED && args.raster_group) ? args.raster_group : 8u;
+    const uint32_t rg = args.raster_group & ~kFetchFromOnePatch;
+    const uint32_t group = (Cfg::PACKED && rg) ? rg : 8u;
     map_tile_batched(blockIdx.x, args.tiles_m, args.tiles_n, args.batch, tile_m, tile_n, tile_b, group);
   } else {
     map_tile(blockIdx.x, args.tiles_m, args.tiles_n, tile_m, tile_n, args.raster_group ? args.raster_group : 8u);
@@ -971,8 +989,12 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
     const float *ap = a_tile + (uint64_t)kt * a_kstep;
     const float *bp = b_tile + (uint64_t)kt * b_kstep;
     if constexpr (Cfg::PACKED) {
-      LA::template load_packed<NP * NCOMP>(ra, ap, (uint32_t)args.lda * 64u);
-      LB::template load_packed<NP * NCOMP>(rb, bp, (uint32_t)args.ldb * 64u);
+      // (register-staged copy of the planes: the three-buffer forms only; the
+      // two-buffer form never comes here)
+      if constexpr (Cfg::DEEP) {
+        LA::template load_packed<NP * NCOMP>(ra, ap, (uint32_t)args.lda * 64u);
+        LB::template load_packed<NP * NCOMP>(rb, bp, (uint32_t)args.ldb * 64u);
+      }
     } else if constexpr (FAST) {
       LA::load_fast(ra, ap, args.lda, offa);
       LB::load_fast(rb, bp, args.ldb, offb);
@@ -986,8 +1008,10 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
     char *sa = lds + stage * Cfg::STAGE_BYTES;
     char *sb = sa + Cfg::A_STAGE_BYTES;
     if constexpr (Cfg::PACKED) {
-      LA::template store_packed<NP * NCOMP>(ra, sa, tid);
-      LB::template store_packed<NP * NCOMP>(rb, sb, tid);
+      if constexpr (Cfg::DEEP) {
+        LA::template store_packed<NP * NCOMP>(ra, sa, tid);
+        LB::template store_packed<NP * NCOMP>(rb, sb, tid);
+      }
     } else {
       LA::template store<P, Cfg::SCALED>(ra, sa, tid, coef_a, coef_a2048);
       LB::template store<P, Cfg::SCALED>(rb, sb, tid, coef_b, coef_b2048);
@@ -1223,16 +1247,30 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
     const uint32_t total = args.tiles_m * args.tiles_n * args.batch;
     const uint32_t my_tiles = (total - blockIdx.x + gridDim.x - 1) / gridDim.x;
     const int nk = klen / BK;
+    // (profiler experiment, kFetchFromOnePatch: every workgroup reads the planes
+    // of the tile that its slot has in the first round of XCD 0, first K-step
+    // only -- 32 tiles' worth of operands that every L2 keeps, so that nothing
+    // but the first touch goes over the fabric -- while C is written where it
+    // belongs.  The results are meaningless; the time is that of the same
+    // instruction stream without operand traffic beyond the L2.)
+    const bool one_patch = (args.raster_group & kFetchFromOnePatch) != 0;
+    const uint32_t group = (args.raster_group & ~kFetchFromOnePatch) ? (args.raster_group & ~kFetchFromOnePatch) : 8u;
     auto tile_at = [&](uint32_t i, const float *&at, const float *&bt, float *&ct, uint32_t &om0, uint32_t &on0) {
       uint32_t tm, tn, bat;
       map_tile_batched(blockIdx.x + (i < my_tiles ? i : my_tiles - 1) * gridDim.x, args.tiles_m,
-                       args.tiles_n, args.batch, tm, tn, bat, args.raster_group ? args.raster_group : 8u);
+                       args.tiles_n, args.batch, tm, tn, bat, group);
       om0 = tm * BM;
       on0 = tn * BN;
-      at = packed_origin(reinterpret_cast<const float *>(args.a), args.lda, om0);
-      bt = packed_origin(reinterpret_cast<const float *>(args.b), args.ldb, on0);
+      if (one_patch) {
+        const uint32_t slot = blockIdx.x / 8u; // position among the workgroups of one XCD
+        tm = slot % group;
+        tn = slot / group;
+      }
+      at = packed_origin(reinterpret_cast<const float *>(args.a), args.lda, tm * BM);
+      bt = packed_origin(reinterpret_cast<const float *>(args.b), args.ldb, tn * BN);
       ct = reinterpret_cast<float *>(args.c);
     };
+    const uint64_t a_adv = one_patch ? 0 : a_kstep, b_adv = one_patch ? 0 : b_kstep;
     constexpr int NDMA = LA::template dma_loads<NP * NCOMP>() + LB::template dma_loads<NP * NCOMP>();
     static_assert(NDMA <= 15, "a K-step's loads must leave room in the 6-bit counter");
     constexpr int WAIT_AFTER_FULL = NDMA + EPI_VMEM > 63 ? 63 : NDMA + EPI_VMEM;
@@ -1242,6 +1280,7 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
     const float *la = a_tile, *lb = b_tile, *la_next, *lb_next;
     float *c_cur = c, *c_ignored;
     uint32_t cm0 = m0, cn0 = n0, i0, i1;
+    if (one_patch) tile_at(0, la, lb, c_ignored, i0, i1);
     tile_at(1, la_next, lb_next, c_ignored, i0, i1);
     int lk = 0;
     auto dma_next = [&](int stage) {
@@ -1251,12 +1290,27 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
       LB::template dma_packed<NP * NCOMP>(lb, (uint32_t)args.ldb * 64u, sb, wave);
       lk++;
       const bool wrap = (lk == nk);
-      la = wrap ? la_next : la + a_kstep;
-      lb = wrap ? lb_next : lb + b_kstep;
+      la = wrap ? la_next : la + a_adv;
+      lb = wrap ? lb_next : lb + b_adv;
       lk = wrap ? 0 : lk;
     };
     Frags f0, f1;
     int b0 = 0, b1 = 1, b2 = 2;
+#if CUMPSGEMM_WALK_STAMPS
+    unsigned long long *stamp_buf = nullptr;
+    if (args.stamps != nullptr && tid == 0 && (blockIdx.x == 0 || blockIdx.x == 101))
+      stamp_buf = args.stamps + (blockIdx.x == 0 ? 0 : 512);
+    int stamp_n = 0;
+    // tag 1: this wave's MFMAs and wait are done; 0: past the barrier; 2: write-out issued
+    auto stamp = [&](unsigned long long tag) {
+      if (stamp_buf != nullptr && stamp_n < 500) {
+        stamp_buf[1 + stamp_n] = (__builtin_readcyclecounter() & 0x0fffffffffffffffull) | (tag << 60);
+        stamp_buf[0] = ++stamp_n;
+      }
+    };
+#else
+    auto stamp = [](unsigned long long) {};
+#endif
     bool after_full = false; // the previous tile was written out by the unguarded epilogue
     // one K-step.  AFTER_WRITEOUT: the stores of the previous tile's write-out
     // stand between the loads it waits for and this step's own, so the number of
@@ -1272,7 +1326,9 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
       } else {
         __builtin_amdgcn_s_waitcnt(waitcnt_vm(NDMA));
       }
+      stamp(1);
       asm volatile("s_barrier" ::: "memory");
+      stamp(0);
       const int tmp = b0;
       b0 = b1;
       b1 = b2;
@@ -1291,6 +1347,7 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
       if (interior) epilogue(c_cur, cm0, cn0, cm0, cn0, std::true_type{});
       else epilogue(c_cur, cm0, cn0, cm0, cn0, std::false_type{});
       after_full = interior;
+      stamp(2);
       zero_acc();
       const float *ua, *ub;
       tile_at(ct + 1, ua, ub, c_cur, cm0, cn0);
@@ -1482,6 +1539,43 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
     }
   };
 
+  if constexpr (Cfg::PACKED && !Cfg::DEEP) {
+    // ---- pre-split operands, two LDS buffers, one tile per workgroup -----------
+    // (complex bf16x3: twelve planes per K-step, 72 KB.)  The planes of step
+    // t + 1 are asked for at the start of step t, into the buffer that step
+    // t - 1 was read from (free since the barrier that ended it), and must have
+    // landed when step t ends: one whole step of MFMAs -- 96 per wave here --
+    // covers the latency.
+    const int nk = klen / BK; // (pre-split operands are padded to whole K-steps)
+    const int last = nk - 1;
+    auto dma = [&](int kt, int stage) {
+      const int kc = kt < last ? kt : last;
+      char *sa = lds + stage * Cfg::STAGE_BYTES;
+      char *sb = sa + Cfg::A_STAGE_BYTES;
+      LA::template dma_packed<NP * NCOMP>(a_tile + (uint64_t)kc * a_kstep, (uint32_t)args.lda * 64u, sa, wave);
+      LB::template dma_packed<NP * NCOMP>(b_tile + (uint64_t)kc * b_kstep, (uint32_t)args.ldb * 64u, sb, wave);
+    };
+    Frags f0, f1;
+    dma(0, 0);
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    frag_load(f0, 0, 0);
+    for (int t = 0; t < nk; t++) {
+      const int cur = t & 1;
+      frag_load(f1, cur, 1);
+      dma(t + 1, cur ^ 1); // (past the end: a re-read of the last step, unused)
+      frag_mma(f0, f1);
+      __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+      asm volatile("s_barrier" ::: "memory");
+      frag_load(f0, cur ^ 1, 0);
+    }
+    if (ml0 == m0 && nl0 == n0 && rows_a == BM && rows_b == BN) {
+      epilogue(c, ml0, nl0, m0, n0, std::true_type{});
+    } else {
+      epilogue(c, ml0, nl0, m0, n0, std::false_type{});
+    }
+    return;
+  }
   if constexpr (Cfg::PACKED && !Cfg::PERSIST) {
     // ---- pre-split operands, one tile per workgroup: global -> LDS loads ------
     // The planes go from memory straight into the LDS buffers: no staging

@@ -117,6 +117,7 @@ void launch_packed_fp16tc_s(const GemmArgs &args, dim3 grid, hipStream_t stream,
 void launch_packed_bf16x2_s(const GemmArgs &args, dim3 grid, hipStream_t stream, bool walk);
 void launch_packed_fp16tc_c(const GemmArgs &args, dim3 grid, hipStream_t stream, bool walk);  // complex, 128x64
 void launch_packed_bf16x2_c(const GemmArgs &args, dim3 grid, hipStream_t stream, bool walk);
+void launch_packed_bf16x3_c(const GemmArgs &args, dim3 grid, hipStream_t stream); // complex, 128x64, two LDS buffers
 // load the real pre-split kernels (GEMM and pre-pass) onto the current device
 void prepare_packed_fp16tcec_s();
 void prepare_packed_bf16x3_s();

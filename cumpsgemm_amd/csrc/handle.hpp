@@ -66,6 +66,10 @@ struct Tuning {
   int packed = -1;      // CUMPSGEMM_PACKED: 0 never / 1 whenever possible take the pre-split path
   int packed_walk = -1; // CUMPSGEMM_PACKED_WALK: 0 / 1 force the one-tile / persistent pre-split kernel
   int raster_group = 0; // CUMPSGEMM_RASTER_GROUP: tile rows per column group (0: built-in choice)
+  // CUMPSGEMM_EXP_FETCH_FROM_ONE_PATCH (profiler experiment, WRONG RESULTS): the
+  // tile-walking pre-split kernel reads every tile's operands from one
+  // L2-resident patch, which shows what its operand traffic over the fabric costs
+  bool fetch_from_one_patch = false;
   int force_cls = -1;   // CUMPSGEMM_FORCE_TILE_CLASS
   int force_split = 0;  // CUMPSGEMM_FORCE_KSPLIT
   bool no_persistent = false;    // CUMPSGEMM_NO_PERSISTENT

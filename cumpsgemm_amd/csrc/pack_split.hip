@@ -280,6 +280,10 @@ void launch_pack_split_pair(hipStream_t stream, const PackOperand &a, const Pack
     launch_pair_of<Prec::FP16TC, true>(stream, ja, a.k_contiguous, jb, b.k_contiguous, scale_flag, launch_flag,
                                        flag_accept_mask);
     break;
+  case PackKind::BF16X3_COMPLEX:
+    launch_pair_of<Prec::BF16X3, true>(stream, ja, a.k_contiguous, jb, b.k_contiguous, scale_flag, launch_flag,
+                                       flag_accept_mask);
+    break;
   case PackKind::BF16X2_COMPLEX:
     launch_pair_of<Prec::BF16X2, true>(stream, ja, a.k_contiguous, jb, b.k_contiguous, scale_flag, launch_flag,
                                        flag_accept_mask);

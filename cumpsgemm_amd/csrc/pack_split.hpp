@@ -11,7 +11,9 @@ inline uint64_t packed_bytes(uint64_t rows_pad, uint64_t k, unsigned planes = 2)
   return ((k + 31) / 32) * planes * rows_pad * 64;
 }
 inline uint32_t packed_rows(uint64_t rows) { return (uint32_t)((rows + 255) / 256 * 256); }
-enum class PackKind { FP16_REAL, FP16_COMPLEX, BF16X3_REAL, FP16TC_REAL, BF16X2_REAL, FP16TC_COMPLEX, BF16X2_COMPLEX };
+enum class PackKind {
+  FP16_REAL, FP16_COMPLEX, BF16X3_REAL, FP16TC_REAL, BF16X2_REAL, FP16TC_COMPLEX, BF16X2_COMPLEX, BF16X3_COMPLEX
+};
 // One pre-pass launch converts both operands of a GEMM (same K).  `ld` in
 // elements of the source (complex: complex elements).  scale_max / scale_flag:
 // optional power-of-two scaling fused into the split (nullptr: none; A's is

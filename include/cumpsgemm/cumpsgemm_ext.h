@@ -54,6 +54,15 @@ hipblasStatus_t cuMpSGEMM_sgemm_no_alloc(cuMpSGEMM_handle_t handle, hipblasOpera
                                          uint64_t ldc, cuMpSGEMM_compute_mode_t compute_mode);
 size_t cuMpSGEMM_get_static_scratch_size(void);
 
+/* Diagnostic: a library built with -DCUMPSGEMM_WALK_STAMPS=1 makes the
+ * tile-walking pre-split kernel record the shader clock around every K-step's
+ * barrier and after every write-out into `device_buffer` (2 x 512 64-bit words,
+ * zeroed by the caller: per traced workgroup a count, then the stamps with a tag
+ * in bits 60-63: 1 = before the barrier, 0 = behind it, 2 = write-out issued);
+ * NULL stops it.  The library that is shipped returns
+ * HIPBLAS_STATUS_NOT_SUPPORTED.  No counterpart in the reference. */
+hipblasStatus_t cuMpSGEMM_set_walk_stamp_buffer(void *device_buffer);
+
 /* Human-readable description of one tile-config table entry; 0 on success. */
 int cuMpSGEMM_describe_tile_config(int compute_mode, int is_complex, int op_A, int op_B,
                                    int tile_class, char *buf, size_t buf_len);

@@ -10,7 +10,8 @@ import numpy as np
 import pytest
 
 from cumpsgemm_amd import inputs
-from gpu_util import N, T, C, assert_same_up_to_summation_order, make_operand, oracle_gemm, rel_diff, run_gemm
+from gpu_util import (N, T, C, assert_same_up_to_summation_order, make_operand, oracle_gemm, rel_diff, run_gemm,
+                      stored_shape)
 
 pytestmark = pytest.mark.gpu
 
@@ -364,7 +365,7 @@ def test_packed_path_matches_in_loop_split(O, handle, dev, monkeypatch, mode, op
     (N, T, 1280, 2100, 520, (0, 5, 0), 1.0, 1.0),
     (T, C, 1700, 1500, 129, (2, 0, 1), -1.0j, 0.25),
 ])
-@pytest.mark.parametrize("mode", [FP16TCEC, FP16TC, TF32TC])
+@pytest.mark.parametrize("mode", [FP16TCEC, TF32TCEC, FP16TC, TF32TC])
 def test_complex_packed_path_matches_in_loop_split(O, handle, dev, monkeypatch, mode, opa, opb, m, n, k, pads, alpha,
                                                    beta):
     gen = _gen(True)
@@ -381,13 +382,46 @@ def test_complex_packed_path_matches_in_loop_split(O, handle, dev, monkeypatch, 
         outs.append(c)
     assert_same_up_to_summation_order(outs[0], outs[1], k)
     ref = O.gemm_fp64(opa, opb, m, n, k, alpha, a, lda, b, ldb, beta, c0, ldc)
-    if mode == FP16TCEC:
+    if mode in (FP16TCEC, TF32TCEC):
         cf = oracle_gemm(O, FP32, opa, opb, m, n, k, alpha, a, lda, b, ldb, beta, c0, ldc)
         assert O.residual(ref, outs[0], m, n, ldc) <= 2.0 * O.residual(ref, cf, m, n, ldc)
     else:
         assert O.residual(ref, outs[0], m, n, ldc) <= (2.0 ** -10 if mode == FP16TC else 2.0 ** -14)
     if pads[2]:
         assert np.array_equal(outs[0].reshape(n, ldc)[:, m:], c0.reshape(n, ldc)[:, m:])
+
+
+@pytest.mark.parametrize("mode", [FP16TCEC, TF32TCEC, FP16TC, TF32TC])
+@pytest.mark.parametrize("cplx,opa,opb", [(False, N, N), (False, T, T), (True, N, N), (True, C, T), (True, T, C)])
+def test_packed_path_is_exact_on_small_integers(handle, dev, monkeypatch, mode, cplx, opa, opb):
+    """Operands with small integer values (Gaussian integers for complex data) are held exactly by
+    every plane format and every partial sum fits FP32, so whatever the order of summation the
+    pre-split kernels must return the exact product, bit for bit -- a misplaced plane, a wrong
+    sign in the complex combination or a dropped K-step would show."""
+    m, n, k = 3100, 2900, 292   # (the path needs at least one 256x128 tile per CU)
+    rng = np.random.default_rng(77)
+
+    def ints(count):
+        if cplx:
+            return (rng.integers(-8, 9, count) + 1j * rng.integers(-8, 9, count)).astype(np.complex64)
+        return rng.integers(-8, 9, count).astype(np.float32)
+    ra, ca = stored_shape(opa, m, k)
+    rb, cb = stored_shape(opb, k, n)
+    a, b = ints(ra * ca), ints(rb * cb)
+    monkeypatch.setenv("CUMPSGEMM_PACKED", "1")
+    c, st, mid = run_gemm(handle, dev, mode, opa, opb, m, n, k, 1.0, a, ra, b, rb, 0.0, np.zeros(m * n, a.dtype), m,
+                          cplx, want_module_id=True)
+    assert st == 0 and mid == 200
+
+    def logical(x, op, rows, cols):       # column-major flat buffer -> op(X) as rows x cols, in wide integers
+        r, cc = stored_shape(op, rows, cols)
+        mat = x.reshape(cc, r).T.astype(np.complex128 if cplx else np.float64)
+        if op != N:
+            mat = mat.T
+        return np.conj(mat) if op == C else mat
+    want = logical(a, opa, m, k) @ logical(b, opb, k, n)          # exact: |sums| < 2^24
+    got = c.reshape(n, m).T
+    assert np.array_equal(got.astype(want.dtype), want)
 
 
 @pytest.mark.parametrize("cplx,opa,opb,m,n,k,batch", [
