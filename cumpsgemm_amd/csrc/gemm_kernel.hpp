@@ -39,12 +39,6 @@
 #ifndef CUMPSGEMM_MFMA_EDGE_INLOOP
 #define CUMPSGEMM_MFMA_EDGE_INLOOP 32
 #endif
-// Tile-walking pre-split kernel: 1 = the barrier of a K-step stands in the
-// middle of its MFMAs and the fragment reads are spread over its four
-// quadrants ("rolling" form), 0 = barrier at the end of the step.
-#ifndef CUMPSGEMM_WALK_ROLLING
-#define CUMPSGEMM_WALK_ROLLING 0
-#endif
 // Diagnostic build (-DCUMPSGEMM_WALK_STAMPS=1): the tile-walking pre-split
 // kernel records the shader clock in front of and behind every K-step's barrier
 // and after every write-out (first wave of two workgroups), see
@@ -384,36 +378,25 @@ __device__ inline void block_sync_lds() {
 constexpr int waitcnt_vm(int n) { return (n & 15) | ((n >> 4) << 14) | (7 << 4) | (15 << 8); }
 static_assert(waitcnt_vm(6) == 0x0f76 && waitcnt_vm(63) == 0xcf7f, "s_waitcnt vmcnt immediate");
 
-// The tile-walking pre-split kernels keep global -> LDS loads in flight across
+// The tile-walking pre-split kernel keeps global -> LDS loads in flight across
 // a tile's write-out, and a wave learns that a load has landed only from its
 // vector-memory counter, which counts loads and stores alike and retires them
 // in issue order: "at most n in flight" means everything but the n youngest
 // operations is complete.  Seen from one wave, around a write-out (L(i): the
-// `ndma` loads of the next tile's K-step i), in the form with the barrier at
-// the end of a step:
+// `ndma` loads of the next tile's K-step i):
 //     last step of a tile:  L(1), MFMAs, wait(ndma), barrier
 //     write-out:            S stores
 //     first step:           L(2), MFMAs, wait(w), barrier; step 1 is read next -> L(1) complete?
 //     second step on:       L(i + 2), MFMAs, wait(ndma), barrier
 // Younger than L(1) at the first step's wait: the stores and L(2), so that
-// wait is safe iff w <= ndma + S.  In the rolling form (`ahead`) a step reads
-// the next step's planes from its own barrier on and requests run three steps
-// ahead, issued right behind the barrier:
-//     last step of a tile:  MFMAs, wait(ndma), barrier, L(2), MFMAs
-//     write-out:            S stores
-//     first step:           MFMAs, wait(w), barrier [L(1) complete?], L(3), MFMAs
-//     second step:          MFMAs, wait(w), barrier [L(2) complete?], L(4), MFMAs
-//     third step on:        MFMAs, wait(ndma), barrier, L(i + 3), MFMAs
-// Younger than L(1) at the first wait: L(2) and the stores; younger than L(2)
-// at the second: the stores and L(3): again w <= ndma + S, for two steps.
-// This function plays the sequence for three tiles of `nk` steps with S stores
-// after each and reports whether every buffer is complete when the barrier
-// before its first read is passed.
-constexpr bool walk_waits_cover(int ndma, int stores, int w, int nk, bool ahead) {
+// wait is safe iff w <= ndma + S.  This function plays the sequence for three
+// tiles of `nk` steps with S stores after each and reports whether every
+// buffer is complete when the barrier before its first read is passed.
+constexpr bool walk_waits_cover(int ndma, int stores, int w, int nk) {
   int issued = 0;        // operations issued so far
   int complete = 0;      // operations known complete (a prefix, by the in-order rule)
   int load_end[64] = {}; // issue count right after the loads of step i
-  if (3 * nk + 3 > 64 || nk < (ahead ? 4 : 2)) return false;
+  if (3 * nk + 2 > 64 || nk < 2) return false;
   auto issue_loads = [&](int step) {
     issued += ndma;
     load_end[step] = issued;
@@ -423,38 +406,28 @@ constexpr bool walk_waits_cover(int ndma, int stores, int w, int nk, bool ahead)
   };
   issue_loads(0);
   issue_loads(1);
-  if (ahead) {
-    issue_loads(2);
-    wait(2 * ndma);
-    if (load_end[0] > complete) return false; // the first step's planes are read right away
-  } else {
-    wait(0);
-  }
+  wait(0);
   for (int t = 0; t < 3; t++) {
     for (int s = 0; s < nk; s++) {
       const int step = t * nk + s;
-      if (!ahead) issue_loads(step + 2);
-      const bool after_writeout = t > 0 && (s == 0 || (ahead && s == 1));
-      wait(after_writeout ? w : ndma);
-      // barrier; from here on the planes of step + 1 are read
+      issue_loads(step + 2);
+      wait(t > 0 && s == 0 ? w : ndma);
+      // barrier; the next step reads the planes of step + 1
       if (load_end[step + 1] > complete) return false;
-      if (ahead) issue_loads(step + 3);
     }
     issued += stores; // write-out
   }
   return true;
 }
-constexpr bool walk_waits_cover_range(int ndma, int stores_lo, int stores_hi, int w, bool ahead = false) {
+constexpr bool walk_waits_cover_range(int ndma, int stores_lo, int stores_hi, int w) {
   for (int s = stores_lo; s <= stores_hi; s++)
-    for (int nk = 4; nk <= 7; nk++)
-      if (!walk_waits_cover(ndma, s, w, nk, ahead)) return false;
+    for (int nk = 2; nk <= 6; nk++)
+      if (!walk_waits_cover(ndma, s, w, nk)) return false;
   return true;
 }
 // (the model itself: one store fewer than the wait allows for must fail it)
-static_assert(walk_waits_cover_range(6, 57, 128, 63) && !walk_waits_cover(6, 56, 63, 4, false) &&
-                  walk_waits_cover_range(6, 0, 64, 6) && !walk_waits_cover(6, 0, 7, 4, false) &&
-                  walk_waits_cover_range(6, 57, 128, 63, true) && !walk_waits_cover(6, 56, 63, 4, true) &&
-                  walk_waits_cover_range(6, 0, 64, 6, true) && !walk_waits_cover(6, 0, 7, 4, true),
+static_assert(walk_waits_cover_range(6, 57, 128, 63) && !walk_waits_cover(6, 56, 63, 4) &&
+                  walk_waits_cover_range(6, 0, 64, 6) && !walk_waits_cover(6, 0, 7, 4),
               "model of the in-order vector-memory counter");
 
 // Map a linear workgroup id to a tile so that (a) workgroups that the
@@ -1093,29 +1066,6 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
                                                          b_frag_off[h] + (jb + j) * MT * 64);
       }
   };
-  // one operand half of a set only (edge 16: half h of the row / column blocks)
-  auto frag_load_a = [&](Frags &f, int stage, int h) {
-    const char *sa = lds + stage * Cfg::STAGE_BYTES;
-#pragma unroll
-    for (int q = 0; q < NCOMP; q++)
-#pragma unroll
-      for (int p = 0; p < NP; p++)
-#pragma unroll
-        for (int i = 0; i < FA; i++)
-          f.a[q][p][i] = *reinterpret_cast<const u4_t *>(sa + (q * NP + p) * Cfg::A_PLANE_BYTES + a_frag_off[h] +
-                                                         (h * FA + i) * MT * 64);
-  };
-  auto frag_load_b = [&](Frags &f, int stage, int h) {
-    const char *sb = lds + stage * Cfg::STAGE_BYTES + Cfg::A_STAGE_BYTES;
-#pragma unroll
-    for (int q = 0; q < NCOMP; q++)
-#pragma unroll
-      for (int p = 0; p < NP; p++)
-#pragma unroll
-        for (int j = 0; j < FB; j++)
-          f.b[q][p][j] = *reinterpret_cast<const u4_t *>(sb + (q * NP + p) * Cfg::B_PLANE_BYTES + b_frag_off[h] +
-                                                         (h * FB + j) * MT * 64);
-  };
   // blocks [ib, ib + FA) x [jb, jb + FB) of the wave tile += fb.b x fa.a
   // (one product after the other, so that the two correction products of a
   // block are FA * FB MFMAs apart)
@@ -1283,171 +1233,6 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
             for (int v = 0; v < NV; v++) acc[q][s][j][i][v] = 0.0f;
   };
 
-  if constexpr (Cfg::PERSIST && Cfg::PACKED && CUMPSGEMM_WALK_ROLLING != 0 && MT == 16) {
-    // ---- persistent walk over pre-split operands, rolling fragments -------------
-    // One workgroup walks its list of tiles.  A K-step's MFMAs are the four
-    // quadrants of the wave tile, from four register halves (A0, A1: the two
-    // halves of the row blocks, B0, B1: of the column blocks):
-    //     Q00 (A0, B0)   while B1 of this step is read from LDS
-    //     Q01 (A0, B1)   while A1 of this step is read
-    //     -- own loads of step t + 1 landed? barrier --  planes of step t + 3 requested
-    //     Q10 (A1, B0)   while A0 of step t + 1 is read (A0 is free since Q01)
-    //     Q11 (A1, B1)   while B0 of step t + 1 is read (B0 is free since Q10)
-    // Every quadrant's operands were requested a quadrant or more ahead, every
-    // read lands in registers the quadrant before it has released, and a step's
-    // 4 x 4 LDS reads are spread evenly over its MFMAs instead of standing in a
-    // block behind the barrier, where all eight waves wait for them together.
-    // By the barrier every wave has read the last of step t's planes (its wait
-    // covers the LDS counter too), so that buffer takes step t + 3: requests
-    // run three steps ahead and, as in the form below, have two steps to land.
-    // Around a write-out (see walk_waits_cover): the requests of the next
-    // tile's steps 1 and 2 are older than its stores, those of step 3 younger,
-    // so the waits of that tile's first two steps may leave the stores in flight
-    // (after an interior tile, whose store count is known) and no other wait may.
-    const uint32_t total = args.tiles_m * args.tiles_n * args.batch;
-    const uint32_t my_tiles = (total - blockIdx.x + gridDim.x - 1) / gridDim.x;
-    const int nk = klen / BK; // >= 4 (host): the loader changes tile at most once per tile of the multiplier
-    const bool one_patch = (args.raster_group & kFetchFromOnePatch) != 0;
-    const uint32_t group = (args.raster_group & ~kFetchFromOnePatch) ? (args.raster_group & ~kFetchFromOnePatch) : 8u;
-    auto tile_at = [&](uint32_t i, const float *&at, const float *&bt, float *&ct, uint32_t &om0, uint32_t &on0) {
-      uint32_t tm, tn, bat;
-      map_tile_batched(blockIdx.x + (i < my_tiles ? i : my_tiles - 1) * gridDim.x, args.tiles_m,
-                       args.tiles_n, args.batch, tm, tn, bat, group);
-      om0 = tm * BM;
-      on0 = tn * BN;
-      if (one_patch) { // (profiler experiment, see kFetchFromOnePatch)
-        const uint32_t slot = blockIdx.x / 8u;
-        tm = slot % group;
-        tn = slot / group;
-      }
-      at = packed_origin(reinterpret_cast<const float *>(args.a), args.lda, tm * BM);
-      bt = packed_origin(reinterpret_cast<const float *>(args.b), args.ldb, tn * BN);
-      ct = reinterpret_cast<float *>(args.c);
-    };
-    const uint64_t a_adv = one_patch ? 0 : a_kstep, b_adv = one_patch ? 0 : b_kstep;
-    constexpr int NDMA = LA::template dma_loads<NP * NCOMP>() + LB::template dma_loads<NP * NCOMP>();
-    static_assert(2 * NDMA <= 63, "two K-steps of loads in the 6-bit counter");
-    constexpr int WAIT_AFTER_FULL = NDMA + EPI_VMEM > 63 ? 63 : NDMA + EPI_VMEM;
-    static_assert(walk_waits_cover_range(NDMA, EPI_VMEM, 2 * EPI_VMEM, WAIT_AFTER_FULL, true),
-                  "waits of the first two steps after an interior write-out");
-    static_assert(walk_waits_cover_range(NDMA, 0, 2 * EPI_VMEM, NDMA, true),
-                  "waits of the first two steps after an edge write-out");
-    const float *la = a_tile, *lb = b_tile, *la_next, *lb_next;
-    float *c_cur = c, *c_ignored;
-    uint32_t cm0 = m0, cn0 = n0, i0, i1;
-    if (one_patch) tile_at(0, la, lb, c_ignored, i0, i1);
-    tile_at(1, la_next, lb_next, c_ignored, i0, i1);
-    int lk = 0;
-    auto dma_next = [&](int stage) {
-      char *sa = lds + stage * Cfg::STAGE_BYTES;
-      char *sb = sa + Cfg::A_STAGE_BYTES;
-      LA::template dma_packed<NP * NCOMP>(la, (uint32_t)args.lda * 64u, sa, wave);
-      LB::template dma_packed<NP * NCOMP>(lb, (uint32_t)args.ldb * 64u, sb, wave);
-      lk++;
-      const bool wrap = (lk == nk);
-      la = wrap ? la_next : la + a_adv;
-      lb = wrap ? lb_next : lb + b_adv;
-      lk = wrap ? 0 : lk;
-    };
-#if CUMPSGEMM_WALK_STAMPS
-    unsigned long long *stamp_buf = nullptr;
-    if (args.stamps != nullptr && tid == 0 && (blockIdx.x == 0 || blockIdx.x == 101))
-      stamp_buf = args.stamps + (blockIdx.x == 0 ? 0 : 512);
-    int stamp_n = 0;
-    auto stamp = [&](unsigned long long tag) {
-      if (stamp_buf != nullptr && stamp_n < 500) {
-        stamp_buf[1 + stamp_n] = (__builtin_readcyclecounter() & 0x0fffffffffffffffull) | (tag << 60);
-        stamp_buf[0] = ++stamp_n;
-      }
-    };
-#else
-    auto stamp = [](unsigned long long) {};
-#endif
-    Frags f0, f1; // f0 = (A0, B0), f1 = (A1, B1)
-    int b0 = 0, b1 = 1, b2 = 2; // buffers of steps t, t + 1, t + 2
-    bool after_full = false;    // the previous tile was written out by the unguarded epilogue
-    // wait for this wave's loads of the next step (and for its LDS reads of this one)
-    auto wait_next = [&](auto after_writeout_tag) {
-      constexpr int LGKM0 = ~(15 << 8); // lgkmcnt(0) instead of "any"
-      if constexpr (decltype(after_writeout_tag)::value) {
-        if (after_full) __builtin_amdgcn_s_waitcnt(waitcnt_vm(WAIT_AFTER_FULL) & LGKM0);
-        else __builtin_amdgcn_s_waitcnt(waitcnt_vm(NDMA) & LGKM0);
-      } else {
-        __builtin_amdgcn_s_waitcnt(waitcnt_vm(NDMA) & LGKM0);
-      }
-    };
-    // The reads of a quadrant are issued in front of its MFMAs (the scheduler is
-    // told the order, or it sinks them towards their first use), followed by an
-    // explicit wait that lets exactly those reads stay in flight: LDS reads
-    // return in order, so everything older -- the operands of the quadrant that
-    // starts -- has landed.  (Left to itself the compiler waits for all of them
-    // there: what is pending across the loop's back edge is more than it tracks.)
-    constexpr int QUAD_MFMAS = PT::NPROD * FA * FB * (CPLX ? 4 : 1);
-    constexpr int READS_A = NCOMP * NP * FA, READS_B = NCOMP * NP * FB;
-    static_assert(READS_A <= 15 && READS_B <= 15, "lgkmcnt immediate");
-    auto quadrant_order = [&](auto reads_tag) {
-      __builtin_amdgcn_sched_group_barrier(0x100, decltype(reads_tag)::value, 0); // LDS reads
-      __builtin_amdgcn_sched_group_barrier(0x008, QUAD_MFMAS, 0);                 // MFMAs
-      __builtin_amdgcn_sched_barrier(0);
-    };
-    auto older_reads_landed = [&](auto reads_tag) { // s_waitcnt lgkmcnt(reads), other counters untouched
-      __builtin_amdgcn_s_waitcnt((waitcnt_vm(63) & ~(15 << 8)) | (decltype(reads_tag)::value << 8));
-      __builtin_amdgcn_sched_barrier(0); // (no MFMA of the quadrant may move in front of the wait)
-    };
-    using reads_a = std::integral_constant<int, READS_A>;
-    using reads_b = std::integral_constant<int, READS_B>;
-    auto step = [&](auto after_writeout_tag) {
-      frag_load_b(f1, b0, 1);
-      frag_mma_part(f0, f0, 0, 0);    // Q00 (A0, B0 landed: the wait that ended the previous step)
-      quadrant_order(reads_b{});
-      frag_load_a(f1, b0, 1);
-      older_reads_landed(reads_a{});  // B1
-      frag_mma_part(f0, f1, 0, FB);   // Q01
-      quadrant_order(reads_a{});
-      wait_next(after_writeout_tag);
-      stamp(1);
-      asm volatile("s_barrier" ::: "memory");
-      stamp(0);
-      dma_next(b0); // (read to the end by every wave: it takes step t + 3)
-      __builtin_amdgcn_sched_barrier(0);
-      frag_load_a(f0, b1, 0);
-      frag_mma_part(f1, f0, FA, 0);   // Q10 (A1 landed: the wait in front of the barrier)
-      quadrant_order(reads_a{});
-      frag_load_b(f0, b1, 0);
-      frag_mma_part(f1, f1, FA, FB);  // Q11
-      quadrant_order(reads_b{});
-      // (A0 and B0 of the next step, requested one and two quadrants of MFMAs ago:
-      // waited for here, so that nothing is pending at the loop's back edge)
-      older_reads_landed(std::integral_constant<int, 0>{});
-      const int tmp = b0;
-      b0 = b1;
-      b1 = b2;
-      b2 = tmp;
-    };
-    dma_next(0);
-    dma_next(1);
-    dma_next(2);
-    __builtin_amdgcn_s_waitcnt(waitcnt_vm(2 * NDMA)); // the first step's planes
-    __syncthreads();
-    frag_load_a(f0, 0, 0);
-    frag_load_b(f0, 0, 0);
-    for (uint32_t ct = 0; ct < my_tiles; ct++) {
-      step(std::true_type{});
-      step(std::true_type{});
-      for (int kk = 2; kk < nk; kk++) step(std::false_type{});
-      const bool interior = cm0 + BM <= args.m && cn0 + BN <= args.n;
-      if (interior) epilogue(c_cur, cm0, cn0, cm0, cn0, std::true_type{});
-      else epilogue(c_cur, cm0, cn0, cm0, cn0, std::false_type{});
-      after_full = interior;
-      stamp(2);
-      zero_acc();
-      const float *ua, *ub;
-      tile_at(ct + 1, ua, ub, c_cur, cm0, cn0);
-      tile_at(ct + 2, la_next, lb_next, c_ignored, i0, i1);
-    }
-    __builtin_amdgcn_s_waitcnt(0);
-    return;
-  }
   if constexpr (Cfg::PERSIST && Cfg::PACKED) {
     // ---- persistent walk over pre-split operands with global -> LDS loads -----
     // One workgroup walks its list of tiles; the planes of step t + 2 are asked
