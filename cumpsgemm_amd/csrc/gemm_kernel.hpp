@@ -128,6 +128,9 @@ struct GemmArgs {
   // flag -- so that no host synchronisation is needed.
   const uint32_t *scale_max_a, *scale_max_b; // bits of 2^floor(log2 max|x|)
   const int *scale_flag;                     // bit 6: scale A, bit 5: scale B
+  // Tile-walking pre-split kernel: workgroup w starts (w / 8 mod 4) * stagger_clocks
+  // shader clocks late (0: all together), see there.
+  uint32_t stagger_clocks;
 #if CUMPSGEMM_WALK_STAMPS
   unsigned long long *stamps; // 2 x 512 words: [count, stamps...] of workgroups 0 and 101
 #endif
@@ -1131,16 +1134,21 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
   const float sgn_ab = sgn_a * sgn_b;
   // (em0, en0): origin the tile was computed from; (lo_m, lo_n): first row /
   // column this tile owns (differs from the origin for a moved edge tile).
-  auto epilogue = [&](float *cb, const uint32_t em0, const uint32_t en0, const uint32_t lo_m,
-                      const uint32_t lo_n, auto full_tag) {
+  // How a result reaches C is the same for every element of a launch, so it is
+  // decided once per tile, outside the element loops (decided per element, the
+  // write-out is a chain of scalar branches, two taken per store):
+  constexpr int OUT_STORE = 0, OUT_BETA = 1, OUT_ATOMIC = 2; // C = x | C = x + beta * C | C += x (split-K)
+  auto epilogue_body = [&](float *cb, const uint32_t em0, const uint32_t en0, const uint32_t lo_m,
+                           const uint32_t lo_n, auto full_tag, auto out_tag) {
     constexpr bool FULL = decltype(full_tag)::value;
+    constexpr int OUT = decltype(out_tag)::value;
     // one real result
     auto put = [&](const float x, const uint32_t mm, const uint32_t nn) {
       if (FULL || (mm < args.m && nn < args.n && mm >= lo_m && nn >= lo_n)) {
         float *cp = cb + ((uint64_t)nn * args.ldc + mm);
-        if (args.atomic_out) {
+        if constexpr (OUT == OUT_ATOMIC) {
           atomicAdd(cp, x * alpha_re);
-        } else if (beta_zero) {
+        } else if constexpr (OUT == OUT_STORE) {
           // the result is not read again by this kernel: streaming store
           __builtin_nontemporal_store(x * alpha_re, cp);
         } else {
@@ -1200,11 +1208,11 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
             const float y = sgn_b * p[2] + sgn_a * p[3];
             float rx = x * alpha_re - y * alpha_im;
             float ry = y * alpha_re + x * alpha_im;
-            if (args.atomic_out) {
+            if constexpr (OUT == OUT_ATOMIC) {
               atomicAdd(cp, rx);
               atomicAdd(cp + 1, ry);
             } else {
-              if (!beta_zero) {
+              if constexpr (OUT == OUT_BETA) {
                 const float2 old = *reinterpret_cast<const float2 *>(cp);
                 rx = x * alpha_re - y * alpha_im +
                      (args.beta_re * old.x - args.beta_im * old.y);
@@ -1219,6 +1227,16 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
           }
         }
       }
+  };
+  auto epilogue = [&](float *cb, const uint32_t em0, const uint32_t en0, const uint32_t lo_m, const uint32_t lo_n,
+                      auto full_tag) {
+    if (args.atomic_out) {
+      epilogue_body(cb, em0, en0, lo_m, lo_n, full_tag, std::integral_constant<int, OUT_ATOMIC>{});
+    } else if (beta_zero) {
+      epilogue_body(cb, em0, en0, lo_m, lo_n, full_tag, std::integral_constant<int, OUT_STORE>{});
+    } else {
+      epilogue_body(cb, em0, en0, lo_m, lo_n, full_tag, std::integral_constant<int, OUT_BETA>{});
+    }
   };
   auto zero_acc = [&]() {
 #pragma unroll
@@ -1335,6 +1353,20 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
       b2 = tmp;
       frag_load(f0, b0, 0);
     };
+    // Workgroups that start together stay together: same tiles, same step time,
+    // so all 256 write their tiles out at the same moment, at a quarter of the
+    // rate a CU stores at when at most 64 of them do (the chip's store rate is
+    // reached by 64 CUs).  Starting the workgroups in four phases, neighbours
+    // on an XCD in different ones, lets a quarter of the chip write while the
+    // rest multiplies; the phases persist, every workgroup having the same period.
+    if (args.stagger_clocks != 0) {
+      const uint64_t wait_clocks = (uint64_t)((blockIdx.x >> 3) & 3u) * args.stagger_clocks;
+      if (wave == 0) {
+        const uint64_t t0 = __builtin_readcyclecounter();
+        while (__builtin_readcyclecounter() - t0 < wait_clocks) __builtin_amdgcn_s_sleep(32);
+      }
+      __syncthreads();
+    }
     dma_next(0);
     dma_next(1);
     __builtin_amdgcn_s_waitcnt(0);
