@@ -1142,10 +1142,32 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
                            const uint32_t lo_n, auto full_tag, auto out_tag) {
     constexpr bool FULL = decltype(full_tag)::value;
     constexpr int OUT = decltype(out_tag)::value;
+    // Addresses: every lane keeps the 64-bit address of the first result it
+    // holds (row lane_m, column lane_n of C); every other result of the lane is
+    // dm rows and dn columns further on, the same dm, dn for all lanes and
+    // known at compile time, so that its address is that base plus a wave-uniform
+    // offset -- one 64-bit vector add per column instead of a 64-bit multiply by
+    // ldc per element.
+    //   16x16 blocks, real (after the lane swap below): lane l holds rows l % 32, columns 8 * (l / 32) + ...
+    //   32x32 blocks: rows l % 32, columns 4 * (l / 32) + ...;  16x16, complex: rows l % 16, columns 4 * (l / 16) + ...
+    constexpr bool SWAPPED = !CPLX && MT == 16;
+    const uint32_t lane_m = em0 + wm * Cfg::WM + (SWAPPED ? (lane & 31) : (lane & (MT - 1)));
+    const uint32_t lane_n = en0 + wn * Cfg::WN + (SWAPPED ? 8 * (lane >> 5) : 4 * (lane / MT));
+    float *const lane_base = cb + ((uint64_t)lane_n * args.ldc + lane_m) * ES;
+    // (taken by the kernels over pre-split operands; the kernels that split in the K loop are at their
+    // register limit and measure 2 - 4 % slower with the extra base address live: they multiply per element)
+    auto address = [&](const int dm, const int dn) {
+      if constexpr (Cfg::PACKED) return lane_base + ((uint64_t)dn * args.ldc + (uint64_t)dm) * ES;
+      else return cb + ((uint64_t)(lane_n + dn) * args.ldc + (lane_m + dm)) * ES;
+    };
+    auto inside = [&](const int dm, const int dn) {
+      const uint32_t mm = lane_m + dm, nn = lane_n + dn;
+      return FULL || (mm < args.m && nn < args.n && mm >= lo_m && nn >= lo_n);
+    };
     // one real result
-    auto put = [&](const float x, const uint32_t mm, const uint32_t nn) {
-      if (FULL || (mm < args.m && nn < args.n && mm >= lo_m && nn >= lo_n)) {
-        float *cp = cb + ((uint64_t)nn * args.ldc + mm);
+    auto put = [&](const float x, const int dm, const int dn) {
+      if (inside(dm, dn)) {
+        float *cp = address(dm, dn);
         if constexpr (OUT == OUT_ATOMIC) {
           atomicAdd(cp, x * alpha_re);
         } else if constexpr (OUT == OUT_STORE) {
@@ -1161,7 +1183,7 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
       if constexpr (PT::NACC == 2) x += acc[0][1][j][i][v] * PT::CORR_SCALE;
       return x;
     };
-    if constexpr (!CPLX && MT == 16) {
+    if constexpr (SWAPPED) {
       static_assert(TN * (TM / 2) * 4 * 2 == EPI_VMEM, "stores of the write-out");
       // Two neighbouring row blocks trade their odd / even 16-lane rows, after
       // which register v of lane l holds column 4*(2*(l/32) + w) + v, row l%32
@@ -1171,14 +1193,12 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
       for (int j = 0; j < TN; j++)
 #pragma unroll
         for (int i = 0; i < TM; i += 2) {
-          const uint32_t mm = em0 + wm * Cfg::WM + i * 16 + (lane & 31);
 #pragma unroll
           for (int v = 0; v < 4; v++) {
             const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(real_value(j, i, v)),
                                                             __float_as_uint(real_value(j, i + 1, v)), false, false);
 #pragma unroll
-            for (int w = 0; w < 2; w++)
-              put(__uint_as_float(r[w]), mm, en0 + wn * Cfg::WN + j * 16 + 4 * (2 * (lane >> 5) + w) + v);
+            for (int w = 0; w < 2; w++) put(__uint_as_float(r[w]), i * 16, j * 16 + 4 * w + v);
           }
         }
       return;
@@ -1187,15 +1207,13 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
     for (int j = 0; j < TN; j++)
 #pragma unroll
       for (int i = 0; i < TM; i++) {
-        const uint32_t mm = em0 + wm * Cfg::WM + i * MT + (lane & (MT - 1));
 #pragma unroll
         for (int v = 0; v < NV; v++) {
-          const uint32_t nn = en0 + wn * Cfg::WN + j * MT +
-                              (MT == 32 ? 8 * (v / 4) + 4 * (lane >> 5) + (v & 3) : 4 * (lane >> 4) + v);
+          const int dm = i * MT, dn = j * MT + (MT == 32 ? 8 * (v / 4) + (v & 3) : v);
           if constexpr (!CPLX) {
-            put(real_value(j, i, v), mm, nn);
-          } else if (FULL || (mm < args.m && nn < args.n && mm >= lo_m && nn >= lo_n)) {
-            float *cp = cb + ((uint64_t)nn * args.ldc + mm) * ES;
+            put(real_value(j, i, v), dm, dn);
+          } else if (inside(dm, dn)) {
+            float *cp = address(dm, dn);
             // re = ar*br - sa*sb*ai*bi, im = sb*ar*bi + sa*ai*br with
             // sa (sb) = -1 when op(A) (op(B)) conjugates
             float p[4];
