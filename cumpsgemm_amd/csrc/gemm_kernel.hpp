@@ -1164,8 +1164,20 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
       const uint32_t mm = lane_m + dm, nn = lane_n + dn;
       return FULL || (mm < args.m && nn < args.n && mm >= lo_m && nn >= lo_n);
     };
+    // C = x + beta * C: the old values of a group of results are fetched first,
+    // all loads in flight together, then the group is combined and stored.  (One
+    // element at a time, every load would have to wait for the store before it,
+    // which the compiler cannot tell apart from it, and every store for its load:
+    // a round trip to memory per element.)
+    auto old_value = [&](const int dm, const int dn) {
+      float o = 0.0f;
+      if constexpr (OUT == OUT_BETA) {
+        if (inside(dm, dn)) o = *address(dm, dn);
+      }
+      return o;
+    };
     // one real result
-    auto put = [&](const float x, const int dm, const int dn) {
+    auto put = [&](const float x, const float old, const int dm, const int dn) {
       if (inside(dm, dn)) {
         float *cp = address(dm, dn);
         if constexpr (OUT == OUT_ATOMIC) {
@@ -1174,7 +1186,7 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
           // the result is not read again by this kernel: streaming store
           __builtin_nontemporal_store(x * alpha_re, cp);
         } else {
-          *cp = x * alpha_re + args.beta_re * (*cp);
+          *cp = x * alpha_re + args.beta_re * old;
         }
       }
     };
@@ -1190,7 +1202,14 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
       // of the block pair (w = 0, 1: the first / second register of the pair):
       // 32 lanes write 128 contiguous bytes, as with the 32x32 blocks.
 #pragma unroll
-      for (int j = 0; j < TN; j++)
+      for (int j = 0; j < TN; j++) {
+        float old[TM / 2][4][2];
+#pragma unroll
+        for (int i = 0; i < TM; i += 2)
+#pragma unroll
+          for (int v = 0; v < 4; v++)
+#pragma unroll
+            for (int w = 0; w < 2; w++) old[i / 2][v][w] = old_value(i * 16, j * 16 + 4 * w + v);
 #pragma unroll
         for (int i = 0; i < TM; i += 2) {
 #pragma unroll
@@ -1198,21 +1217,56 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
             const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(real_value(j, i, v)),
                                                             __float_as_uint(real_value(j, i + 1, v)), false, false);
 #pragma unroll
-            for (int w = 0; w < 2; w++) put(__uint_as_float(r[w]), i * 16, j * 16 + 4 * w + v);
+            for (int w = 0; w < 2; w++) put(__uint_as_float(r[w]), old[i / 2][v][w], i * 16, j * 16 + 4 * w + v);
           }
         }
+      }
       return;
     }
 #pragma unroll
     for (int j = 0; j < TN; j++)
 #pragma unroll
       for (int i = 0; i < TM; i++) {
+        auto offsets = [&](const int v, int &dm, int &dn) {
+          dm = i * MT;
+          dn = j * MT + (MT == 32 ? 8 * (v / 4) + (v & 3) : v);
+        };
+        // (groups of four: the kernels that split in the K loop have no registers to spare)
+        if constexpr (!CPLX) {
 #pragma unroll
-        for (int v = 0; v < NV; v++) {
-          const int dm = i * MT, dn = j * MT + (MT == 32 ? 8 * (v / 4) + (v & 3) : v);
-          if constexpr (!CPLX) {
-            put(real_value(j, i, v), dm, dn);
-          } else if (inside(dm, dn)) {
+          for (int g = 0; g < NV; g += 4) {
+            float old[4];
+#pragma unroll
+            for (int v = g; v < g + 4; v++) {
+              int dm, dn;
+              offsets(v, dm, dn);
+              old[v - g] = old_value(dm, dn);
+            }
+#pragma unroll
+            for (int v = g; v < g + 4; v++) {
+              int dm, dn;
+              offsets(v, dm, dn);
+              put(real_value(j, i, v), old[v - g], dm, dn);
+            }
+          }
+        } else {
+#pragma unroll
+          for (int g = 0; g < NV; g += 4) {
+          float2 old[4];
+          if constexpr (OUT == OUT_BETA) {
+#pragma unroll
+            for (int v = g; v < g + 4; v++) {
+              int dm, dn;
+              offsets(v, dm, dn);
+              old[v - g] = make_float2(0.0f, 0.0f);
+              if (inside(dm, dn)) old[v - g] = *reinterpret_cast<const float2 *>(address(dm, dn));
+            }
+          }
+#pragma unroll
+          for (int v = g; v < g + 4; v++) {
+            int dm, dn;
+            offsets(v, dm, dn);
+            if (!inside(dm, dn)) continue;
             float *cp = address(dm, dn);
             // re = ar*br - sa*sb*ai*bi, im = sb*ar*bi + sa*ai*br with
             // sa (sb) = -1 when op(A) (op(B)) conjugates
@@ -1231,17 +1285,15 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
               atomicAdd(cp + 1, ry);
             } else {
               if constexpr (OUT == OUT_BETA) {
-                const float2 old = *reinterpret_cast<const float2 *>(cp);
-                rx = x * alpha_re - y * alpha_im +
-                     (args.beta_re * old.x - args.beta_im * old.y);
-                ry = y * alpha_re + x * alpha_im +
-                     (args.beta_im * old.x + args.beta_re * old.y);
+                rx = x * alpha_re - y * alpha_im + (args.beta_re * old[v - g].x - args.beta_im * old[v - g].y);
+                ry = y * alpha_re + x * alpha_im + (args.beta_im * old[v - g].x + args.beta_re * old[v - g].y);
               }
               // the result is not read again by this kernel: streaming store
               typedef float f2v_t __attribute__((ext_vector_type(2)));
               f2v_t out2 = {rx, ry};
               __builtin_nontemporal_store(out2, reinterpret_cast<f2v_t *>(cp));
             }
+          }
           }
         }
       }
