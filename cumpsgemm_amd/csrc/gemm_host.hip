@@ -368,8 +368,10 @@ PreSplitChoice choose_pre_split(const cuMpSGEMM_handle *h, bool a_kc, bool b_kc,
   const bool shape_ok = batch == 1 && k >= 128 &&
                         (forced || (uint64_t)m * n >= (uint64_t)h->num_cus * ch.bm * ch.bn) && k / 32 < 65535;
   const double mn_ratio = (double)m * (double)n / ((double)m + (double)n);
-  // (K = 256: 6144^2 + 8 %, 4096^2 - 4 %)
-  const bool pays_nt_shape = !a_kc && !b_kc && ((k >= 512 && mn_ratio >= 1800.0) || (k >= 256 && mn_ratio >= 2800.0));
+  // (in-loop -> pre-split, TFLOP/s: 4096^2 x 256 198 -> 211, 4096^2 x 384 224 -> 260, 5120^2 x 256 176 -> 209,
+  // 3072^2 x 512 177 -> 191, 3072^2 x 1024 201 -> 237, 8192 x 4096 x 256 211 -> 245, 4096 x 8192 x 384 232 -> 316;
+  // 3072^2 x 2048 level)
+  const bool pays_nt_shape = !a_kc && !b_kc && ((k >= 384 && mn_ratio >= 1500.0) || (k >= 256 && mn_ratio >= 2000.0));
   // Every other layout: the pre-split kernel, freed of the split arithmetic,
   // outruns the in-loop one by more than the pre-pass costs once the problem
   // is large (8192^3: 381 vs 361 - 372 TFLOP/s; 8192^2 x 1024: 351 vs 318 -
@@ -405,14 +407,20 @@ PreSplitChoice choose_pre_split(const cuMpSGEMM_handle *h, bool a_kc, bool b_kc,
     // 8192^2 x 384 287 / 297 -> 314 / 313, 6144^2 x 384 254 / 266 -> 280 / 282, 6144^2 x 512 274 / 285 -> 306 / 307,
     // 4096^2 x 1024 326 / 333 -> 343 / 343, 4096^2 x 2048 350 / 357 -> 384 / 384; 6144^2 x 256 and 4096^2 x 512
     // are level and stay in-loop, 4096^2 x 256 would lose 8 - 11 %).
+    // (re-measured with the cheaper write-out of the pre-split kernels, NN / TN, packed over in-loop: 4096^2 x 384
+    // 1.00 / 0.99, 4096 x 8192 x 384 1.12 / 1.14, 6144^2 x 384 1.06 / 1.04, 4096^2 x 512 1.01 / 1.01, 4096^2 x 768
+    // 1.08 / 1.07, 6144^2 x 256 1.06 / 1.01, 8192 x 4096 x 256 0.96 / 0.95, 5120^2 x 256 0.91 / 0.90)
     const bool pays_short = !CPLX && ro &&
-                            ((k >= 256 && mn_ratio >= 4000.0) || (k >= 384 && mn_ratio >= 3000.0) ||
-                             (k >= 1024 && mn_ratio >= 2000.0));
+                            ((k >= 256 && mn_ratio >= 4000.0) || (k >= 384 && mn_ratio >= 2500.0) ||
+                             (k >= 768 && mn_ratio >= 2000.0));
     // (complex, in-loop -> pre-split, NN / TN: 4096^3 367 / 378 -> 432 / 435 TFLOP/s, 2048^3 355 / 364 -> 401 / 400,
     // 2048^2 x 1024 349 / 347 -> 372 / 374, 3072^2 x 384 309 / 314 -> 329 / 325, 4096^2 x 256 313 / 320 -> 342 / 349,
     // 8192^2 x 256 323 / 321 -> 368 / 373; 2048^2 x 512 level, 2048^2 x 384 would lose 5 %, 3072^2 x 256 level)
-    const bool pays_cplx = ro && ((k >= 256 && mn_ratio >= 2000.0) || (k >= 384 && mn_ratio >= 1500.0) ||
-                                  (k >= 1024 && mn_ratio >= 1000.0));
+    // (re-measured with the cheaper write-out, packed over in-loop, NN / TN / NT: 2048^2 x 512 1.03 / 1.02 / 1.10,
+    // 2048^2 x 768 1.06 / 1.04 / 1.06, 2560^2 x 384 1.03 / 1.05 / 1.09, 3072^2 x 256 1.03 / 1.03 / 1.05; 2048^2 x 384
+    // 0.98 / 0.95 / 1.03, 2560^2 x 256 0.96 / 0.97 / 1.00, 1536^2 x 2048 0.94 / 0.91 / 1.02 stay in-loop)
+    const bool pays_cplx = ro && ((k >= 256 && mn_ratio >= 1500.0) || (k >= 384 && mn_ratio >= 1250.0) ||
+                                  (k >= 512 && mn_ratio >= 1000.0));
     const bool pays = CPLX ? pays_cplx : (pays_nt || pays_short);
     // The uncorrected modes issue a third (FP16TC) or as many (bf16x2) MFMAs per
     // element as FP16TCEC, so the same pre-pass weighs three times as much for
