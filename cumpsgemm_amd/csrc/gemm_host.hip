@@ -193,15 +193,24 @@ unsigned resident_groups(const KernelEntry *e) {
 // small outputs (src/cumpsgemm.cu:242-253, x32 for batches :453-454).  Here
 // every (class, split) pair gets a cost from a small model fitted to
 // measurements on MI355X, and the cheapest wins:
-//   cost = rounds * (K-steps per chunk + 4) * tile area * resident groups / efficiency
+//   cost = rounds * (K-steps per chunk + F) * tile area * resident groups / efficiency
 //          [+ a fixed charge when K is split]
 // rounds     = how many times the chip's CU slots must be refilled (a problem
 //              smaller than one round is charged for the workgroups a CU
 //              really holds),
-// + 4        = a tile's fixed cost (pipeline fill, write-out) in K-steps,
+// + F        = a tile's fixed cost (pipeline fill, write-out) in K-steps: 5 for
+//              the 256x128 tiles, 3 for 128x128, 4 for the others,
 // efficiency = sustained MFMA rate relative to the 64x64 wave tile, which has
 //              the fewest LDS fragment reads per MFMA (64x32: 0.83, 32x32: 0.55,
-//              less when a CU holds under two waves per SIMD),
+//              less when a CU holds under two waves per SIMD; the 128x256 tile of
+//              the layout with both operands M/N-contiguous: 0.85),
+// (F and the 0.85 were fitted on 34 shapes x 3 layouts x {FP16TCEC, bf16x3}, single
+// and strided-batch, each timed with every class forced: with F = 4 throughout the
+// model kept the large tile for batches of small matrices and for K <= 256,
+// where 128x128 measures 5 - 30 % faster -- 384^3 x 128 201 -> 226, 4096^2 x 128
+// 162 -> 175, 768^3 x 32 NT 199 -> 240, bf16x3 512^2 x 128 x 128 116 -> 131 TFLOP/s;
+// the sum of the relative losses against the best class fell from 2.6 to 0.73
+// (FP16TCEC) and from 3.8 to 1.2 (bf16x3).)
 // split charge = the extra launch that prepares C (about four K-steps of the
 //              largest tile) plus the atomic write-out, which grows with the
 //              number of chunks adding into the same C.
@@ -229,8 +238,9 @@ Plan make_plan(const cuMpSGEMM_handle *h, Prec p, bool cplx, bool a_kc, bool b_k
     // efficiency with `groups` workgroups on a CU: the 32x32 wave tiles need
     // two waves per SIMD to hide their own latencies (0.52 us per K-step for a
     // lone 4-wave 64x64 workgroup, 0.65 us for two of them side by side)
+    const bool transposed_large = !a_kc && !b_kc && e->bm == 128 && e->bn == 256;
     auto eff_of = [&](double groups) {
-      if (wave_area >= 4096) return 1.0;
+      if (wave_area >= 4096) return transposed_large ? 0.85 : 1.0;
       if (wave_area >= 2048) return 0.83;
       const double waves_per_simd = (double)e->threads * groups / 256.0;
       return waves_per_simd >= 2.0 ? 0.55 : (waves_per_simd >= 1.0 ? 0.375 : 0.19);
@@ -238,6 +248,8 @@ Plan make_plan(const cuMpSGEMM_handle *h, Prec p, bool cplx, bool a_kc, bool b_k
     // (a tile's operand traffic per flop grows with 1/bm + 1/bn: charged lightly,
     // which also settles ties in favour of the larger tile)
     const double area = (double)e->bm * e->bn * (1.0 + 2.0 / e->bm + 2.0 / e->bn);
+    const int tile_elems = e->bm * e->bn;
+    const double fixed_steps = tile_elems >= 256 * 128 ? 5.0 : (tile_elems >= 128 * 128 ? 3.0 : 4.0);
     const double unit = area * res / eff_of((double)res);
     const double atomics = (double)m * (double)n * (double)batch * (cplx ? 2.0 : 1.0);
     for (uint64_t sp = 1; sp <= max_split; sp *= 2) {
@@ -245,7 +257,7 @@ Plan make_plan(const cuMpSGEMM_handle *h, Prec p, bool cplx, bool a_kc, bool b_k
       // a problem that does not fill the CU slots once keeps fewer workgroups on
       // a CU than could live there; otherwise whole rounds are charged
       const uint64_t groups = tiles * sp;
-      const double steps = (double)((nk + sp - 1) / sp) + 4.0;
+      const double steps = (double)((nk + sp - 1) / sp) + fixed_steps;
       double cost;
       if (groups < slots) {
         const double per_cu = (double)((groups + h->num_cus - 1) / h->num_cus);
