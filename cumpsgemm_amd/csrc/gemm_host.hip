@@ -32,6 +32,7 @@ Tuning read_tuning_env() {
   t.force_split = as_int("CUMPSGEMM_FORCE_KSPLIT", 0);
   t.no_persistent = std::getenv("CUMPSGEMM_NO_PERSISTENT") != nullptr;
   t.no_column_split = std::getenv("CUMPSGEMM_NO_COLUMN_SPLIT") != nullptr;
+  t.cut_percent = as_int("CUMPSGEMM_CUT_PERCENT", t.cut_percent);
   t.no_kslices = std::getenv("CUMPSGEMM_NO_KSLICE_GROUPS") != nullptr;
   t.no_fused_scaling = std::getenv("CUMPSGEMM_NO_FUSED_SCALING") != nullptr;
   if (const char *v = std::getenv("CUMPSGEMM_PERSISTENT_MAX_STEPS")) t.persistent_max_steps = (unsigned)std::atoi(v);
@@ -199,18 +200,23 @@ unsigned resident_groups(const KernelEntry *e) {
 //              smaller than one round is charged for the workgroups a CU
 //              really holds),
 // + F        = a tile's fixed cost (pipeline fill, write-out) in K-steps: 5 for
-//              the 256x128 tiles, 3 for 128x128, 4 for the others,
+//              the 256x128 tiles, 3 for 128x128, 4 for the others (FP16TC, a
+//              third of the MFMAs per step: 4 throughout; complex: 3 for 128x64,
+//              4 for the others),
 // efficiency = sustained MFMA rate relative to the 64x64 wave tile, which has
 //              the fewest LDS fragment reads per MFMA (64x32: 0.83, 32x32: 0.55,
 //              less when a CU holds under two waves per SIMD; the 128x256 tile of
-//              the layout with both operands M/N-contiguous: 0.85),
+//              the layout with both operands M/N-contiguous: 0.85; the complex
+//              64x64 and 64x32 tiles, which are not persistent: x 0.8),
 // (F and the 0.85 were fitted on 34 shapes x 3 layouts x {FP16TCEC, bf16x3}, single
 // and strided-batch, each timed with every class forced: with F = 4 throughout the
 // model kept the large tile for batches of small matrices and for K <= 256,
 // where 128x128 measures 5 - 30 % faster -- 384^3 x 128 201 -> 226, 4096^2 x 128
 // 162 -> 175, 768^3 x 32 NT 199 -> 240, bf16x3 512^2 x 128 x 128 116 -> 131 TFLOP/s;
 // the sum of the relative losses against the best class fell from 2.6 to 0.73
-// (FP16TCEC) and from 3.8 to 1.2 (bf16x3).)
+// (FP16TCEC) and from 3.8 to 1.2 (bf16x3); complex FP16TCEC 1.3 -> 0.53 -- 320^3 x 256
+// 208 -> 250, 1024^2 x 4096 NT 221 -> 283 TFLOP/s --, complex bf16x3 0.73 -> 0.06;
+// FP16TC fits best with what it had.)
 // split charge = the extra launch that prepares C (about four K-steps of the
 //              largest tile) plus the atomic write-out, which grows with the
 //              number of chunks adding into the same C.
@@ -239,17 +245,21 @@ Plan make_plan(const cuMpSGEMM_handle *h, Prec p, bool cplx, bool a_kc, bool b_k
     // two waves per SIMD to hide their own latencies (0.52 us per K-step for a
     // lone 4-wave 64x64 workgroup, 0.65 us for two of them side by side)
     const bool transposed_large = !a_kc && !b_kc && e->bm == 128 && e->bn == 256;
+    const int tile_elems = e->bm * e->bn;
+    const bool cplx_large = cplx && tile_elems >= 128 * 64;
+    const double fixed_steps = cplx ? (cplx_large ? 3.0 : 4.0)
+                               : (p == Prec::FP16TC ? 4.0
+                                  : (tile_elems >= 256 * 128 ? 5.0 : (tile_elems >= 128 * 128 ? 3.0 : 4.0)));
+    const double small_cplx = (cplx && !cplx_large) ? 0.8 : 1.0;
     auto eff_of = [&](double groups) {
       if (wave_area >= 4096) return transposed_large ? 0.85 : 1.0;
       if (wave_area >= 2048) return 0.83;
       const double waves_per_simd = (double)e->threads * groups / 256.0;
-      return waves_per_simd >= 2.0 ? 0.55 : (waves_per_simd >= 1.0 ? 0.375 : 0.19);
+      return small_cplx * (waves_per_simd >= 2.0 ? 0.55 : (waves_per_simd >= 1.0 ? 0.375 : 0.19));
     };
     // (a tile's operand traffic per flop grows with 1/bm + 1/bn: charged lightly,
     // which also settles ties in favour of the larger tile)
     const double area = (double)e->bm * e->bn * (1.0 + 2.0 / e->bm + 2.0 / e->bn);
-    const int tile_elems = e->bm * e->bn;
-    const double fixed_steps = tile_elems >= 256 * 128 ? 5.0 : (tile_elems >= 128 * 128 ? 3.0 : 4.0);
     const double unit = area * res / eff_of((double)res);
     const double atomics = (double)m * (double)n * (double)batch * (cplx ? 2.0 : 1.0);
     for (uint64_t sp = 1; sp <= max_split; sp *= 2) {
@@ -822,7 +832,17 @@ hipblasStatus_t run_gemm(cuMpSGEMM_handle *h, hipblasOperation_t op_A,
     }
     const bool by_rows = cost_rows >= 0.0 && (cost_cols < 0.0 || cost_rows < cost_cols);
     const double cost_cut = by_rows ? cost_rows : cost_cols;
-    if (cost_cut >= 0.0 && cost_cut < 0.93 * plan0.cost) return run_cut(by_rows, m1, n1, 1);
+    // How far below the uncut plan the model must price the two parts.  Measured
+    // against the model on 15 shapes per kind with the cut forced and forbidden
+    // (ratio of the two times): real kernels run 0.00 - 0.08 above the model's
+    // ratio, complex FP16TCEC within 0.03 of it, and complex bf16x3 -- whose
+    // large tile is the one kernel of a table that does not walk its tiles --
+    // 0.15 - 0.23 below it (1536^3: model 0.94, measured 0.73; 1600^2 x 800: 1.09, 0.91;
+    // 1920^2 x 384: 1.21, 1.03).
+    const int cut_percent = tuning().cut_percent > 0
+                                ? tuning().cut_percent
+                                : (CPLX ? (launches[0].p == Prec::BF16X3 ? 110 : 96) : 93);
+    if (cost_cut >= 0.0 && cost_cut < 0.01 * cut_percent * plan0.cost) return run_cut(by_rows, m1, n1, 1);
   }
 
   if (split) {

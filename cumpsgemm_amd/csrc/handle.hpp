@@ -77,6 +77,8 @@ struct Tuning {
   int force_split = 0;  // CUMPSGEMM_FORCE_KSPLIT
   bool no_persistent = false;    // CUMPSGEMM_NO_PERSISTENT
   bool no_column_split = false;  // CUMPSGEMM_NO_COLUMN_SPLIT
+  int cut_percent = -1;          // CUMPSGEMM_CUT_PERCENT: C is cut when the model prices the two parts below this
+                                 // share of the uncut plan (unset: 93, complex 96, complex bf16x3 110)
   bool no_kslices = false;       // CUMPSGEMM_NO_KSLICE_GROUPS
   bool no_fused_scaling = false; // CUMPSGEMM_NO_FUSED_SCALING
   unsigned persistent_max_steps = 32; // CUMPSGEMM_PERSISTENT_MAX_STEPS
