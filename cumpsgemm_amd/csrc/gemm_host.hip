@@ -216,7 +216,10 @@ unsigned resident_groups(const KernelEntry *e) {
 // the sum of the relative losses against the best class fell from 2.6 to 0.73
 // (FP16TCEC) and from 3.8 to 1.2 (bf16x3); complex FP16TCEC 1.3 -> 0.53 -- 320^3 x 256
 // 208 -> 250, 1024^2 x 4096 NT 221 -> 283 TFLOP/s --, complex bf16x3 0.73 -> 0.06;
-// FP16TC fits best with what it had.)
+// FP16TC fits best with what it had; the 256x128 kernel of bf16x2 that splits in the
+// K loop loses to its 128x128 one on every shape of the sweep, also where both
+// fill the chip evenly -- 4096^2 x 512 215 against 250, 512^3 x 64 213 against 244 --:
+// 0.7, sum of losses 6.0 -> 0.6.)
 // split charge = the extra launch that prepares C (about four K-steps of the
 //              largest tile) plus the atomic write-out, which grows with the
 //              number of chunks adding into the same C.
@@ -252,7 +255,7 @@ Plan make_plan(const cuMpSGEMM_handle *h, Prec p, bool cplx, bool a_kc, bool b_k
                                   : (tile_elems >= 256 * 128 ? 5.0 : (tile_elems >= 128 * 128 ? 3.0 : 4.0)));
     const double small_cplx = (cplx && !cplx_large) ? 0.8 : 1.0;
     auto eff_of = [&](double groups) {
-      if (wave_area >= 4096) return transposed_large ? 0.85 : 1.0;
+      if (wave_area >= 4096) return transposed_large ? 0.85 : (p == Prec::BF16X2 ? 0.7 : 1.0);
       if (wave_area >= 2048) return 0.83;
       const double waves_per_simd = (double)e->threads * groups / 256.0;
       return small_cplx * (waves_per_simd >= 2.0 ? 0.55 : (waves_per_simd >= 1.0 ? 0.375 : 0.19));
