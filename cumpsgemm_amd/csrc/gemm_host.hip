@@ -26,7 +26,6 @@ Tuning read_tuning_env() {
   const int rg = as_int("CUMPSGEMM_RASTER_GROUP", 0);
   t.raster_group = (rg >= 1 && rg <= 64) ? rg : 0;
   t.fetch_from_one_patch = std::getenv("CUMPSGEMM_EXP_FETCH_FROM_ONE_PATCH") != nullptr;
-  t.walk_stagger = as_int("CUMPSGEMM_WALK_STAGGER", -1);
   t.force_cls = as_int("CUMPSGEMM_FORCE_TILE_CLASS", -1);
   if (t.force_cls < 0 || t.force_cls >= kNumTileClasses) t.force_cls = -1;
   t.force_split = as_int("CUMPSGEMM_FORCE_KSPLIT", 0);
@@ -599,7 +598,6 @@ PreSplit run_pre_split(cuMpSGEMM_handle *h, const GemmArgs &args, bool a_kc, boo
     if (tuning().packed_walk >= 0) walk = tuning().packed_walk == 1;
     if (kind == PackKind::BF16X3_COMPLEX) walk = false; // (its kernel has the one-tile form only)
     if (walk && tuning().fetch_from_one_patch) pargs.raster_group |= kFetchFromOnePatch; // (profiler experiment)
-    pargs.stagger_clocks = (walk && tuning().walk_stagger > 0) ? (uint32_t)tuning().walk_stagger : 0u;
     const dim3 grid = walk ? dim3((unsigned)std::min<uint64_t>(total, h->num_cus), 1, 1)
                            : dim3((unsigned)total, 1, 1);
     launch_kernel(pargs, grid, walk);

@@ -128,9 +128,6 @@ struct GemmArgs {
   // flag -- so that no host synchronisation is needed.
   const uint32_t *scale_max_a, *scale_max_b; // bits of 2^floor(log2 max|x|)
   const int *scale_flag;                     // bit 6: scale A, bit 5: scale B
-  // Tile-walking pre-split kernel: workgroup w starts (w / 8 mod 4) * stagger_clocks
-  // shader clocks late (0: all together), see there.
-  uint32_t stagger_clocks;
 #if CUMPSGEMM_WALK_STAMPS
   unsigned long long *stamps; // 2 x 512 words: [count, stamps...] of workgroups 0 and 101
 #endif
@@ -1423,20 +1420,6 @@ __attribute__((amdgpu_waves_per_eu(Cfg::OCC, Cfg::OCC))) void gemm_tcec_kernel(c
       b2 = tmp;
       frag_load(f0, b0, 0);
     };
-    // Workgroups that start together stay together: same tiles, same step time,
-    // so all 256 write their tiles out at the same moment, at a quarter of the
-    // rate a CU stores at when at most 64 of them do (the chip's store rate is
-    // reached by 64 CUs).  Starting the workgroups in four phases, neighbours
-    // on an XCD in different ones, lets a quarter of the chip write while the
-    // rest multiplies; the phases persist, every workgroup having the same period.
-    if (args.stagger_clocks != 0) {
-      const uint64_t wait_clocks = (uint64_t)((blockIdx.x >> 3) & 3u) * args.stagger_clocks;
-      if (wave == 0) {
-        const uint64_t t0 = __builtin_readcyclecounter();
-        while (__builtin_readcyclecounter() - t0 < wait_clocks) __builtin_amdgcn_s_sleep(32);
-      }
-      __syncthreads();
-    }
     dma_next(0);
     dma_next(1);
     __builtin_amdgcn_s_waitcnt(0);

@@ -70,9 +70,6 @@ struct Tuning {
   // tile-walking pre-split kernel reads every tile's operands from one
   // L2-resident patch, which shows what its operand traffic over the fabric costs
   bool fetch_from_one_patch = false;
-  // CUMPSGEMM_WALK_STAGGER: shader clocks between the four start phases of the
-  // tile-walking pre-split kernel's workgroups (-1: the built-in rule, 0: none)
-  int walk_stagger = -1;
   int force_cls = -1;   // CUMPSGEMM_FORCE_TILE_CLASS
   int force_split = 0;  // CUMPSGEMM_FORCE_KSPLIT
   bool no_persistent = false;    // CUMPSGEMM_NO_PERSISTENT
