@@ -735,3 +735,28 @@ def test_seeded_random_shapes_all_paths(O, handle, dev):
         beta = 0.0 if rng.integers(0, 3) == 0 else (complex(rng.normal(), rng.normal()) if cplx else float(rng.normal()))
         pads = tuple(int(x) for x in rng.integers(0, 4, 3))
         _check(O, handle, dev, mode, opa, opb, m, n, k, cplx, alpha, beta, pads=pads, seed=1000 + case)
+
+
+# ---- the planner's choices ------------------------------------------------------
+# The tile class behind a call is reported as the module id (class, + 100 with K split,
+# 200 for the pre-split path).  These shapes sit where the cost model was fitted on
+# timings of every class: short K and the layout with both operands M/N-contiguous
+# take the 128x128 class although the 256x128 one fills the chip, a long-K complex
+# product keeps the 128x64 tile with K split, and a tile count just above one round
+# of CUs is cut in two (the reported id is that of the second part).
+@pytest.mark.parametrize("mode,cplx,opa,opb,m,n,k,expected", [
+    (FP16TCEC, False, N, N, 4096, 4096, 128, (1,)),
+    (FP16TCEC, False, N, T, 2560, 2560, 512, (1,)),
+    (FP16TCEC, False, N, N, 2560, 2560, 512, (0,)),
+    (TF32TCEC, False, N, N, 4096, 4096, 128, (1,)),
+    (TF32TC, False, N, T, 2560, 2560, 512, (1,)),
+    (FP16TCEC, True, N, T, 1024, 1024, 4096, (0, 100)),
+])
+def test_planner_takes_the_class_the_sweeps_found_best(handle, dev, mode, cplx, opa, opb, m, n, k, expected):
+    gen = _gen(cplx)
+    a, lda = make_operand(gen, 41, opa, m, k, 0)
+    b, ldb = make_operand(gen, 42, opb, k, n, 0)
+    c0 = gen(43, m * n)
+    c, st, mid = run_gemm(handle, dev, mode, opa, opb, m, n, k, 1.0, a, lda, b, ldb, 0.0, c0, m, cplx,
+                          want_module_id=True)
+    assert st == 0 and mid in expected, mid
