@@ -201,13 +201,14 @@ unsigned resident_groups(const KernelEntry *e) {
 // + F        = a tile's fixed cost (pipeline fill, write-out) in K-steps: 5 for
 //              the 256x128 tiles, 3 for 128x128, 4 for the others (FP16TC, a
 //              third of the MFMAs per step: 4 throughout; complex: 3 for 128x64,
-//              4 for the others),
+//              4 for the others; the tables whose large tile uses 16x16x32
+//              MFMAs in the K loop: 6 and 4),
 // efficiency = sustained MFMA rate relative to the 64x64 wave tile, which has
 //              the fewest LDS fragment reads per MFMA (64x32: 0.83, 32x32: 0.55,
-//              less when a CU holds under two waves per SIMD; the 128x256 tile of
-//              the layout with both operands M/N-contiguous: 0.85; the complex
-//              64x64 and 64x32 tiles, which are not persistent: x 0.8),
-// (F and the 0.85 were fitted on 34 shapes x 3 layouts x {FP16TCEC, bf16x3}, single
+//              less when a CU holds under two waves per SIMD; the in-loop large
+//              tiles with 16x16x32 MFMAs: 1.1; the complex 64x64 and 64x32
+//              tiles, which are not persistent: x 0.8),
+// (F and the efficiencies were fitted on 34 shapes x 3 layouts x {FP16TCEC, bf16x3}, single
 // and strided-batch, each timed with every class forced: with F = 4 throughout the
 // model kept the large tile for batches of small matrices and for K <= 256,
 // where 128x128 measures 5 - 30 % faster -- 384^3 x 128 201 -> 226, 4096^2 x 128
@@ -215,10 +216,10 @@ unsigned resident_groups(const KernelEntry *e) {
 // the sum of the relative losses against the best class fell from 2.6 to 0.73
 // (FP16TCEC) and from 3.8 to 1.2 (bf16x3); complex FP16TCEC 1.3 -> 0.53 -- 320^3 x 256
 // 208 -> 250, 1024^2 x 4096 NT 221 -> 283 TFLOP/s --, complex bf16x3 0.73 -> 0.06;
-// FP16TC fits best with what it had; the 256x128 kernel of bf16x2 that splits in the
-// K loop loses to its 128x128 one on every shape of the sweep, also where both
-// fill the chip evenly -- 4096^2 x 512 215 against 250, 512^3 x 64 213 against 244 --:
-// 0.7, sum of losses 6.0 -> 0.6.)
+// FP16TC fits best with what it had.  The 256x128 kernels of bf16x2 and the 128x256
+// one of FP16TCEC were then rebuilt on 16x16x32 MFMAs -- bf16x2 512^3 x 64 213 -> 305,
+// 4096^2 x 512 221 -> 310, FP16TCEC NT 1024^3 x 8 256 -> 324 TFLOP/s -- and their
+// tables fitted again: 6 / 4 K-steps, 1.1.)
 // split charge = the extra launch that prepares C (about four K-steps of the
 //              largest tile) plus the atomic write-out, which grows with the
 //              number of chunks adding into the same C.
@@ -246,15 +247,18 @@ Plan make_plan(const cuMpSGEMM_handle *h, Prec p, bool cplx, bool a_kc, bool b_k
     // efficiency with `groups` workgroups on a CU: the 32x32 wave tiles need
     // two waves per SIMD to hide their own latencies (0.52 us per K-step for a
     // lone 4-wave 64x64 workgroup, 0.65 us for two of them side by side)
-    const bool transposed_large = !a_kc && !b_kc && e->bm == 128 && e->bn == 256;
+    // (tables whose large tile multiplies with 16x16x32 MFMAs in the K loop: real bf16x2, and
+    // real FP16TCEC when both operands are M/N-contiguous)
+    const bool edge16_table = !cplx && (p == Prec::BF16X2 || (p == Prec::FP16TCEC && !a_kc && !b_kc));
     const int tile_elems = e->bm * e->bn;
     const bool cplx_large = cplx && tile_elems >= 128 * 64;
     const double fixed_steps = cplx ? (cplx_large ? 3.0 : 4.0)
                                : (p == Prec::FP16TC ? 4.0
-                                  : (tile_elems >= 256 * 128 ? 5.0 : (tile_elems >= 128 * 128 ? 3.0 : 4.0)));
+                                  : (tile_elems >= 256 * 128 ? (edge16_table ? 6.0 : 5.0)
+                                                             : (tile_elems >= 128 * 128 ? (edge16_table ? 4.0 : 3.0) : 4.0)));
     const double small_cplx = (cplx && !cplx_large) ? 0.8 : 1.0;
     auto eff_of = [&](double groups) {
-      if (wave_area >= 4096) return transposed_large ? 0.85 : (p == Prec::BF16X2 ? 0.7 : 1.0);
+      if (wave_area >= 4096) return edge16_table ? 1.1 : 1.0;
       if (wave_area >= 2048) return 0.83;
       const double waves_per_simd = (double)e->threads * groups / 256.0;
       return small_cplx * (waves_per_simd >= 2.0 ? 0.55 : (waves_per_simd >= 1.0 ? 0.375 : 0.19));

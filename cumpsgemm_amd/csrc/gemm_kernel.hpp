@@ -305,12 +305,18 @@ struct GemmCfg {
   static constexpr int NWAVES = TILE_WAVES * (KS2_ ? 2 : 1);
   static constexpr int NT = NWAVES * 64;
   // MFMA block edge, blocks per wave tile, accumulator registers per block
-  // (in-loop kernels measured with edge 16, all sizes and batches: complex
-  // bf16x3 + 5 - 7 % throughout; the others between - 8 % and + 9 % with a mean
-  // of zero, so they keep 32)
+  // (in-loop kernels measured with edge 16 over 34 shapes x 3 layouts, single
+  // and strided-batch, every tile class forced: complex bf16x3 + 5 - 7 %
+  // throughout; the 256x128 kernels of bf16x2, which spill 230 - 260 B per
+  // lane with edge 32 and nothing with 16, x 1.2 - 2.4; the 128x256 kernel of
+  // FP16TCEC for two M/N-contiguous operands + 15 - 35 %; the others between
+  // - 8 % and + 9 % with a mean of zero, so they keep 32)
+  static constexpr bool EDGE16_INLOOP =
+      (P_ == Prec::BF16X3 && CPLX_) || (P_ == Prec::BF16X2 && !CPLX_ && BM_ * BN_ >= 256 * 128) ||
+      (P_ == Prec::FP16TCEC && !CPLX_ && !A_KC_ && !B_KC_ && BM_ == 128 && BN_ == 256);
   static constexpr int MT = PACKED_ ? CUMPSGEMM_MFMA_EDGE_PACKED
-                            : (P_ == Prec::BF16X3 && CPLX_) ? CUMPSGEMM_MFMA_EDGE_PACKED
-                                                            : CUMPSGEMM_MFMA_EDGE_INLOOP;
+                            : EDGE16_INLOOP ? CUMPSGEMM_MFMA_EDGE_PACKED
+                                            : CUMPSGEMM_MFMA_EDGE_INLOOP;
   static_assert(MT == 32 || MT == 16, "MFMA block edge");
   static constexpr int TM = WM / MT, TN = WN / MT;
   static constexpr int NV = MT * MT / 64;

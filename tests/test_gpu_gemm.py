@@ -740,16 +740,16 @@ def test_seeded_random_shapes_all_paths(O, handle, dev):
 # ---- the planner's choices ------------------------------------------------------
 # The tile class behind a call is reported as the module id (class, + 100 with K split,
 # 200 for the pre-split path).  These shapes sit where the cost model was fitted on
-# timings of every class: short K and the layout with both operands M/N-contiguous
-# take the 128x128 class although the 256x128 one fills the chip, a long-K complex
-# product keeps the 128x64 tile with K split, and a tile count just above one round
-# of CUs is cut in two (the reported id is that of the second part).
+# timings of every class: four K-steps take the 128x128 class although the 256x128 one
+# fills the chip, sixteen take the large one (for two M/N-contiguous operands and for
+# bf16x2 that is the kernel on 16x16x32 MFMAs), and a long-K complex product keeps the
+# 128x64 tile with K split.
 @pytest.mark.parametrize("mode,cplx,opa,opb,m,n,k,expected", [
     (FP16TCEC, False, N, N, 4096, 4096, 128, (1,)),
-    (FP16TCEC, False, N, T, 2560, 2560, 512, (1,)),
+    (FP16TCEC, False, N, T, 2560, 2560, 512, (0,)),
     (FP16TCEC, False, N, N, 2560, 2560, 512, (0,)),
     (TF32TCEC, False, N, N, 4096, 4096, 128, (1,)),
-    (TF32TC, False, N, T, 2560, 2560, 512, (1,)),
+    (TF32TC, False, N, T, 2560, 2560, 512, (0,)),
     (FP16TCEC, True, N, T, 1024, 1024, 4096, (0, 100)),
 ])
 def test_planner_takes_the_class_the_sweeps_found_best(handle, dev, mode, cplx, opa, opb, m, n, k, expected):
