@@ -274,7 +274,7 @@ __device__ inline f4v_t mfma_block(const u4_t a, const u4_t b, const f4v_t c) {
 //         shorten the chain LDS read -> MFMA -> split -> LDS write of a step.
 template <Prec P_, bool CPLX_, bool A_KC_, bool B_KC_, int BM_, int BN_, int WM_,
           int WN_, int OCC_ = 1, bool DEEP_ = false, bool PERSIST_ = false, bool SCALED_ = false,
-          bool PACKED_ = false, bool KS2_ = false>
+          bool PACKED_ = false, bool KS2_ = false, bool E16_ = false>
 struct GemmCfg {
   static_assert(!KS2_ || (!DEEP_ && !PACKED_), "K-slice split: two-buffer kernels");
   static constexpr bool KS2 = KS2_;
@@ -289,9 +289,12 @@ struct GemmCfg {
   static_assert(!PERSIST_ || DEEP_, "persistent kernels use the three-buffer pipeline");
   static_assert(!SCALED_ || P_ == Prec::FP16TCEC, "scaling guards the fp16 range only");
   using persistent_type =
-      GemmCfg<P_, CPLX_, A_KC_, B_KC_, BM_, BN_, WM_, WN_, OCC_, DEEP_, DEEP_, SCALED_>;
+      GemmCfg<P_, CPLX_, A_KC_, B_KC_, BM_, BN_, WM_, WN_, OCC_, DEEP_, DEEP_, SCALED_, false, false, E16_>;
   using scaled_type = GemmCfg<P_, CPLX_, A_KC_, B_KC_, BM_, BN_, WM_, WN_, OCC_, DEEP_, PERSIST_,
-                              P_ == Prec::FP16TCEC>;
+                              P_ == Prec::FP16TCEC, false, false, E16_>;
+  // the same kernel on 16x16x32 MFMAs (E16_: asked for by the table)
+  using edge16_type = GemmCfg<P_, CPLX_, A_KC_, B_KC_, BM_, BN_, WM_, WN_, OCC_, DEEP_, PERSIST_, SCALED_,
+                              PACKED_, KS2_, true>;
   static constexpr bool SCALED = SCALED_;
   static constexpr int OCC = OCC_;
   static constexpr bool DEEP = DEEP_;
@@ -315,8 +318,16 @@ struct GemmCfg {
       (P_ == Prec::BF16X3 && CPLX_) || (P_ == Prec::BF16X2 && !CPLX_ && BM_ * BN_ >= 256 * 128) ||
       (P_ == Prec::FP16TCEC && !CPLX_ && !A_KC_ && !B_KC_ && BM_ == 128 && BN_ == 256);
   static constexpr int MT = PACKED_ ? CUMPSGEMM_MFMA_EDGE_PACKED
-                            : EDGE16_INLOOP ? CUMPSGEMM_MFMA_EDGE_PACKED
-                                            : CUMPSGEMM_MFMA_EDGE_INLOOP;
+                            : (EDGE16_INLOOP || E16_) ? CUMPSGEMM_MFMA_EDGE_PACKED
+                                                      : CUMPSGEMM_MFMA_EDGE_INLOOP;
+  // Real FP16TCEC, 256x128, tile-walking: a second instance on 16x16x32 MFMAs for
+  // launches that keep every CU busy.  There the part runs against its power
+  // limit and the 16x16x32 form, which needs less energy per flop, measures
+  // 3 - 9 % faster (512^3 x 64 279 -> 296, 4096^2 x 512 284 -> 301, 256^3 x 512
+  // 222 -> 243 TFLOP/s); on launches that leave CUs idle the clock is higher and
+  // 32x32x16 wins by 4 - 8 % (2304^2 x 768 242 -> 223).
+  static constexpr bool HAS_EDGE16_TWIN = P_ == Prec::FP16TCEC && !CPLX_ && !PACKED_ && DEEP_ && !KS2_ &&
+                                          BM_ * BN_ >= 256 * 128 && !EDGE16_INLOOP && !E16_;
   static_assert(MT == 32 || MT == 16, "MFMA block edge");
   static constexpr int TM = WM / MT, TN = WN / MT;
   static constexpr int NV = MT * MT / 64;

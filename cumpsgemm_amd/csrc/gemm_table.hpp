@@ -23,6 +23,10 @@ struct KernelEntry {
   // (small real tiles only, else nullptr): for problems of no more tiles than CUs
   void (*launch_kslices)(const GemmArgs &, dim3 grid, hipStream_t stream);
   void (*launch_scaled_kslices)(const GemmArgs &, dim3 grid, hipStream_t stream); // (FP16TCEC tables only)
+  // the persistent variants on 16x16x32 MFMAs (large real FP16TCEC tile only, else
+  // nullptr): for launches that fill the chip
+  void (*launch_persistent_edge16)(const GemmArgs &, dim3 grid, hipStream_t stream);
+  void (*launch_scaled_persistent_edge16)(const GemmArgs &, dim3 grid, hipStream_t stream);
   int bm, bn;      // workgroup tile
   int wm, wn;      // wave tile
   int threads;     // workgroup size
@@ -83,6 +87,10 @@ template <class Cfg> constexpr KernelEntry make_entry(const char *name) {
       e.launch_scaled_kslices = &launch_cfg<GemmCfg<Cfg::P, Cfg::CPLX, Cfg::A_KC, Cfg::B_KC, Cfg::BM, Cfg::BN,
                                                     Cfg::WM, Cfg::WN, Cfg::OCC, false, false, true, false, true>>;
     }
+  }
+  if constexpr (Cfg::HAS_EDGE16_TWIN) {
+    e.launch_persistent_edge16 = &launch_cfg<typename Cfg::persistent_type::edge16_type>;
+    e.launch_scaled_persistent_edge16 = &launch_cfg<typename Cfg::scaled_type::persistent_type::edge16_type>;
   }
   e.bm = Cfg::BM;
   e.bn = Cfg::BN;

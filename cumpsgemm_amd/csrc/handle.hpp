@@ -74,6 +74,7 @@ struct Tuning {
   int force_split = 0;  // CUMPSGEMM_FORCE_KSPLIT
   bool no_persistent = false;    // CUMPSGEMM_NO_PERSISTENT
   bool no_column_split = false;  // CUMPSGEMM_NO_COLUMN_SPLIT
+  bool no_edge16_twin = false;   // CUMPSGEMM_NO_EDGE16_TWIN: never the 16x16x32 instance of the large in-loop tile
   int cut_percent = -1;          // CUMPSGEMM_CUT_PERCENT: C is cut when the model prices the two parts below this
                                  // share of the uncut plan (unset: 93, complex 96, complex bf16x3 110)
   bool no_kslices = false;       // CUMPSGEMM_NO_KSLICE_GROUPS

@@ -82,7 +82,7 @@ const void *cuMpSGEMM_get_workspace_pointer(cuMpSGEMM_handle_t handle);
 
 /* The tuning variables of the GEMM path (CUMPSGEMM_PACKED, _PACKED_WALK,
  * _RASTER_GROUP, _FORCE_TILE_CLASS, _FORCE_KSPLIT, _NO_PERSISTENT,
- * _NO_COLUMN_SPLIT, _CUT_PERCENT, _NO_KSLICE_GROUPS, _NO_FUSED_SCALING,
+ * _NO_COLUMN_SPLIT, _CUT_PERCENT, _NO_KSLICE_GROUPS, _NO_EDGE16_TWIN, _NO_FUSED_SCALING,
  * _PERSISTENT_MAX_STEPS, _MAX_WORKSPACE_BYTES) are read from the environment
  * once per process; this reads them again and publishes the new set as one
  * immutable snapshot.  Safe to call while other threads run GEMMs: a call in

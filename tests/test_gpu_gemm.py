@@ -760,3 +760,52 @@ def test_planner_takes_the_class_the_sweeps_found_best(handle, dev, mode, cplx, 
     c, st, mid = run_gemm(handle, dev, mode, opa, opb, m, n, k, 1.0, a, lda, b, ldb, 0.0, c0, m, cplx,
                           want_module_id=True)
     assert st == 0 and mid in expected, mid
+
+
+# ---- the large real FP16TCEC tile on 16x16x32 MFMAs ------------------------------
+# A tile-walking launch that keeps every CU busy takes a second instance of the 256x128
+# kernel, built on 16x16x32 instead of 32x32x16 MFMAs: the same products, 32 K-values per
+# MFMA instead of 16.  Against the 32x32x16 instance (CUMPSGEMM_NO_EDGE16_TWIN): equal up
+# to the order of summation on random data, bit for bit on small integers, where every
+# partial sum is exact.
+@pytest.mark.parametrize("opa,opb", [(N, N), (T, N), (T, T)])
+@pytest.mark.parametrize("scaled", [False, True])
+def test_large_in_loop_tile_on_16x16x32_mfmas(cg, handle, dev, monkeypatch, opa, opb, scaled):
+    m, n, k, batch = 512, 512, 288, 64           # 8 tiles per matrix: two per CU
+    ra, _ = stored_shape(opa, m, k)
+    rb, _ = stored_shape(opb, k, n)
+    sa, sb, sc = m * k, k * n, m * n
+    rng = np.random.default_rng(5)
+    for exact in (False, True):
+        if exact:
+            a = rng.integers(-8, 9, sa * batch).astype(np.float32)
+            b = rng.integers(-8, 9, sb * batch).astype(np.float32)
+        else:
+            a, b = inputs.uniform(61, sa * batch), inputs.uniform(62, sb * batch)
+        c0 = inputs.uniform(63, sc * batch)
+        da, db = dev.up(a), dev.up(b)
+        outs = []
+        for twin in (True, False):
+            if twin:
+                monkeypatch.delenv("CUMPSGEMM_NO_EDGE16_TWIN", raising=False)
+            else:
+                monkeypatch.setenv("CUMPSGEMM_NO_EDGE16_TWIN", "1")
+            dc = dev.up(c0)
+            if scaled:
+                st, _ = handle.gemm_pipeline(opa, opb, m, n, k, 1.0, da, ra, db, rb, 0.0, dc, m,
+                                             cg.FP16TCEC_SCALING, stridea=sa, strideb=sb, stridec=sc, batch=batch)
+            else:
+                st = handle.gemm_strided_batch(opa, opb, m, n, k, 1.0, da, ra, sa, db, rb, sb, 0.0, dc, m, sc,
+                                               batch, FP16TCEC)
+            assert st == 0
+            outs.append(dev.down(dc))
+        if exact:
+            assert np.array_equal(outs[0], outs[1])
+            A = a[:sa].reshape(-1, ra).T.astype(np.float64)
+            B = b[:sb].reshape(-1, rb).T.astype(np.float64)
+            A = A if opa == N else A.T
+            B = B if opb == N else B.T
+            assert np.array_equal(outs[0][:sc].reshape(n, m).T.astype(np.float64), A @ B)
+        else:
+            assert not np.array_equal(outs[0], outs[1])      # (the two instances did run)
+            assert_same_up_to_summation_order(outs[0], outs[1], k)
