@@ -222,8 +222,8 @@ unsigned resident_groups(const KernelEntry *e) {
 // 4096^2 x 512 221 -> 310, FP16TCEC NT 1024^3 x 8 256 -> 324 TFLOP/s -- and their
 // tables fitted again: 6 / 4 K-steps, 1.1.)
 // split charge = the extra launch that prepares C (about four K-steps of the
-//              largest tile) plus the atomic write-out, which grows with the
-//              number of chunks adding into the same C.
+//              largest tile; real: one) plus the atomic write-out, which grows
+//              with the number of chunks adding into the same C.
 // K-chunks are multiples of the 32-wide step and at least four steps long.
 Plan make_plan(const cuMpSGEMM_handle *h, Prec p, bool cplx, bool a_kc, bool b_kc,
                uint64_t m, uint64_t n, uint64_t k, uint64_t batch, int force_cls, int force_split) {
@@ -258,16 +258,23 @@ Plan make_plan(const cuMpSGEMM_handle *h, Prec p, bool cplx, bool a_kc, bool b_k
                                   : (tile_elems >= 256 * 128 ? (edge16_table ? 6.0 : 5.0)
                                                              : (tile_elems >= 128 * 128 ? (edge16_table ? 4.0 : 3.0) : 4.0)));
     const double small_cplx = (cplx && !cplx_large) ? 0.8 : 1.0;
-    auto eff_of = [&](double groups) {
+    auto eff_of = [&](double groups, bool whole_rounds = false) {
       if (wave_area >= 4096) return edge16_table ? 1.1 : 1.0;
       if (wave_area >= 2048) return 0.83;
       const double waves_per_simd = (double)e->threads * groups / 256.0;
-      return small_cplx * (waves_per_simd >= 2.0 ? 0.55 : (waves_per_simd >= 1.0 ? 0.375 : 0.19));
+      if (cplx) return small_cplx * (waves_per_simd >= 2.0 ? 0.55 : (waves_per_simd >= 1.0 ? 0.375 : 0.19));
+      // (real 64x64 tiles, fitted on 22 shapes from 256^3 to 1536^3 and 896^2 x 2048 x 4 layouts x
+      // {FP16TCEC, bf16x3} x {class 1, 2} x {K split 1, 2, 4, 8}: a lone workgroup on a CU runs as
+      // two wave groups when an operand is K-contiguous)
+      // (whole rounds of a chip full of small workgroups: 0.55 -- with 0.65 there, batches of 320^3
+      // matrices took 64x64 tiles at half the rate of 128x128)
+      return waves_per_simd >= 2.0 ? (whole_rounds ? 0.55 : 0.65)
+                                   : (waves_per_simd >= 1.0 ? ((a_kc || b_kc) ? 0.45 : 0.375) : 0.19);
     };
     // (a tile's operand traffic per flop grows with 1/bm + 1/bn: charged lightly,
     // which also settles ties in favour of the larger tile)
     const double area = (double)e->bm * e->bn * (1.0 + 2.0 / e->bm + 2.0 / e->bn);
-    const double unit = area * res / eff_of((double)res);
+    const double unit = area * res / eff_of((double)res, true);
     const double atomics = (double)m * (double)n * (double)batch * (cplx ? 2.0 : 1.0);
     for (uint64_t sp = 1; sp <= max_split; sp *= 2) {
       if (forced_split != 0 && sp != forced_split) continue;
@@ -282,7 +289,10 @@ Plan make_plan(const cuMpSGEMM_handle *h, Prec p, bool cplx, bool a_kc, bool b_k
       } else {
         cost = steps * (double)((groups + slots - 1) / slots) * unit;
       }
-      if (sp > 1) cost += 4.0 * 256.0 * 128.0 + 0.1 * atomics * (double)sp;
+      // (real: fitted with the efficiencies above; the larger charge kept 896^2 x 2048 unsplit at 32 - 59 us
+      // where two K-chunks take 25 - 28, and 512^3 ... 1024^3 with two M/N-contiguous operands 10 - 50 % slow)
+      if (sp > 1) cost += cplx ? 4.0 * 256.0 * 128.0 + 0.1 * atomics * (double)sp
+                               : 256.0 * 128.0 + 0.05 * atomics * (double)sp;
       if (best < 0.0 || cost < best) {
         best = cost;
         cls = c;
