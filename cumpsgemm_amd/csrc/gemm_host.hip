@@ -283,7 +283,7 @@ Plan make_plan(const cuMpSGEMM_handle *h, Prec p, bool cplx, bool a_kc, bool b_k
       const uint64_t groups = tiles * sp;
       const double steps = (double)((nk + sp - 1) / sp) + fixed_steps;
       double cost;
-      if (groups < slots) {
+      if (groups <= slots) { // (one round at most: the workgroups of a CU start together)
         const double per_cu = (double)((groups + h->num_cus - 1) / h->num_cus);
         cost = steps * per_cu * area / eff_of(per_cu);
       } else {
