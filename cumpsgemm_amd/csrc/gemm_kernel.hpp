@@ -320,14 +320,15 @@ struct GemmCfg {
   static constexpr int MT = PACKED_ ? CUMPSGEMM_MFMA_EDGE_PACKED
                             : (EDGE16_INLOOP || E16_) ? CUMPSGEMM_MFMA_EDGE_PACKED
                                                       : CUMPSGEMM_MFMA_EDGE_INLOOP;
-  // Real FP16TCEC, 256x128, tile-walking: a second instance on 16x16x32 MFMAs for
-  // launches that keep every CU busy.  There the part runs against its power
+  // Real FP16TCEC, 256x128 and 128x128, tile-walking: a second instance on 16x16x32
+  // MFMAs for launches that keep every CU busy.  There the part runs against its power
   // limit and the 16x16x32 form, which needs less energy per flop, measures
   // 3 - 9 % faster (512^3 x 64 279 -> 296, 4096^2 x 512 284 -> 301, 256^3 x 512
-  // 222 -> 243 TFLOP/s); on launches that leave CUs idle the clock is higher and
-  // 32x32x16 wins by 4 - 8 % (2304^2 x 768 242 -> 223).
+  // 222 -> 243 TFLOP/s; 128x128: 1152^2 x 384 x 16 236 -> 244, 768^2 x 256 x 64 229 -> 234);
+  // on launches that leave CUs idle the clock is higher and 32x32x16 wins by 4 - 8 %
+  // (2304^2 x 768 242 -> 223).
   static constexpr bool HAS_EDGE16_TWIN = P_ == Prec::FP16TCEC && !CPLX_ && !PACKED_ && DEEP_ && !KS2_ &&
-                                          BM_ * BN_ >= 256 * 128 && !EDGE16_INLOOP && !E16_;
+                                          BM_ * BN_ >= 128 * 128 && !EDGE16_INLOOP && !E16_;
   static_assert(MT == 32 || MT == 16, "MFMA block edge");
   static constexpr int TM = WM / MT, TN = WN / MT;
   static constexpr int NV = MT * MT / 64;

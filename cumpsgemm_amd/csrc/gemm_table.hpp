@@ -23,8 +23,8 @@ struct KernelEntry {
   // (small real tiles only, else nullptr): for problems of no more tiles than CUs
   void (*launch_kslices)(const GemmArgs &, dim3 grid, hipStream_t stream);
   void (*launch_scaled_kslices)(const GemmArgs &, dim3 grid, hipStream_t stream); // (FP16TCEC tables only)
-  // the persistent variants on 16x16x32 MFMAs (large real FP16TCEC tile only, else
-  // nullptr): for launches that fill the chip
+  // the persistent variants on 16x16x32 MFMAs (256x128 and 128x128 real FP16TCEC
+  // tiles only, else nullptr): for launches that fill the chip
   void (*launch_persistent_edge16)(const GemmArgs &, dim3 grid, hipStream_t stream);
   void (*launch_scaled_persistent_edge16)(const GemmArgs &, dim3 grid, hipStream_t stream);
   int bm, bn;      // workgroup tile

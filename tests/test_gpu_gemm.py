@@ -770,8 +770,9 @@ def test_planner_takes_the_class_the_sweeps_found_best(handle, dev, mode, cplx, 
 # partial sum is exact.
 @pytest.mark.parametrize("opa,opb", [(N, N), (T, N), (T, T)])
 @pytest.mark.parametrize("scaled", [False, True])
-def test_large_in_loop_tile_on_16x16x32_mfmas(cg, handle, dev, monkeypatch, opa, opb, scaled):
-    m, n, k, batch = 512, 512, 288, 64           # 8 tiles per matrix: two per CU
+# (512^2: eight 256x128 tiles per matrix, two per CU; 384^2: nine 128x128 tiles per matrix, nine per CU)
+@pytest.mark.parametrize("m,n,k,batch", [(512, 512, 288, 64), (384, 384, 288, 256)])
+def test_large_in_loop_tile_on_16x16x32_mfmas(cg, handle, dev, monkeypatch, opa, opb, scaled, m, n, k, batch):
     ra, _ = stored_shape(opa, m, k)
     rb, _ = stored_shape(opb, k, n)
     sa, sb, sc = m * k, k * n, m * n
