@@ -327,8 +327,12 @@ struct GemmCfg {
   // 222 -> 243 TFLOP/s; 128x128: 1152^2 x 384 x 16 236 -> 244, 768^2 x 256 x 64 229 -> 234);
   // on launches that leave CUs idle the clock is higher and 32x32x16 wins by 4 - 8 %
   // (2304^2 x 768 242 -> 223).
-  static constexpr bool HAS_EDGE16_TWIN = P_ == Prec::FP16TCEC && !CPLX_ && !PACKED_ && DEEP_ && !KS2_ &&
-                                          BM_ * BN_ >= 128 * 128 && !EDGE16_INLOOP && !E16_;
+  // (the same for the 128x128 kernel of real bf16x3 -- 512^3 x 64 176 -> 182 / 174 -> 188 NN / TN,
+  // 384^3 x 128 158 -> 166 / 157 -> 169 -- and the 256x128 one of FP16TC -- 1024^3 x 8 553 -> 567 / 558 -> 609)
+  static constexpr bool HAS_EDGE16_TWIN =
+      !CPLX_ && !PACKED_ && DEEP_ && !KS2_ && !EDGE16_INLOOP && !E16_ &&
+      ((P_ == Prec::FP16TCEC && BM_ * BN_ >= 128 * 128) || (P_ == Prec::BF16X3 && BM_ * BN_ == 128 * 128) ||
+       (P_ == Prec::FP16TC && BM_ * BN_ >= 256 * 128));
   static_assert(MT == 32 || MT == 16, "MFMA block edge");
   static constexpr int TM = WM / MT, TN = WN / MT;
   static constexpr int NV = MT * MT / 64;

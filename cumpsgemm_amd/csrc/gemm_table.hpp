@@ -23,8 +23,8 @@ struct KernelEntry {
   // (small real tiles only, else nullptr): for problems of no more tiles than CUs
   void (*launch_kslices)(const GemmArgs &, dim3 grid, hipStream_t stream);
   void (*launch_scaled_kslices)(const GemmArgs &, dim3 grid, hipStream_t stream); // (FP16TCEC tables only)
-  // the persistent variants on 16x16x32 MFMAs (256x128 and 128x128 real FP16TCEC
-  // tiles only, else nullptr): for launches that fill the chip
+  // the persistent variants on 16x16x32 MFMAs (real FP16TCEC 256x128 and 128x128,
+  // real bf16x3 128x128, real FP16TC 256x128; else nullptr): for launches that fill the chip
   void (*launch_persistent_edge16)(const GemmArgs &, dim3 grid, hipStream_t stream);
   void (*launch_scaled_persistent_edge16)(const GemmArgs &, dim3 grid, hipStream_t stream);
   int bm, bn;      // workgroup tile
@@ -90,7 +90,8 @@ template <class Cfg> constexpr KernelEntry make_entry(const char *name) {
   }
   if constexpr (Cfg::HAS_EDGE16_TWIN) {
     e.launch_persistent_edge16 = &launch_cfg<typename Cfg::persistent_type::edge16_type>;
-    e.launch_scaled_persistent_edge16 = &launch_cfg<typename Cfg::scaled_type::persistent_type::edge16_type>;
+    if constexpr (Cfg::P == Prec::FP16TCEC)
+      e.launch_scaled_persistent_edge16 = &launch_cfg<typename Cfg::scaled_type::persistent_type::edge16_type>;
   }
   e.bm = Cfg::BM;
   e.bn = Cfg::BN;

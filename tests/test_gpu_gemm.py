@@ -769,10 +769,14 @@ def test_planner_takes_the_class_the_sweeps_found_best(handle, dev, mode, cplx, 
 # to the order of summation on random data, bit for bit on small integers, where every
 # partial sum is exact.
 @pytest.mark.parametrize("opa,opb", [(N, N), (T, N), (T, T)])
-@pytest.mark.parametrize("scaled", [False, True])
-# (512^2: eight 256x128 tiles per matrix, two per CU; 384^2: nine 128x128 tiles per matrix, nine per CU)
-@pytest.mark.parametrize("m,n,k,batch", [(512, 512, 288, 64), (384, 384, 288, 256)])
-def test_large_in_loop_tile_on_16x16x32_mfmas(cg, handle, dev, monkeypatch, opa, opb, scaled, m, n, k, batch):
+# (512^2: eight 256x128 tiles per matrix, two per CU; 384^2: nine 128x128 tiles per matrix, nine per CU;
+# the tables with such a pair of instances: real FP16TCEC both tiles, plain and with fused scaling, real
+# bf16x3 128x128, real FP16TC 256x128)
+@pytest.mark.parametrize("mode,scaled,m,n,k,batch", [
+    (FP16TCEC, False, 512, 512, 288, 64), (FP16TCEC, True, 512, 512, 288, 64),
+    (FP16TCEC, False, 384, 384, 288, 256), (FP16TCEC, True, 384, 384, 288, 256),
+    (TF32TCEC, False, 384, 384, 288, 256), (FP16TC, False, 512, 512, 288, 64)])
+def test_large_in_loop_tile_on_16x16x32_mfmas(cg, handle, dev, monkeypatch, opa, opb, mode, scaled, m, n, k, batch):
     ra, _ = stored_shape(opa, m, k)
     rb, _ = stored_shape(opb, k, n)
     sa, sb, sc = m * k, k * n, m * n
@@ -797,7 +801,7 @@ def test_large_in_loop_tile_on_16x16x32_mfmas(cg, handle, dev, monkeypatch, opa,
                                              cg.FP16TCEC_SCALING, stridea=sa, strideb=sb, stridec=sc, batch=batch)
             else:
                 st = handle.gemm_strided_batch(opa, opb, m, n, k, 1.0, da, ra, sa, db, rb, sb, 0.0, dc, m, sc,
-                                               batch, FP16TCEC)
+                                               batch, mode)
             assert st == 0
             outs.append(dev.down(dc))
         if exact:
@@ -807,6 +811,10 @@ def test_large_in_loop_tile_on_16x16x32_mfmas(cg, handle, dev, monkeypatch, opa,
             A = A if opa == N else A.T
             B = B if opb == N else B.T
             assert np.array_equal(outs[0][:sc].reshape(n, m).T.astype(np.float64), A @ B)
+        elif mode == FP16TC:
+            # one product per block, one accumulator: a 16x16x32 MFMA adds its 32 K-values like two
+            # 32x32x16 MFMAs add their 16 each, and the two instances agree bit for bit
+            assert np.array_equal(outs[0], outs[1])
         else:
             assert not np.array_equal(outs[0], outs[1])      # (the two instances did run)
             assert_same_up_to_summation_order(outs[0], outs[1], k)
